@@ -1,0 +1,135 @@
+/*
+ * mctsnc_hip.h -- C ABI of libmctsnc_hip.so, the MI355X (gfx950) MCTS-NC search engine.
+ *
+ * The reference implements this path as a Python class whose methods launch numba.cuda kernels
+ * (src/mctsnc.py).  It has no C interface of its own for it, so each entry point below names the
+ * reference method it stands in for; a Python (ctypes) class with the reference's constructor and
+ * run() signature sits directly on top of these calls.
+ *
+ * Conventions: every function returns 0 on success and a negative MCTSNC_E_* code on failure;
+ * mctsnc_last_error() returns a human-readable description of the last failure on the calling
+ * thread.  All pointers are host pointers; the engine owns every device allocation.  One engine
+ * may be used from one host thread at a time; several engines may coexist in a process.
+ */
+#ifndef MCTSNC_HIP_H
+#define MCTSNC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MCTSNC_MAX_ACTIONS 512 /* MCTSNC.MAX_STATE_MAX_ACTIONS, src/mctsnc.py:193 */
+
+enum { MCTSNC_GAME_C4 = 0, MCTSNC_GAME_GOMOKU = 1 };
+/* order of MCTSNC.VARIANTS, src/mctsnc.py:180 */
+enum { MCTSNC_OCP_THRIFTY = 0, MCTSNC_OCP_PRODIGAL = 1, MCTSNC_ACP_THRIFTY = 2, MCTSNC_ACP_PRODIGAL = 3 };
+
+enum {
+    MCTSNC_OK = 0,
+    MCTSNC_E_INVALID = -1,     /* bad argument / unsupported configuration */
+    MCTSNC_E_HIP = -2,         /* a HIP runtime call failed */
+    MCTSNC_E_STATE = -3,       /* call order violated (e.g. run before init_device) */
+    MCTSNC_E_ROOT = -4,        /* root position inconsistent with the game's rules */
+    MCTSNC_E_DEVICE_SYNC = -5  /* the on-device step synchronisation timed out */
+};
+
+/* Constructor arguments of MCTSNC (src/mctsnc.py:199-204) after validation, plus the node-pool size that
+ * init_device_side_arrays derives from device_memory (src/mctsnc.py:350-358). */
+typedef struct mctsnc_config {
+    int32_t game;               /* MCTSNC_GAME_* (the reference selects the game by editing source, src/mctsnc_game_mechanics.py:59-87) */
+    int32_t board_m, board_n;   /* state_board_shape */
+    int32_t extra_info_memory;  /* state_extra_info_memory, >= 1 */
+    int32_t max_actions;        /* state_max_actions */
+    int32_t n_trees;
+    int32_t n_playouts;         /* power of two, <= 512 */
+    int32_t variant;            /* MCTSNC_OCP_THRIFTY .. MCTSNC_ACP_PRODIGAL */
+    float ucb_c;
+    uint64_t seed;
+    int64_t max_tree_size;      /* nodes per tree */
+    int32_t device;             /* HIP device ordinal */
+} mctsnc_config;
+
+/* What run() leaves on the instance in the reference: best_* (src/mctsnc.py:1242-1247), the reduced root
+ * table (dev_root_ns, dev_actions_*; :396-404), the memorised root expansion row (:1683-1688), step count,
+ * timings (:448-470) and the tree statistics of _make_performance_info (:472-492). */
+typedef struct mctsnc_result {
+    int64_t steps;
+    int32_t best_action;
+    int32_t best_win_flag;
+    int64_t best_n, best_n_wins;
+    int32_t n_root_entries;                         /* thrifty: number of root actions; prodigal: max_actions */
+    int16_t root_actions_expanded[MCTSNC_MAX_ACTIONS + 2];
+    int64_t root_ns[MCTSNC_MAX_ACTIONS];
+    int64_t actions_ns[MCTSNC_MAX_ACTIONS];
+    int64_t actions_ns_wins[MCTSNC_MAX_ACTIONS];
+    uint8_t actions_win_flags[MCTSNC_MAX_ACTIONS];
+    double time_total, time_loop, time_reduce;      /* host wall clock, seconds */
+    double time_device_loop;                        /* HIP-event time of the search kernels, seconds */
+    int64_t depth_sum;                              /* sum of node depths over all trees */
+    int64_t size_sum;                               /* sum of tree sizes */
+    int32_t max_depth, max_size;
+    uint64_t playout_plies;                         /* playout moves made during this run */
+    uint64_t u1_events;                             /* playout draws that rounded up to 1.0f during this run */
+} mctsnc_result;
+
+typedef struct mctsnc_engine mctsnc_engine;
+
+/* MCTSNC.__init__ (src/mctsnc.py:199-276): validates the configuration; no device work. */
+int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out);
+
+/* MCTSNC.init_device_side_arrays (src/mctsnc.py:318-407): allocates the node pools and seeds the
+ * xoroshiro128+ streams exactly as create_xoroshiro128p_states does (stream i = stream i-1 jumped 2^64). */
+int mctsnc_init_device(mctsnc_engine *e);
+
+/* MCTSNC.run / _run_<variant> (src/mctsnc.py:409-434, :565-1257).  board: int8[m*n] row-major, values in
+ * {-1, 0, +1}; extra: int8[extra_len] or NULL; turn: -1 or +1.  steps_limit / time_limit_s may be INFINITY;
+ * forced_steps_limit < INFINITY overrides both (src/mctsnc.py:1112-1116).  Blocking. RNG streams carry over
+ * from the previous run on the same engine, as in the reference. */
+int mctsnc_run(mctsnc_engine *e, const int8_t *board, const int8_t *extra, int32_t extra_len, int32_t turn,
+               double steps_limit, double time_limit_s, double forced_steps_limit, mctsnc_result *out);
+
+/* Arrays of the last run in the reference's layout and dtypes, one tree at a time (what _json_dump copies
+ * back, src/mctsnc.py:2393-2438).  mctsnc_read_size returns the byte size needed for (array_id, tree). */
+enum {
+    MCTSNC_ARR_TREES = 0,                     /* int32 [size][1 + A]: parent, children (-1 where absent) */
+    MCTSNC_ARR_DEPTHS = 1,                    /* int16 [size] */
+    MCTSNC_ARR_TURNS = 2,                     /* int8  [size] */
+    MCTSNC_ARR_LEAVES = 3,                    /* uint8 [size] */
+    MCTSNC_ARR_TERMINALS = 4,                 /* uint8 [size] */
+    MCTSNC_ARR_OUTCOMES = 5,                  /* int8  [size] (root: 2) */
+    MCTSNC_ARR_NS = 6,                        /* int32 [size] */
+    MCTSNC_ARR_NS_WINS = 7,                   /* int32 [size] */
+    MCTSNC_ARR_BOARDS = 8,                    /* int8  [size][m][n] */
+    MCTSNC_ARR_EXTRA_INFOS = 9,               /* int8  [size][E] */
+    MCTSNC_ARR_SELECTED_PATH = 10,            /* int32 [path_len] of the last step */
+    MCTSNC_ARR_ACTIONS_EXPANDED = 11,         /* int16 [A + 2] of the last step */
+    MCTSNC_ARR_PLAYOUT_OUTCOMES = 12,         /* int32 [2] */
+    MCTSNC_ARR_PLAYOUT_OUTCOMES_CHILDREN = 13,/* int32 [A][2] (ACP variants) */
+    MCTSNC_ARR_NODE_SELECTED = 14,            /* int32 [1] */
+    MCTSNC_ARR_RNG_PLAYOUT = 15,              /* uint64 [n][2], whole array (tree argument ignored) */
+    MCTSNC_ARR_RNG_EXPAND = 16                /* uint64 [n][2], OCP variants, whole array */
+};
+int64_t mctsnc_read_size(mctsnc_engine *e, int32_t array_id, int32_t tree);
+int mctsnc_read(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t dst_bytes);
+
+/* Re-creates the RNG streams from the engine's seed (what constructing a fresh MCTSNC + init_device_side_arrays
+ * does to the generators, src/mctsnc.py:390-394). */
+int mctsnc_reseed(mctsnc_engine *e);
+
+/* Runs n engines of identical configuration concurrently, one search each, in a single device pass
+ * (no counterpart in the reference, which runs one search at a time; results per engine equal those of
+ * mctsnc_run).  boards: n * m*n bytes, extras: n * extra_len bytes or NULL, turns: n entries. */
+int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
+                     const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
+                     mctsnc_result *out);
+
+void mctsnc_destroy(mctsnc_engine *e);
+const char *mctsnc_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,113 @@
+// Device-side building blocks shared by the MCTS-NC search kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mctsnc {
+
+constexpr int kWave = 64;
+
+// ------------------------------------------------------------------------------------------------
+// xoroshiro128+ (rotations 55/14/36) exactly as numba.cuda.random generates it: the reference draws
+// every random number through xoroshiro128p_uniform_float32 (src/mctsnc.py:1435,1882,1971,2061).
+// ------------------------------------------------------------------------------------------------
+__host__ __device__ __forceinline__ uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+
+__host__ __device__ __forceinline__ uint64_t rng_next(uint64_t &s0, uint64_t &s1) {
+    const uint64_t r = s0 + s1;
+    const uint64_t t = s1 ^ s0;
+    s0 = rotl64(s0, 55) ^ t ^ (t << 14);
+    s1 = rotl64(t, 36);
+    return r;
+}
+
+// float32((x >> 11) * 2^-53): the double product is exact, the narrowing rounds to nearest even and
+// can therefore return exactly 1.0f.
+__host__ __device__ __forceinline__ float rng_uniform(uint64_t &s0, uint64_t &s1) {
+    return (float)((double)(rng_next(s0, s1) >> 11) * (1.0 / 9007199254740992.0));
+}
+
+// ------------------------------------------------------------------------------------------------
+// Natural logarithm built only from IEEE-754 basic operations (no fused multiply-add, no library
+// call), so that host and device evaluate bit-identical UCB values.  Classic table-free scheme:
+// x = 2^k (1 + f), s = f / (2 + f), log(1 + f) = f - hfsq + s (hfsq + R(s^2)); error below 1 ulp.
+// Valid for positive normal x (the callers pass visit counts >= 1).
+// ------------------------------------------------------------------------------------------------
+__host__ __device__ inline double det_log(double x) {
+    const double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
+    const double Lg1 = 6.666666666666735130e-01, Lg2 = 3.999999999940941908e-01, Lg3 = 2.857142874366239149e-01,
+                 Lg4 = 2.222219843214978396e-01, Lg5 = 1.818357216161805012e-01, Lg6 = 1.531383769920937332e-01,
+                 Lg7 = 1.479819860511658591e-01;
+    union { double d; uint64_t u; } v;
+    v.d = x;
+    int32_t hx = (int32_t)(v.u >> 32);
+    const uint32_t lx = (uint32_t)v.u;
+    int32_t k = (hx >> 20) - 1023;
+    hx &= 0x000fffff;
+    int32_t i = (hx + 0x95f64) & 0x100000;
+    v.u = ((uint64_t)(uint32_t)(hx | (i ^ 0x3ff00000)) << 32) | lx;  // normalise x or x/2
+    k += (i >> 20);
+    const double f = v.d - 1.0;
+    const double dk = (double)k;
+    if ((0x000fffff & (2 + hx)) < 3) {  // |f| < 2^-20
+        if (f == 0.0) {
+            if (k == 0) return 0.0;
+            return dk * ln2_hi + dk * ln2_lo;
+        }
+        const double R = f * f * (0.5 - 0.33333333333333333 * f);
+        if (k == 0) return f - R;
+        return dk * ln2_hi - ((R - dk * ln2_lo) - f);
+    }
+    const double s = f / (2.0 + f);
+    const double z = s * s;
+    i = hx - 0x6147a;
+    const double w = z * z;
+    const int32_t j = 0x6b851 - hx;
+    const double t1 = w * (Lg2 + w * (Lg4 + w * Lg6));
+    const double t2 = z * (Lg1 + w * (Lg3 + w * (Lg5 + w * Lg7)));
+    i |= j;
+    const double R = t2 + t1;
+    if (i > 0) {
+        const double hfsq = 0.5 * f * f;
+        if (k == 0) return f - (hfsq - s * (hfsq + R));
+        return dk * ln2_hi - ((hfsq - (s * (hfsq + R) + dk * ln2_lo)) - f);
+    }
+    if (k == 0) return f - s * (f - R);
+    return dk * ln2_hi - ((s * (f - R) - dk * ln2_lo) - f);
+}
+
+#ifdef __HIPCC__
+// UCB of one child with the reference's numba typing (src/mctsnc.py:1337): float64 arithmetic on
+// float32(child_n) and a float32 exploration constant, the sum narrowed to float32.
+__device__ __forceinline__ float ucb_value(int32_t wins, int32_t n, double log_parent_n, float c) {
+    const double q = (double)wins / (double)(float)n;
+    const double e = (double)c * __dsqrt_rn(log_parent_n / (double)n);
+    return (float)(q + e);
+}
+
+// Reverses the low three bits.  The reference's strided max-argmax keeps the left slot on ties
+// (src/mctsnc.py:1343-1351), which makes the winner among tied slots the one whose bit-reversed index
+// is smallest; for slots below 8 the order of the 3-bit reversal equals that of any wider reversal.
+__device__ __forceinline__ uint32_t bitrev3(uint32_t a) { return ((a & 1u) << 2) | (a & 2u) | ((a >> 2) & 1u); }
+
+// ---- agent-scope synchronisation between workgroups --------------------------------------------
+__device__ __forceinline__ uint32_t atomic_add_acq_rel(uint32_t *p, uint32_t v) {
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t atomic_load_acquire(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t atomic_load_relaxed(const uint32_t *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void atomic_store_release(uint32_t *p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void atomic_store_relaxed(uint32_t *p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void fence_acquire_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
+__device__ __forceinline__ void fence_release_agent() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
+#endif
+
+}  // namespace mctsnc

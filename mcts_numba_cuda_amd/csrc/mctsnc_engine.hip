@@ -1,0 +1,556 @@
+// libmctsnc_hip.so: host side of the MI355X MCTS-NC engine (C ABI declared in include/mctsnc_hip.h).
+// Host responsibilities mirror MCTSNC.init_device_side_arrays / run / _reduce_over_* / _json_dump of the
+// reference (src/mctsnc.py:318-434, :2222-2462); the search loop itself runs on the device.
+#include "../../include/mctsnc_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "c4_kernels.hpp"
+
+using namespace mctsnc;
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                               \
+    do {                                                                                            \
+        hipError_t err__ = (expr);                                                                  \
+        if (err__ != hipSuccess) return fail(MCTSNC_E_HIP, "%s failed: %s", #expr, hipGetErrorString(err__)); \
+    } while (0)
+
+double now_s() {
+    return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+int next_pow2(int x) { int p = 1; while (p < x) p *= 2; return p; }
+
+// create_xoroshiro128p_states (numba.cuda.random): state 0 from one splitmix64 round, state i = state i-1
+// advanced by 2^64 draws.
+void rng_jump(uint64_t &s0, uint64_t &s1) {
+    static const uint64_t J[2] = {0xbeac0467eba5facbULL, 0xd86b048b86aa9922ULL};
+    uint64_t a = 0, b = 0;
+    for (int i = 0; i < 2; i++)
+        for (int bit = 0; bit < 64; bit++) {
+            if (J[i] & (1ULL << bit)) { a ^= s0; b ^= s1; }
+            rng_next(s0, s1);
+        }
+    s0 = a; s1 = b;
+}
+
+void rng_states(std::vector<uint64_t> &out, int64_t n, uint64_t seed) {
+    out.resize((size_t)n * 2);
+    if (n < 1) return;
+    uint64_t z = seed + 0x9E3779B97F4A7C15ULL;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    z = z ^ (z >> 31);
+    uint64_t s0 = z, s1 = z;
+    out[0] = s0; out[1] = s1;
+    for (int64_t i = 1; i < n; i++) {
+        rng_jump(s0, s1);
+        out[2 * i] = s0; out[2 * i + 1] = s1;
+    }
+}
+
+}  // namespace
+
+struct mctsnc_engine {
+    mctsnc_config cfg;
+    bool inited = false;
+    bool acp = false, thrifty = false;
+    int G = 1, block = 64, tpb_e1 = 64;
+    c4::Node *d_nodes = nullptr;
+    c4::TreeHdr *d_hdrs = nullptr;
+    uint64_t *d_rng_playout = nullptr, *d_rng_expand = nullptr;
+    c4::TreeRef *d_refs = nullptr;
+    c4::TreeDigest *d_digest = nullptr;
+    uint64_t *d_root_bb = nullptr;
+    int32_t *d_root_turns = nullptr, *d_abort = nullptr;
+    int64_t n_rng_playout = 0, n_rng_expand = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool has_run = false;
+};
+
+namespace {
+
+// Bitboards of a position given in the reference's state layout (src/c4.py:24-47: board[i][j], row 0 on top,
+// extra_info[j] = discs in column j).  Rejects what the rules cannot produce.
+int c4_encode_root(const mctsnc_config &c, const int8_t *board, const int8_t *extra, int extra_len, uint64_t bb[2]) {
+    const int m = c.board_m, n = c.board_n, H = m + 1;
+    bb[0] = bb[1] = 0;
+    for (int j = 0; j < n; j++) {
+        int fill = 0;
+        bool gap = false;
+        for (int r = 0; r < m; r++) {
+            const int8_t v = board[(m - 1 - r) * n + j];
+            if (v != -1 && v != 0 && v != 1) return fail(MCTSNC_E_ROOT, "board holds %d at (%d, %d); cells must be -1, 0 or +1", v, m - 1 - r, j);
+            if (v == 0) gap = true;
+            else {
+                if (gap) return fail(MCTSNC_E_ROOT, "column %d has a disc above an empty cell", j);
+                fill = r + 1;
+                bb[v == 1 ? 0 : 1] |= 1ull << (j * H + r);
+            }
+        }
+        if (extra && j < extra_len && extra[j] != fill)
+            return fail(MCTSNC_E_ROOT, "extra_info[%d] = %d but column %d holds %d discs", j, extra[j], j, fill);
+    }
+    if (!extra || extra_len < n) return fail(MCTSNC_E_ROOT, "Connect 4 needs the column fills as extra_info (%d bytes)", n);
+    for (int p = 0; p < 2; p++) {
+        const uint64_t x = bb[p];
+        const int sh[4] = {1, H, H - 1, H + 1};
+        for (int d = 0; d < 4; d++) {
+            const uint64_t t = x & (x >> sh[d]);
+            if (t & (t >> (2 * sh[d]))) return fail(MCTSNC_E_ROOT, "root position already holds four in a row");
+        }
+    }
+    return MCTSNC_OK;
+}
+
+void free_device(mctsnc_engine *e) {
+    if (e->d_nodes) (void)hipFree(e->d_nodes);
+    if (e->d_hdrs) (void)hipFree(e->d_hdrs);
+    if (e->d_rng_playout) (void)hipFree(e->d_rng_playout);
+    if (e->d_rng_expand) (void)hipFree(e->d_rng_expand);
+    if (e->d_refs) (void)hipFree(e->d_refs);
+    if (e->d_digest) (void)hipFree(e->d_digest);
+    if (e->d_root_bb) (void)hipFree(e->d_root_bb);
+    if (e->d_root_turns) (void)hipFree(e->d_root_turns);
+    if (e->d_abort) (void)hipFree(e->d_abort);
+    if (e->ev0) (void)hipEventDestroy(e->ev0);
+    if (e->ev1) (void)hipEventDestroy(e->ev1);
+    if (e->stream) (void)hipStreamDestroy(e->stream);
+    e->d_nodes = nullptr; e->d_hdrs = nullptr; e->d_rng_playout = nullptr; e->d_rng_expand = nullptr; e->d_refs = nullptr;
+    e->d_digest = nullptr; e->d_root_bb = nullptr; e->d_root_turns = nullptr; e->d_abort = nullptr;
+    e->ev0 = e->ev1 = nullptr; e->stream = nullptr;
+    e->inited = false;
+}
+
+int upload_rng(mctsnc_engine *e) {
+    const mctsnc_config &c = e->cfg;
+    std::vector<uint64_t> st;
+    // src/mctsnc.py:390-394: OCP seeds T * tpb_e1 expand generators (only element ti * tpb_e1 is ever used)
+    // and T * P playout generators from the same seed; ACP seeds T * A * P playout generators.
+    rng_states(st, e->n_rng_playout, c.seed);
+    HIP_TRY(hipMemcpy(e->d_rng_playout, st.data(), st.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    if (!e->acp) {
+        std::vector<uint64_t> full, used((size_t)c.n_trees * 2);
+        rng_states(full, (int64_t)c.n_trees * e->tpb_e1, c.seed);
+        for (int t = 0; t < c.n_trees; t++) {
+            used[2 * t] = full[2 * (size_t)t * e->tpb_e1];
+            used[2 * t + 1] = full[2 * (size_t)t * e->tpb_e1 + 1];
+        }
+        HIP_TRY(hipMemcpy(e->d_rng_expand, used.data(), used.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    }
+    return MCTSNC_OK;
+}
+
+struct Budget {
+    double steps_limit, time_limit, forced;
+};
+
+// Final reductions over trees and actions (src/mctsnc.py:2222-2375) from the per-tree digests.
+void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_turn, mctsnc_result *out) {
+    const mctsnc_config &c = e->cfg;
+    const int A = c.max_actions, T = c.n_trees;
+    const int16_t *rae = dg[0].root_ae;
+    for (int i = 0; i < A + 2; i++) out->root_actions_expanded[i] = rae[i];
+    const int nb = e->thrifty ? rae[A + 1] : A;
+    out->n_root_entries = nb;
+    for (int b = 0; b < A; b++) { out->root_ns[b] = 0; out->actions_ns[b] = 0; out->actions_ns_wins[b] = 0; out->actions_win_flags[b] = 0; }
+    for (int b = 0; b < nb; b++) {
+        const int action = e->thrifty ? rae[b] : b;
+        if (action < 0 || action >= A) continue;
+        if (e->thrifty || rae[action] != -1) {
+            for (int t = 0; t < T; t++) {
+                out->root_ns[b] += dg[t].root_ns;
+                if ((dg[t].child_mask >> action) & 1) { out->actions_ns[b] += dg[t].child_ns[action]; out->actions_ns_wins[b] += dg[t].child_wins[action]; }
+            }
+        }
+        out->actions_win_flags[b] = ((dg[0].child_mask >> action) & 1) && dg[0].child_terminal[action] && dg[0].child_outcome[action] == root_turn;
+    }
+    // strided max-argmax over (win_flag, n, n_wins) with the left slot kept on ties (:2318-2330)
+    const int size = next_pow2(A);
+    std::vector<int> idx(size);
+    std::vector<uint8_t> f(size, 0);
+    std::vector<int64_t> ns(size, 0), ws(size, 0);
+    for (int a = 0; a < size; a++) {
+        idx[a] = a;
+        if (a < nb) { f[a] = out->actions_win_flags[a]; ns[a] = out->actions_ns[a]; ws[a] = out->actions_ns_wins[a]; }
+    }
+    for (int stride = size >> 1; stride > 0; stride >>= 1)
+        for (int a = 0; a < stride; a++) {
+            const int b = a + stride;
+            if ((f[a] < f[b]) || (f[a] == f[b] && ns[a] < ns[b]) || (f[a] == f[b] && ns[a] == ns[b] && ws[a] < ws[b])) {
+                idx[a] = idx[b]; f[a] = f[b]; ns[a] = ns[b]; ws[a] = ws[b];
+            }
+        }
+    const int best = idx[0];
+    out->best_win_flag = f[0];
+    out->best_n = ns[0];
+    out->best_n_wins = ws[0];
+    out->best_action = e->thrifty ? ((best < A + 2) ? rae[best] : -1) : best;
+    out->depth_sum = 0; out->size_sum = 0; out->max_depth = -1; out->max_size = 0;
+    out->playout_plies = 0; out->u1_events = 0;
+    for (int t = 0; t < T; t++) {
+        out->depth_sum += dg[t].depth_sum; out->size_sum += dg[t].size;
+        if (dg[t].max_depth > out->max_depth) out->max_depth = dg[t].max_depth;
+        if (dg[t].size > out->max_size) out->max_size = dg[t].size;
+        out->playout_plies += dg[t].plies; out->u1_events += dg[t].u1_events;
+    }
+}
+
+int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
+             const Budget &bud, mctsnc_result *out) {
+    if (n < 1) return fail(MCTSNC_E_INVALID, "no engines given");
+    mctsnc_engine *e0 = engines[0];
+    for (int i = 0; i < n; i++) {
+        mctsnc_engine *e = engines[i];
+        if (!e || !e->inited) return fail(MCTSNC_E_STATE, "init_device has not been called on engine %d", i);
+        const mctsnc_config &a = e->cfg, &b = e0->cfg;
+        if (a.game != b.game || a.board_m != b.board_m || a.board_n != b.board_n || a.n_trees != b.n_trees || a.n_playouts != b.n_playouts ||
+            a.variant != b.variant || a.max_tree_size != b.max_tree_size || a.ucb_c != b.ucb_c || a.device != b.device)
+            return fail(MCTSNC_E_INVALID, "engines of one batch must share their configuration");
+        for (int j = 0; j < i; j++)
+            if (engines[j] == e) return fail(MCTSNC_E_INVALID, "engine %d appears twice in the batch", i);
+    }
+    const mctsnc_config &c = e0->cfg;
+    const int T = c.n_trees, mn = c.board_m * c.board_n;
+    const int n_refs = n * T;
+    const double t_start = now_s();
+    HIP_TRY(hipSetDevice(c.device));
+
+    for (int i = 0; i < n; i++)
+        if (turns[i] != 1 && turns[i] != -1) return fail(MCTSNC_E_ROOT, "root_turn must be -1 or +1");
+    std::vector<uint64_t> bb((size_t)n_refs * 2);
+    std::vector<int32_t> tr((size_t)n_refs);
+    for (int i = 0; i < n; i++) {
+        uint64_t b2[2];
+        int rc = c4_encode_root(c, boards + (size_t)i * mn, extras ? extras + (size_t)i * extra_len : nullptr, extra_len, b2);
+        if (rc) return rc;
+        for (int t = 0; t < T; t++) { bb[2 * ((size_t)i * T + t)] = b2[0]; bb[2 * ((size_t)i * T + t) + 1] = b2[1]; tr[(size_t)i * T + t] = turns[i]; }
+    }
+
+    // the refs / root / digest buffers of a batch are laid out engine after engine
+    c4::TreeRef *d_refs = e0->d_refs;
+    uint64_t *d_bb = e0->d_root_bb;
+    int32_t *d_turns = e0->d_root_turns;
+    c4::TreeDigest *d_digest = e0->d_digest;
+    bool temp = false;
+    if (n > 1) {
+        temp = true;
+        std::vector<c4::TreeRef> refs((size_t)n_refs);
+        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->d_refs, sizeof(c4::TreeRef) * T, hipMemcpyDeviceToHost));
+        HIP_TRY(hipMalloc(&d_refs, sizeof(c4::TreeRef) * n_refs));
+        HIP_TRY(hipMalloc(&d_bb, sizeof(uint64_t) * 2 * n_refs));
+        HIP_TRY(hipMalloc(&d_turns, sizeof(int32_t) * n_refs));
+        HIP_TRY(hipMalloc(&d_digest, sizeof(c4::TreeDigest) * n_refs));
+        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
+    }
+    auto cleanup = [&]() {
+        if (temp) { (void)hipFree(d_refs); (void)hipFree(d_bb); (void)hipFree(d_turns); (void)hipFree(d_digest); }
+    };
+    hipStream_t stream = e0->stream;
+    hipError_t herr;
+#define HIP_TRY_C(expr) do { herr = (expr); if (herr != hipSuccess) { cleanup(); return fail(MCTSNC_E_HIP, "%s failed: %s", #expr, hipGetErrorString(herr)); } } while (0)
+    HIP_TRY_C(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY_C(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY_C(hipMemsetAsync(e0->d_abort, 0, sizeof(int32_t), stream));
+    hipLaunchKernelGGL(c4::reset_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_bb, d_turns);
+    HIP_TRY_C(hipGetLastError());
+    HIP_TRY_C(hipStreamSynchronize(stream));
+
+    // ---- the search loop: chunks of steps on the device, the budget checked between chunks ----
+    c4::SearchArgs args;
+    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
+    args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
+    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    const bool forced = bud.forced < INFINITY;
+    const double step_budget = forced ? bud.forced : bud.steps_limit;
+    const double time_budget = forced ? INFINITY : bud.time_limit;
+    int64_t steps = 0;
+    double dev_time = 0.0;
+    const double t_loop = now_s();
+    for (;;) {
+        const double elapsed = now_s() - t_loop;
+        if ((double)steps >= step_budget || elapsed >= time_budget) break;
+        double chunk = step_budget - (double)steps;
+        if (chunk > 1048576.0) chunk = 1048576.0;
+        if (time_budget < INFINITY) {
+            double by_time = 64.0;
+            if (steps > 0 && elapsed > 0) {
+                const double rate = (double)steps / elapsed;
+                double slice = time_budget - elapsed;
+                const double cap = time_budget / 64.0 > 0.002 ? time_budget / 64.0 : 0.002;
+                if (slice > cap) slice = cap;
+                by_time = rate * slice;
+            }
+            if (by_time < 1.0) by_time = 1.0;
+            if (chunk > by_time) chunk = by_time;
+        }
+        args.nsteps = (int32_t)chunk;
+        if (args.nsteps < 1) break;
+        HIP_TRY_C(hipEventRecord(e0->ev0, stream));
+        if (e0->acp) {
+            void *kargs[] = {&args};
+            HIP_TRY_C(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, 0, stream));
+        } else {
+            hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, 0, stream, args);
+            HIP_TRY_C(hipGetLastError());
+        }
+        HIP_TRY_C(hipEventRecord(e0->ev1, stream));
+        HIP_TRY_C(hipStreamSynchronize(stream));
+        float ms = 0.f;
+        HIP_TRY_C(hipEventElapsedTime(&ms, e0->ev0, e0->ev1));
+        dev_time += ms * 1e-3;
+        steps += args.nsteps;
+        int32_t aborted = 0;
+        HIP_TRY_C(hipMemcpy(&aborted, e0->d_abort, sizeof aborted, hipMemcpyDeviceToHost));
+        if (aborted) { cleanup(); return fail(MCTSNC_E_DEVICE_SYNC, "device-side step synchronisation timed out after %lld steps", (long long)steps); }
+    }
+    const double time_loop = now_s() - t_loop;
+
+    // ---- final reductions ----
+    const double t_red = now_s();
+    hipLaunchKernelGGL(c4::digest_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_digest);
+    HIP_TRY_C(hipGetLastError());
+    std::vector<c4::TreeDigest> dg((size_t)n_refs);
+    HIP_TRY_C(hipMemcpyAsync(dg.data(), d_digest, sizeof(c4::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
+    HIP_TRY_C(hipStreamSynchronize(stream));
+    for (int i = 0; i < n; i++) {
+        mctsnc_result *o = out + i;
+        memset(o, 0, sizeof *o);
+        reduce_result(engines[i], dg.data() + (size_t)i * T, turns[i], o);
+        o->steps = steps;
+        engines[i]->has_run = true;
+    }
+    const double t_end = now_s();
+    for (int i = 0; i < n; i++) {
+        out[i].time_loop = time_loop; out[i].time_reduce = t_end - t_red; out[i].time_total = t_end - t_start; out[i].time_device_loop = dev_time;
+    }
+    cleanup();
+#undef HIP_TRY_C
+    return MCTSNC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *mctsnc_last_error(void) { return g_error.c_str(); }
+
+int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
+    if (!cfg || !out) return fail(MCTSNC_E_INVALID, "null argument");
+    const mctsnc_config &c = *cfg;
+    if (c.game != MCTSNC_GAME_C4) return fail(MCTSNC_E_INVALID, "game %d is not available in this build (Connect 4 only)", c.game);
+    if (c.board_m < 1 || c.board_n < 1 || c.board_n > c4::kMaxCols || (c.board_m + 1) * c.board_n > 64)
+        return fail(MCTSNC_E_INVALID, "Connect 4 board %dx%d unsupported: needs columns <= %d and (rows + 1) * columns <= 64", c.board_m, c.board_n, c4::kMaxCols);
+    if (c.max_actions != c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 has one action per column (%d), got max_actions = %d", c.board_n, c.max_actions);
+    if (c.extra_info_memory < c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 keeps the column fills in extra_info: needs >= %d bytes", c.board_n);
+    if (c.n_trees < 1 || c.n_trees > 512) return fail(MCTSNC_E_INVALID, "n_trees must be in [1, 512]");
+    if (c.n_playouts < 1 || c.n_playouts > 512 || (c.n_playouts & (c.n_playouts - 1))) return fail(MCTSNC_E_INVALID, "n_playouts must be a power of two <= 512");
+    if (c.variant < MCTSNC_OCP_THRIFTY || c.variant > MCTSNC_ACP_PRODIGAL) return fail(MCTSNC_E_INVALID, "unknown variant %d", c.variant);
+    if (!(c.ucb_c >= 0.0f) || std::isinf(c.ucb_c)) return fail(MCTSNC_E_INVALID, "ucb_c must be finite and >= 0");
+    if (c.max_tree_size < 1 || c.max_tree_size > (1 << 24)) return fail(MCTSNC_E_INVALID, "max_tree_size must be in [1, 2^24]");
+    mctsnc_engine *e = new mctsnc_engine();
+    e->cfg = c;
+    e->acp = c.variant >= MCTSNC_ACP_THRIFTY;
+    e->thrifty = (c.variant == MCTSNC_OCP_THRIFTY || c.variant == MCTSNC_ACP_THRIFTY);
+    e->G = e->acp ? c.board_n : 1;
+    e->block = c.n_playouts < 64 ? 64 : c.n_playouts;
+    // tpb table of src/mctsnc.py:360-365 with cuda_tpb_default = 512: fixes which expand generators OCP uses
+    const int tpb_board = next_pow2(c.board_m * c.board_n), tpb_extra = next_pow2(c.extra_info_memory), tpb_actions = next_pow2(c.max_actions);
+    int tpb_r = tpb_board > tpb_extra ? tpb_board : tpb_extra; if (tpb_r > 512) tpb_r = 512;
+    e->tpb_e1 = tpb_r > tpb_actions ? tpb_r : tpb_actions; if (e->tpb_e1 > 512) e->tpb_e1 = 512;
+    *out = e;
+    return MCTSNC_OK;
+}
+
+int mctsnc_init_device(mctsnc_engine *e) {
+    if (!e) return fail(MCTSNC_E_INVALID, "null engine");
+    if (e->inited) free_device(e);
+    const mctsnc_config &c = e->cfg;
+    int ndev = 0;
+    HIP_TRY(hipGetDeviceCount(&ndev));
+    if (c.device < 0 || c.device >= ndev) return fail(MCTSNC_E_INVALID, "device %d not present (%d visible)", c.device, ndev);
+    HIP_TRY(hipSetDevice(c.device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, c.device));
+    if (prop.warpSize != 64) return fail(MCTSNC_E_INVALID, "this library is built for wave64 devices (gfx950)");
+    const int T = c.n_trees;
+    const size_t S = (size_t)c.max_tree_size;
+    HIP_TRY(hipStreamCreate(&e->stream));
+    HIP_TRY(hipEventCreate(&e->ev0));
+    HIP_TRY(hipEventCreate(&e->ev1));
+    HIP_TRY(hipMalloc(&e->d_nodes, sizeof(c4::Node) * S * T));
+    HIP_TRY(hipMalloc(&e->d_hdrs, sizeof(c4::TreeHdr) * T));
+    HIP_TRY(hipMemset(e->d_hdrs, 0, sizeof(c4::TreeHdr) * T));
+    e->n_rng_playout = e->acp ? (int64_t)T * c.max_actions * c.n_playouts : (int64_t)T * c.n_playouts;
+    e->n_rng_expand = e->acp ? 0 : T;
+    HIP_TRY(hipMalloc(&e->d_rng_playout, sizeof(uint64_t) * 2 * e->n_rng_playout));
+    if (!e->acp) HIP_TRY(hipMalloc(&e->d_rng_expand, sizeof(uint64_t) * 2 * T));
+    HIP_TRY(hipMalloc(&e->d_refs, sizeof(c4::TreeRef) * T));
+    HIP_TRY(hipMalloc(&e->d_digest, sizeof(c4::TreeDigest) * T));
+    HIP_TRY(hipMalloc(&e->d_root_bb, sizeof(uint64_t) * 2 * T));
+    HIP_TRY(hipMalloc(&e->d_root_turns, sizeof(int32_t) * T));
+    HIP_TRY(hipMalloc(&e->d_abort, sizeof(int32_t)));
+    std::vector<c4::TreeRef> refs((size_t)T);
+    for (int t = 0; t < T; t++) {
+        refs[t].nodes = e->d_nodes + (size_t)t * S;
+        refs[t].hdr = e->d_hdrs + t;
+        refs[t].rng_playout = e->d_rng_playout + 2 * (size_t)t * (e->acp ? c.max_actions * c.n_playouts : c.n_playouts);
+        refs[t].rng_expand = e->acp ? nullptr : e->d_rng_expand + 2 * (size_t)t;
+    }
+    HIP_TRY(hipMemcpy(e->d_refs, refs.data(), sizeof(c4::TreeRef) * T, hipMemcpyHostToDevice));
+    int rc = upload_rng(e);
+    if (rc) return rc;
+    if (e->acp) {
+        // the step barrier between the workgroups of a tree needs all of them resident at once
+        int coop = 0;
+        HIP_TRY(hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, c.device));
+        if (!coop) return fail(MCTSNC_E_INVALID, "device does not support cooperative launches");
+    }
+    e->inited = true;
+    e->has_run = false;
+    return MCTSNC_OK;
+}
+
+int mctsnc_reseed(mctsnc_engine *e) {
+    if (!e || !e->inited) return fail(MCTSNC_E_STATE, "init_device has not been called");
+    HIP_TRY(hipSetDevice(e->cfg.device));
+    return upload_rng(e);
+}
+
+int mctsnc_run(mctsnc_engine *e, const int8_t *board, const int8_t *extra, int32_t extra_len, int32_t turn, double steps_limit,
+               double time_limit_s, double forced_steps_limit, mctsnc_result *out) {
+    if (!e || !board || !out) return fail(MCTSNC_E_INVALID, "null argument");
+    Budget b{steps_limit, time_limit_s, forced_steps_limit};
+    return run_many(&e, 1, board, extra, extra_len, &turn, b, out);
+}
+
+int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
+                     const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit, mctsnc_result *out) {
+    if (!engines || !boards || !turns || !out) return fail(MCTSNC_E_INVALID, "null argument");
+    Budget b{steps_limit, time_limit_s, forced_steps_limit};
+    return run_many(engines, n, boards, extras, extra_len, turns, b, out);
+}
+
+void mctsnc_destroy(mctsnc_engine *e) {
+    if (!e) return;
+    if (e->inited) { (void)hipSetDevice(e->cfg.device); free_device(e); }
+    delete e;
+}
+
+int64_t mctsnc_read_size(mctsnc_engine *e, int32_t array_id, int32_t tree) {
+    if (!e || !e->inited) return fail(MCTSNC_E_STATE, "init_device has not been called");
+    const mctsnc_config &c = e->cfg;
+    const int A = c.max_actions;
+    if (array_id == MCTSNC_ARR_RNG_PLAYOUT) return e->n_rng_playout * 16;
+    if (array_id == MCTSNC_ARR_RNG_EXPAND) return e->n_rng_expand * 16;
+    if (tree < 0 || tree >= c.n_trees) return fail(MCTSNC_E_INVALID, "tree %d out of range", tree);
+    if (!e->has_run) return fail(MCTSNC_E_STATE, "no search has run yet");
+    if (hipSetDevice(c.device) != hipSuccess) return fail(MCTSNC_E_HIP, "hipSetDevice failed");
+    c4::TreeHdr h;
+    if (hipMemcpy(&h, e->d_hdrs + tree, sizeof h, hipMemcpyDeviceToHost) != hipSuccess) return fail(MCTSNC_E_HIP, "header copy failed");
+    const int64_t sz = h.size;
+    switch (array_id) {
+        case MCTSNC_ARR_TREES: return sz * (1 + A) * 4;
+        case MCTSNC_ARR_DEPTHS: return sz * 2;
+        case MCTSNC_ARR_TURNS: case MCTSNC_ARR_LEAVES: case MCTSNC_ARR_TERMINALS: case MCTSNC_ARR_OUTCOMES: return sz;
+        case MCTSNC_ARR_NS: case MCTSNC_ARR_NS_WINS: return sz * 4;
+        case MCTSNC_ARR_BOARDS: return sz * c.board_m * c.board_n;
+        case MCTSNC_ARR_EXTRA_INFOS: return sz * c.extra_info_memory;
+        case MCTSNC_ARR_SELECTED_PATH: return (int64_t)h.path_len * 4;
+        case MCTSNC_ARR_ACTIONS_EXPANDED: return (A + 2) * 2;
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES: return 8;
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES_CHILDREN: return A * 8;
+        case MCTSNC_ARR_NODE_SELECTED: return 4;
+        default: return fail(MCTSNC_E_INVALID, "unknown array id %d", array_id);
+    }
+}
+
+int mctsnc_read(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t dst_bytes) {
+    const int64_t need = mctsnc_read_size(e, array_id, tree);
+    if (need < 0) return (int)need;
+    if (!dst || dst_bytes < (size_t)need) return fail(MCTSNC_E_INVALID, "destination too small: %zu < %lld", dst_bytes, (long long)need);
+    const mctsnc_config &c = e->cfg;
+    const int A = c.max_actions, m = c.board_m, n = c.board_n, H = m + 1, E = c.extra_info_memory;
+    if (array_id == MCTSNC_ARR_RNG_PLAYOUT) { HIP_TRY(hipMemcpy(dst, e->d_rng_playout, (size_t)need, hipMemcpyDeviceToHost)); return MCTSNC_OK; }
+    if (array_id == MCTSNC_ARR_RNG_EXPAND) { if (need) HIP_TRY(hipMemcpy(dst, e->d_rng_expand, (size_t)need, hipMemcpyDeviceToHost)); return MCTSNC_OK; }
+    c4::TreeHdr h;
+    HIP_TRY(hipMemcpy(&h, e->d_hdrs + tree, sizeof h, hipMemcpyDeviceToHost));
+    switch (array_id) {
+        case MCTSNC_ARR_SELECTED_PATH: memcpy(dst, h.path, (size_t)h.path_len * 4); return MCTSNC_OK;
+        case MCTSNC_ARR_ACTIONS_EXPANDED: memcpy(dst, h.ae, (size_t)(A + 2) * 2); return MCTSNC_OK;
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES: { int32_t v[2] = {h.po_neg, h.po_pos}; memcpy(dst, v, 8); return MCTSNC_OK; }
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES_CHILDREN: memcpy(dst, h.poc, (size_t)A * 8); return MCTSNC_OK;
+        case MCTSNC_ARR_NODE_SELECTED: memcpy(dst, &h.selected, 4); return MCTSNC_OK;
+        default: break;
+    }
+    const int64_t sz = h.size;
+    std::vector<c4::Node> nd((size_t)sz);
+    HIP_TRY(hipMemcpy(nd.data(), e->d_nodes + (size_t)tree * (size_t)c.max_tree_size, sizeof(c4::Node) * (size_t)sz, hipMemcpyDeviceToHost));
+    for (int64_t i = 0; i < sz; i++) {
+        const c4::Node &x = nd[(size_t)i];
+        switch (array_id) {
+            case MCTSNC_ARR_TREES: {
+                int32_t *row = (int32_t *)dst + i * (1 + A);
+                row[0] = x.parent;
+                for (int a = 0; a < A; a++) {
+                    const bool has = !(x.flags & c4::kLeaf) && ((x.child_mask >> a) & 1);
+                    row[1 + a] = has ? x.child_base + __builtin_popcount(x.child_mask & ((1u << a) - 1u)) : -1;
+                }
+                break;
+            }
+            case MCTSNC_ARR_DEPTHS: ((int16_t *)dst)[i] = x.depth; break;
+            case MCTSNC_ARR_TURNS: ((int8_t *)dst)[i] = x.turn; break;
+            case MCTSNC_ARR_LEAVES: ((uint8_t *)dst)[i] = (x.flags & c4::kLeaf) ? 1 : 0; break;
+            case MCTSNC_ARR_TERMINALS: ((uint8_t *)dst)[i] = (x.flags & c4::kTerminal) ? 1 : 0; break;
+            case MCTSNC_ARR_OUTCOMES: ((int8_t *)dst)[i] = x.outcome; break;
+            case MCTSNC_ARR_NS:
+                ((int32_t *)dst)[i] = (i == 0) ? h.root_ns : nd[(size_t)x.parent].child_ns[x.action];
+                break;
+            case MCTSNC_ARR_NS_WINS:
+                ((int32_t *)dst)[i] = (i == 0) ? h.root_wins : nd[(size_t)x.parent].child_wins[x.action];
+                break;
+            case MCTSNC_ARR_BOARDS: {
+                int8_t *b = (int8_t *)dst + i * m * n;
+                for (int r = 0; r < m; r++)
+                    for (int j = 0; j < n; j++) {
+                        const uint64_t bit = 1ull << (j * H + r);
+                        b[(m - 1 - r) * n + j] = (x.bb_pos & bit) ? 1 : ((x.bb_neg & bit) ? -1 : 0);
+                    }
+                break;
+            }
+            case MCTSNC_ARR_EXTRA_INFOS: {
+                int8_t *x2 = (int8_t *)dst + i * E;
+                memset(x2, 0, (size_t)E);
+                for (int j = 0; j < n; j++) x2[j] = (int8_t)__builtin_popcountll((x.bb_pos | x.bb_neg) & (((1ull << m) - 1ull) << (j * H)));
+                break;
+            }
+            default: return fail(MCTSNC_E_INVALID, "unknown array id %d", array_id);
+        }
+    }
+    return MCTSNC_OK;
+}
+
+}  // extern "C"
