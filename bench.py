@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the MCTS-NC search hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): Connect 4 6x7, 64 seeded roots each reached by 10..20 uniform-random legal
+plies (non-terminal), acp_prodigal, n_trees=4, n_playouts=256, ucb_c=2.0, search_steps_limit=5000,
+device_memory=2 GiB, seed 0, random streams restarted for every root.
+
+One bench "step" = one complete search (5000 MCTS steps) of one root through MCTSNC.run(), i.e. the drop-in call the
+reference's game_runner makes.  `value` = playouts per second over the timed searches (root visit totals / wall time
+of run()), with the engine's pools already resident in HBM.  Extra fields: mcts_steps_per_s, the same workload
+batched (all roots concurrently, one device pass) and the per-stage device times.
+
+roofline: the dominant kernel is the persistent search kernel; `achieved` = algorithmic bytes (element sizes of the
+reference's arrays: selection gathers, expansion, RNG state traffic of the playouts, backup) divided by the kernel's
+duration measured with HIP events on the engine's stream.
+cpu_baseline: the CPU oracle (a scalar restatement of the same algorithm, OpenMP over playouts) timed on this host on
+a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+M, N, A = 6, 7, 7
+T, P, STEPS, DEVICE_MEMORY = 4, 256, 5000, 2.0
+N_ROOTS = 64
+HBM_PEAK_GBS = 8000.0
+# HBM bytes per search-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None until measured
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def has_four(board, token):
+    for i in range(M):
+        for j in range(N):
+            for di, dj in ((0, 1), (1, 0), (1, 1), (1, -1)):
+                if all(0 <= i + di * k < M and 0 <= j + dj * k < N and board[i + di * k, j + dj * k] == token for k in range(4)):
+                    return True
+    return False
+
+
+def make_roots(n_roots, seed=0):
+    """Seeded synthetic roots: 10..20 uniform-random legal plies, rejected when the game got decided on the way."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    roots = []
+    while len(roots) < n_roots:
+        plies = int(rng.integers(10, 21))
+        board = np.zeros((M, N), np.int8)
+        fills = np.zeros(N, np.int8)
+        turn, ok = 1, True
+        for _ in range(plies):
+            legal = np.flatnonzero(fills < M)
+            j = int(rng.choice(legal))
+            board[M - 1 - fills[j], j] = turn
+            fills[j] += 1
+            if has_four(board, turn):
+                ok = False
+                break
+            turn = -turn
+        if ok and (fills < M).any():
+            roots.append((board, fills, turn))
+    return roots
+
+
+def device_synchronize():
+    """hipDeviceSynchronize through the HIP runtime the engine library is linked against (MCTSNC.run() itself
+    returns only after its stream has drained)."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    rc = hip.hipDeviceSynchronize()
+    if rc != 0:
+        raise RuntimeError(f"hipDeviceSynchronize failed with {rc}")
+
+
+def algorithmic_bytes(res, tree_steps, acp=True):
+    """Bytes the reference's arrays would move for the work counted on the device (element sizes of
+    src/mctsnc.py:326-348): selection reads per level a leaf flag, the parent's visit count, the child row and the
+    children's (ns, ns_wins); expansion reads the selected state and writes k children; each played-out node reads
+    its state and reads + writes P generator states; backup updates k children and L + 1 path nodes."""
+    mn_e = M * N + A
+    levels, children, expanded, played = res.stat_levels, res.stat_children, res.stat_expanded, res.stat_played
+    select = levels * (1 + 4 + 4 * A) + 8 * children + tree_steps * (1 + 4) + 4 * (levels + tree_steps)
+    expand = tree_steps * (mn_e + 6 + 4 * A + 2 * (A + 2)) + expanded * (mn_e + 18)
+    playout = played * (mn_e + 2 + 32 * P + 8)
+    backup = (expanded if acp else tree_steps) * (4 + 1 + 8 + 16) + (levels + tree_steps) * (4 + 1 + 8 + 8)
+    return dict(select=select, expand=expand, playout=playout, backup=backup, total=select + expand + playout + backup)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=N_ROOTS, help="number of timed searches (roots)")
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-batched", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (trees are independent and would shard over GPUs with one "
+                 "final all-reduce of the root table, but no multi-GPU path is part of it); run with --gpus 1")
+
+    import contextlib
+    import io
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+
+    roots = make_roots(max(N_ROOTS, 1))
+    quiet = io.StringIO()
+
+    def new_engine():
+        e = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=T, n_playouts=P,
+                   variant="acp_prodigal", device_memory=DEVICE_MEMORY, ucb_c=2.0, seed=0, verbose_info=False)
+        e.init_device_side_arrays()
+        return e
+
+    with contextlib.redirect_stdout(quiet):
+        eng = new_engine()
+        for w in range(args.warmup):
+            b, f, t = roots[w % len(roots)]
+            eng.reseed()
+            eng.run(b, f, t)
+
+        device_synchronize()
+        playouts = mcts_steps = 0
+        dev_time = 0.0
+        alg = dict(select=0, expand=0, playout=0, backup=0, total=0)
+        stage = dict(select=0.0, expand=0.0, playout=0.0, backup=0.0)
+        plies = 0
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            b, f, t = roots[k % len(roots)]
+            eng.reseed()
+            eng.run(b, f, t)
+            playouts += eng.performance_info["playouts"]
+            mcts_steps += eng.steps
+            dev_time += eng.time_device_loop
+            plies += eng.performance_info["playout_plies"]
+            ab = algorithmic_bytes(eng._result, eng.steps * T)
+            for key in alg:
+                alg[key] += ab[key]
+            stage["select"] += eng.time_select
+            stage["expand"] += eng.time_expand
+            stage["playout"] += eng.time_playout
+            stage["backup"] += eng.time_backup
+        device_synchronize()
+        elapsed = time.perf_counter() - t0
+
+        batched = None
+        if not args.no_batched:
+            nb = 16
+            engines = [eng] + [new_engine() for _ in range(nb - 1)]
+            bt, bp = 0.0, 0
+            for start in range(0, min(args.steps, len(roots)) - nb + 1, nb):
+                chunk = roots[start:start + nb]
+                for e in engines:
+                    e.reseed()
+                t1 = time.perf_counter()
+                run_batch(engines, [c[0] for c in chunk], [c[1] for c in chunk], [c[2] for c in chunk])
+                bt += time.perf_counter() - t1
+                bp += sum(e.performance_info["playouts"] for e in engines)
+            if bt > 0:
+                n_searches = (min(args.steps, len(roots)) // nb) * nb
+                batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": n_searches / bt,
+                           "mcts_steps_per_s_all_roots": n_searches * STEPS / bt}
+            del engines
+
+    value = playouts / elapsed
+    launches = args.steps  # one search kernel launch per search at a fixed step budget
+    roofline = {"bound": "hbm", "achieved": alg["total"] / dev_time / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": alg["total"] / dev_time / 1e9 / HBM_PEAK_GBS,
+                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                "kernel": "mctsnc::c4::search_kernel<true>", "algorithmic_bytes_per_launch": alg["total"] / launches,
+                "avg_launch_ms": dev_time / launches * 1e3,
+                "stage_bytes_per_launch": {k: v / launches for k, v in alg.items() if k != "total"},
+                "playout_plies_per_s": plies / dev_time,
+                "note": "latency-bound pointer chasing plus integer playouts on 28 workgroups: a few KB of tree data per step; see DESIGN.md"}
+
+    cpu_baseline = None
+    if not args.no_cpu_baseline:
+        from oracle.oracle import Oracle
+        cores = min(16, os.cpu_count() or 1)
+        n_sample_roots, sample_steps = 8, 400
+        cpu_playouts, dt = 0, 0.0
+        for b, f, t in roots[:n_sample_roots]:
+            o = Oracle("c4", (M, N), A, A, T, P, "acp_prodigal", ucb_c=2.0, seed=0, device_memory=DEVICE_MEMORY, threads=cores)
+            t1 = time.perf_counter()
+            o.run(b, f, t, sample_steps)
+            dt += time.perf_counter() - t1
+            cpu_playouts += int(o.result("root_ns").max())
+        cpu_baseline = {"value": cpu_playouts / dt, "unit": "playouts/s", "cores": cores, "kind": "port",
+                        "mcts_steps_per_s": n_sample_roots * sample_steps / dt,
+                        "sample": f"first {n_sample_roots} roots of the workload, {sample_steps} MCTS steps each ({cpu_playouts} playouts), "
+                                  "CPU oracle (scalar restatement of the reference's kernels) with OpenMP over playouts"}
+
+    out = {"metric": "playouts/s + steps/s, C4 6x7 ACP-prodigal 4x256 on 1 MI355X; % of roofline",
+           "value": value, "unit": "playouts/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "int64 bitboards + int32 counters (UCB in f64 rounded to f32)", "data": "synthetic",
+           "config": {"workload": "C4 6x7, 64 seeded roots (10-20 random plies), acp_prodigal n_trees=4 n_playouts=256 ucb_c=2.0 "
+                                  "search_steps_limit=5000 device_memory=2GiB seed=0; one MCTSNC.run() per root, sequential",
+                      "bench_step": "one search of 5000 MCTS steps"},
+           "mcts_steps_per_s": mcts_steps / elapsed,
+           "device_loop_share": dev_time / elapsed,
+           "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
+           "batched": batched,
+           "roofline": roofline, "cpu_baseline": cpu_baseline}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

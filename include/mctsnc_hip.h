@@ -73,6 +73,12 @@ typedef struct mctsnc_result {
     int32_t max_depth, max_size;
     uint64_t playout_plies;                         /* playout moves made during this run */
     uint64_t u1_events;                             /* playout draws that rounded up to 1.0f during this run */
+    /* work counters summed over trees: tree levels walked by selection, children examined on those walks,
+     * nodes created, nodes played out with real (non-terminal) playouts */
+    uint64_t stat_levels, stat_children, stat_expanded, stat_played;
+    /* per-stage device time of tree 0 in seconds (time_select/expand/playout/backup of the reference,
+     * src/mctsnc.py:1121-1213); zero when stage timing is off */
+    double time_select, time_expand, time_playout, time_backup;
 } mctsnc_result;
 
 typedef struct mctsnc_engine mctsnc_engine;
@@ -125,6 +131,9 @@ int mctsnc_reseed(mctsnc_engine *e);
 int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
                      const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
                      mctsnc_result *out);
+
+/* Switches the per-stage device timers on (default) or off. */
+int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on);
 
 void mctsnc_destroy(mctsnc_engine *e);
 const char *mctsnc_last_error(void);

@@ -28,7 +28,9 @@ class Result(ctypes.Structure):
                 ("time_total", ctypes.c_double), ("time_loop", ctypes.c_double), ("time_reduce", ctypes.c_double),
                 ("time_device_loop", ctypes.c_double), ("depth_sum", ctypes.c_int64), ("size_sum", ctypes.c_int64),
                 ("max_depth", ctypes.c_int32), ("max_size", ctypes.c_int32), ("playout_plies", ctypes.c_uint64),
-                ("u1_events", ctypes.c_uint64)]
+                ("u1_events", ctypes.c_uint64), ("stat_levels", ctypes.c_uint64), ("stat_children", ctypes.c_uint64),
+                ("stat_expanded", ctypes.c_uint64), ("stat_played", ctypes.c_uint64), ("time_select", ctypes.c_double),
+                ("time_expand", ctypes.c_double), ("time_playout", ctypes.c_double), ("time_backup", ctypes.c_double)]
 
 
 ARRAYS = {  # name -> (id, dtype, trailing shape builder)
@@ -74,6 +76,8 @@ def lib():
         L.mctsnc_read.argtypes = [vp, ctypes.c_int32, ctypes.c_int32, vp, ctypes.c_size_t]
         L.mctsnc_reseed.restype = ctypes.c_int
         L.mctsnc_reseed.argtypes = [vp]
+        L.mctsnc_set_stage_timing.restype = ctypes.c_int
+        L.mctsnc_set_stage_timing.argtypes = [vp, ctypes.c_int32]
         L.mctsnc_destroy.restype = None
         L.mctsnc_destroy.argtypes = [vp]
         L.mctsnc_last_error.restype = ctypes.c_char_p

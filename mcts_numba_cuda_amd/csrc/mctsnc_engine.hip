@@ -89,6 +89,8 @@ struct mctsnc_engine {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool has_run = false;
+    bool stage_timing = true;
+    std::vector<uint64_t> rng_init_playout, rng_init_expand;  // the streams as seeded, kept for reseed()
 };
 
 namespace {
@@ -147,20 +149,23 @@ void free_device(mctsnc_engine *e) {
 
 int upload_rng(mctsnc_engine *e) {
     const mctsnc_config &c = e->cfg;
-    std::vector<uint64_t> st;
     // src/mctsnc.py:390-394: OCP seeds T * tpb_e1 expand generators (only element ti * tpb_e1 is ever used)
     // and T * P playout generators from the same seed; ACP seeds T * A * P playout generators.
-    rng_states(st, e->n_rng_playout, c.seed);
-    HIP_TRY(hipMemcpy(e->d_rng_playout, st.data(), st.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
-    if (!e->acp) {
-        std::vector<uint64_t> full, used((size_t)c.n_trees * 2);
-        rng_states(full, (int64_t)c.n_trees * e->tpb_e1, c.seed);
-        for (int t = 0; t < c.n_trees; t++) {
-            used[2 * t] = full[2 * (size_t)t * e->tpb_e1];
-            used[2 * t + 1] = full[2 * (size_t)t * e->tpb_e1 + 1];
+    if (e->rng_init_playout.empty()) {
+        rng_states(e->rng_init_playout, e->n_rng_playout, c.seed);
+        if (!e->acp) {
+            std::vector<uint64_t> full;
+            rng_states(full, (int64_t)c.n_trees * e->tpb_e1, c.seed);
+            e->rng_init_expand.resize((size_t)c.n_trees * 2);
+            for (int t = 0; t < c.n_trees; t++) {
+                e->rng_init_expand[2 * t] = full[2 * (size_t)t * e->tpb_e1];
+                e->rng_init_expand[2 * t + 1] = full[2 * (size_t)t * e->tpb_e1 + 1];
+            }
         }
-        HIP_TRY(hipMemcpy(e->d_rng_expand, used.data(), used.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
     }
+    HIP_TRY(hipMemcpy(e->d_rng_playout, e->rng_init_playout.data(), e->rng_init_playout.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
+    if (!e->acp)
+        HIP_TRY(hipMemcpy(e->d_rng_expand, e->rng_init_expand.data(), e->rng_init_expand.size() * sizeof(uint64_t), hipMemcpyHostToDevice));
     return MCTSNC_OK;
 }
 
@@ -211,7 +216,13 @@ void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_tu
     out->best_action = e->thrifty ? ((best < A + 2) ? rae[best] : -1) : best;
     out->depth_sum = 0; out->size_sum = 0; out->max_depth = -1; out->max_size = 0;
     out->playout_plies = 0; out->u1_events = 0;
+    out->stat_levels = out->stat_children = out->stat_expanded = out->stat_played = 0;
+    const double tick = 1e-8;  // wall_clock64 counts at 100 MHz
+    out->time_select = dg[0].t_select * tick; out->time_expand = dg[0].t_expand * tick;
+    out->time_playout = dg[0].t_playout * tick; out->time_backup = dg[0].t_backup * tick;
     for (int t = 0; t < T; t++) {
+        out->stat_levels += dg[t].stat_levels; out->stat_children += dg[t].stat_children;
+        out->stat_expanded += dg[t].stat_expanded; out->stat_played += dg[t].stat_played;
         out->depth_sum += dg[t].depth_sum; out->size_sum += dg[t].size;
         if (dg[t].max_depth > out->max_depth) out->max_depth = dg[t].max_depth;
         if (dg[t].size > out->max_size) out->max_size = dg[t].size;
@@ -283,6 +294,7 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     c4::SearchArgs args;
     args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
+    args.stage_timing = e0->stage_timing ? 1 : 0;
     const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
     const bool forced = bud.forced < INFINITY;
     const double step_budget = forced ? bud.forced : bud.steps_limit;
@@ -452,6 +464,12 @@ int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, c
     if (!engines || !boards || !turns || !out) return fail(MCTSNC_E_INVALID, "null argument");
     Budget b{steps_limit, time_limit_s, forced_steps_limit};
     return run_many(engines, n, boards, extras, extra_len, turns, b, out);
+}
+
+int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on) {
+    if (!e) return fail(MCTSNC_E_INVALID, "null engine");
+    e->stage_timing = on != 0;
+    return MCTSNC_OK;
 }
 
 void mctsnc_destroy(mctsnc_engine *e) {

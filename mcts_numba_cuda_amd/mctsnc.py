@@ -235,6 +235,8 @@ class MCTSNC:
         self.time_device_loop = res.time_device_loop
         self.time_reduce_over_trees = res.time_reduce
         self.time_reduce_over_actions = 0.0  # both reductions are one pass here
+        self.time_select, self.time_expand = res.time_select, res.time_expand
+        self.time_playout, self.time_backup = res.time_playout, res.time_backup
         self._root_actions_expanded = np.array(res.root_actions_expanded[:A + 2], dtype=np.int16)
         self._root_ns = np.array(res.root_ns[:A], dtype=np.int64)
         self._actions_ns = np.array(res.actions_ns[:A], dtype=np.int64)
@@ -290,8 +292,8 @@ class MCTSNC:
 
     def _make_performance_info(self):
         """Performance dictionary with the reference's keys (src/mctsnc.py:448-494).  The four stages run fused in one
-        kernel, so their per-step means are reported as the device loop time split by measured stage shares when the
-        library provides them, otherwise as the mean step time under ``mean_loop`` only."""
+        kernel; their per-step means come from device clock readings taken between the stages by one workgroup of
+        tree 0 (the backup figure includes the wait for the tree's other workgroups)."""
         res = self._result
         performance_info = {}
         performance_info["steps"] = int(self.steps)

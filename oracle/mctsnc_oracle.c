@@ -28,6 +28,10 @@
  *   - tree-full (-3) step, OCP: the path is backed up, the out-of-bounds child
  *     update of _backup_ocp (src/mctsnc.py:2106-2114 with rand_child == -3) is
  *     skipped; _expand_2_thrifty (:1697-1754) is skipped instead of writing node -1.
+ *   - node pool running out in the middle of an expansion: the reference gives every legal action that
+ *     no longer fits the index of the last child that did (src/mctsnc.py:1427-1429 store the running
+ *     shift for every action), after which several blocks write that one node concurrently; here such
+ *     actions get no child (-1) and only the children that fit are created and played out.
  *   - OCP random child when the uniform draw rounds to 1.0f: the ordinal is
  *     clamped to count-1 (the reference indexes one past its list, :1435,:1511).
  *   - root action without a child node in the final reduction (:2236,:2278 read
@@ -451,8 +455,8 @@ static void k_expand_1(oracle_t *o, int ti) {
             if (legal[i] && (int64_t)size_so_far + child_shift + 1 < o->max_tree_size) {
                 child_shift++;
                 map[child_shift] = (int16_t)i;
-            }
-            shifts[i] = child_shift;
+                shifts[i] = child_shift;
+            }   /* a legal action that no longer fits gets no child: see file header */
         }
         if (child_shift >= 0) {
             ae[A + 1] = (int16_t)(child_shift + 1);
@@ -482,7 +486,7 @@ static void k_expand_1(oracle_t *o, int ti) {
         } else if (prodigal) ae[a] = -1;
         row[1 + a] = child_index;
     }
-    t->size += shifts[A - 1] + 1;
+    t->size += child_shift + 1;
     if (!ocp && (terminal || for_playout == -3)) ae[0] = 0;
 }
 
@@ -492,6 +496,7 @@ static void k_expand_2_block(oracle_t *o, int ti, int action) {
     const int A = o->A, mn = o->m * o->n, E = o->E;
     const int32_t selected = t->selected;
     const int32_t child = t->trees[(int64_t)selected * (1 + A) + 1 + action];
+    if (child < 0) return; /* stale row entry of an action that got no child in this step */
     int8_t *cb = t->boards + (int64_t)child * mn, *ce = t->extras + (int64_t)child * E;
     memcpy(cb, t->boards + (int64_t)selected * mn, (size_t)mn);
     memcpy(ce, t->extras + (int64_t)selected * E, (size_t)E);

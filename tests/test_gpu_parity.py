@@ -82,3 +82,63 @@ def test_against_oracle_full_state(variant, T, P):
     for run, plies in enumerate([8, 24]):
         board, fills, turn = random_c4_root(rng, plies)
         compare_with_oracle(e, o, board, fills, turn, steps=150 if P >= 256 else 300)
+
+
+def test_run_batch_equals_single_runs():
+    """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
+    from mcts_numba_cuda_amd import run_batch
+    rng = np.random.default_rng(5)
+    params = dict(n_trees=4, n_playouts=128, variant="acp_prodigal", device_memory=0.1, ucb_c=2.0, seed=11)
+    roots = [random_c4_root(rng, p) for p in (4, 9, 15, 22, 12)]
+    batch = [make_engine(params) for _ in roots]
+    single = [make_engine(params) for _ in roots]
+    for rounds in range(2):  # second round: random streams carried over on both sides
+        run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=400)
+        for e, r in zip(single, roots):
+            e.run(r[0], r[1], r[2], forced_search_steps_limit=400)
+        for eb, es in zip(batch, single):
+            assert eb.actions_info == es.actions_info
+            assert eb.performance_info["trees"] == es.performance_info["trees"]
+            for ti in range(4):
+                for name in ("trees", "ns", "ns_wins", "depths"):
+                    np.testing.assert_array_equal(eb.read_array(name, ti), es.read_array(name, ti))
+            np.testing.assert_array_equal(eb.read_array("rng_playout"), es.read_array("rng_playout"))
+
+
+def test_time_limited_run_and_chunking():
+    """A time budget is honoured within a few percent and splitting a search over several kernel launches changes
+    nothing: the same number of steps in one launch gives the identical tree."""
+    params = dict(n_trees=4, n_playouts=64, variant="acp_thrifty", device_memory=0.25, ucb_c=2.0, seed=2)
+    from mcts_numba_cuda_amd import MCTSNC
+    e = MCTSNC((6, 7), 7, 7, search_time_limit=0.25, search_steps_limit=np.inf, n_trees=4, n_playouts=64, variant="acp_thrifty",
+               device_memory=0.25, ucb_c=2.0, seed=2, verbose_info=False)
+    e.init_device_side_arrays()
+    board, fills, turn = random_c4_root(np.random.default_rng(3), 7)
+    e.run(board, fills, turn)
+    assert 0.25 <= e.time_loop < 0.30
+    steps = e.steps
+    assert steps > 1000
+    ref = make_engine(params)
+    ref.run(board, fills, turn, forced_search_steps_limit=steps)
+    assert e.actions_info == ref.actions_info
+    for ti in range(4):
+        np.testing.assert_array_equal(e.read_array("ns", ti), ref.read_array("ns", ti))
+        np.testing.assert_array_equal(e.read_array("trees", ti), ref.read_array("trees", ti))
+
+
+def test_tree_full_and_terminal_paths_match_oracle():
+    """A tiny node pool forces the memory-exhausted path; late-game roots force terminal selections."""
+    from oracle.oracle import Oracle
+    rng = np.random.default_rng(9)
+    for variant in ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"]:
+        from mcts_numba_cuda_amd import MCTSNC
+        e = MCTSNC((6, 7), 7, 7, search_time_limit=np.inf, search_steps_limit=np.inf, n_trees=2, n_playouts=64, variant=variant,
+                   device_memory=2.0, ucb_c=2.0, seed=4, verbose_info=False)
+        e.device_memory = float(2 * 95 * 50 + 2 * 8300)  # room for about 50 nodes per tree
+        e.init_device_side_arrays()
+        assert 10 < e.max_tree_size < 120
+        o = Oracle("c4", (6, 7), 7, 7, 2, 64, variant, ucb_c=2.0, seed=4, max_tree_size_override=e.max_tree_size, threads=4)
+        for plies in (5, 30):
+            board, fills, turn = random_c4_root(rng, plies)
+            compare_with_oracle(e, o, board, fills, turn, steps=200)
+        assert max(e.read_array("depths", t).shape[0] for t in range(2)) <= e.max_tree_size
