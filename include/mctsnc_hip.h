@@ -79,6 +79,7 @@ typedef struct mctsnc_result {
     /* per-stage device time of tree 0 in seconds (time_select/expand/playout/backup of the reference,
      * src/mctsnc.py:1121-1213); zero when stage timing is off */
     double time_select, time_expand, time_playout, time_backup;
+    double time_exchange;   /* part of time_backup spent exchanging playout results between workgroups (incl. waiting) */
 } mctsnc_result;
 
 typedef struct mctsnc_engine mctsnc_engine;

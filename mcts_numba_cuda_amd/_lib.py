@@ -30,7 +30,8 @@ class Result(ctypes.Structure):
                 ("max_depth", ctypes.c_int32), ("max_size", ctypes.c_int32), ("playout_plies", ctypes.c_uint64),
                 ("u1_events", ctypes.c_uint64), ("stat_levels", ctypes.c_uint64), ("stat_children", ctypes.c_uint64),
                 ("stat_expanded", ctypes.c_uint64), ("stat_played", ctypes.c_uint64), ("time_select", ctypes.c_double),
-                ("time_expand", ctypes.c_double), ("time_playout", ctypes.c_double), ("time_backup", ctypes.c_double)]
+                ("time_expand", ctypes.c_double), ("time_playout", ctypes.c_double), ("time_backup", ctypes.c_double),
+                ("time_exchange", ctypes.c_double)]
 
 
 ARRAYS = {  # name -> (id, dtype, trailing shape builder)

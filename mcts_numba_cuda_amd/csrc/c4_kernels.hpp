@@ -72,7 +72,7 @@ struct __attribute__((aligned(128))) TreeHdr {
     // looked at during those walks, stat_expanded = nodes created, stat_played = nodes played out with real playouts;
     // t_* = device clock ticks (100 MHz) spent per stage by workgroup 0 of the tree when stage timing is on
     unsigned long long plies, u1_events, stat_levels, stat_children, stat_expanded, stat_played;
-    unsigned long long t_select, t_expand, t_playout, t_backup; int32_t pad5[12];
+    unsigned long long t_select, t_expand, t_playout, t_backup, t_exchange; int32_t pad5[10];
     // lines 6,7: path of the last step
     int32_t path[kMaxPath];
 };
@@ -200,28 +200,114 @@ __device__ inline int exact_playout(ExactScratch &s, const Geometry &g, uint64_t
 }
 
 // ---- one fast playout on bitboards (src/mctsnc.py:2057-2069 with the Connect 4 mechanics) ----------
-// cur: stones of the side to move, opp: the other side's.  Returns -1 / 0 / +1, or 2 when a draw of the
-// uniform rounded up to 1.0f (the caller then replays the playout with exact_playout).
-__device__ __forceinline__ int fast_playout(const Geometry &g, const uint8_t *nth_table, uint64_t cur, uint64_t opp, int turn,
-                                            uint64_t &s0, uint64_t &s1, uint32_t &plies) {
-    uint64_t all = cur | opp;
-    uint32_t legal = g.legal_cols(all);
-    for (;;) {
-        const int count = __popc(legal);
-        if (count == 0) return 0;
-        const float u = rng_uniform(s0, s1);
-        const int ord = (int)(u * (float)count);  // single-precision product, as the reference's float32 * int16
-        if (ord >= count) return 2;
-        const int c = nth_table[legal * 8 + ord];
-        const uint64_t newbit = (all + g.bottom(c)) & g.col_mask(c);
-        cur |= newbit;
-        all |= newbit;
-        plies++;
-        if (g.has_four(cur)) return turn;
-        if (newbit & g.top(c)) legal &= ~(1u << c);
-        const uint64_t t = cur; cur = opp; opp = t;
-        turn = -turn;
+// Everything per lane lives in 32-bit registers: each bitboard as (lo, hi), the column fills as 4-bit fields, the
+// ascending list of legal columns as 4-bit fields with its count (the reference rebuilds that list every ply,
+// src/mctsnc_game_mechanics.py:102-109; removing a column when it fills keeps the same order).
+
+struct BB { uint32_t lo, hi; };
+
+__device__ __forceinline__ BB bb_shr(BB x, int s) {  // 0 < s < 32
+    BB r; r.lo = __builtin_amdgcn_alignbit(x.hi, x.lo, s); r.hi = x.hi >> s; return r;
+}
+__device__ __forceinline__ BB bb_and(BB a, BB b) { BB r; r.lo = a.lo & b.lo; r.hi = a.hi & b.hi; return r; }
+
+// four in a row anywhere in p (equals "through the last stone" while no earlier line exists)
+__device__ __forceinline__ bool bb_has_four(BB p, int H) {
+    BB t = bb_and(p, bb_shr(p, 1));
+    BB r = bb_and(t, bb_shr(t, 2));
+    t = bb_and(p, bb_shr(p, H));
+    BB q = bb_and(t, bb_shr(t, 2 * H));
+    r.lo |= q.lo; r.hi |= q.hi;
+    t = bb_and(p, bb_shr(p, H - 1));
+    q = bb_and(t, bb_shr(t, 2 * (H - 1)));
+    r.lo |= q.lo; r.hi |= q.hi;
+    t = bb_and(p, bb_shr(p, H + 1));
+    q = bb_and(t, bb_shr(t, 2 * (H + 1)));
+    return (r.lo | q.lo | r.hi | q.hi) != 0;
+}
+
+// xoroshiro128+ step on 32-bit halves (the 64-bit shifts of the generic form are slow vector instructions)
+struct Rng32 { uint32_t s0l, s0h, s1l, s1h; };
+
+__device__ __forceinline__ void rng_next32(Rng32 &r, uint32_t &out_lo, uint32_t &out_hi) {
+    const uint64_t sum = (((uint64_t)r.s0h << 32) | r.s0l) + (((uint64_t)r.s1h << 32) | r.s1l);
+    out_lo = (uint32_t)sum; out_hi = (uint32_t)(sum >> 32);
+    const uint32_t tl = r.s1l ^ r.s0l, th = r.s1h ^ r.s0h;
+    // rotl(s0, 55) = rotr(s0, 9); t << 14; rotl(t, 36) = halves swapped, then rotl 4
+    const uint32_t r0l = __builtin_amdgcn_alignbit(r.s0h, r.s0l, 9), r0h = __builtin_amdgcn_alignbit(r.s0l, r.s0h, 9);
+    const uint32_t shl = tl << 14, shh = __builtin_amdgcn_alignbit(th, tl, 18);
+    r.s0l = r0l ^ tl ^ shl; r.s0h = r0h ^ th ^ shh;
+    r.s1l = __builtin_amdgcn_alignbit(th, tl, 28); r.s1h = __builtin_amdgcn_alignbit(tl, th, 28);
+}
+
+// float32((x >> 11) * 2^-53) without double arithmetic.  Write x >> 11 = hi * 2^21 + f with f < 2^21; the value is
+// (hi + f * 2^-21) * 2^-32.  If hi >= 2^25 the float32 rounding drops at least two bits of hi, so folding "f != 0"
+// into bit 0 of hi (a sticky bit) leaves round-to-nearest-even unchanged.  Smaller values are first shifted left by
+// 7 or 14 bits (exact rescaling); below 2^43 (probability 2^-21) the double path is taken.
+__device__ __forceinline__ float uniform_from_bits(uint32_t lo, uint32_t hi) {
+    lo &= 0xfffff800u;  // the 11 bits that x >> 11 discards
+    float scale = 2.3283064365386963e-10f;  // 2^-32
+    if (__builtin_expect(hi < (1u << 25), 0)) {
+        if (hi >= (1u << 11)) {  // shift left by 14: hi' >= 2^25
+            hi = (hi << 14) | (lo >> 18); lo <<= 14; scale = 1.4210854715202004e-14f;  // 2^-46
+        } else {
+            return (float)((double)(((uint64_t)hi << 32 | lo) >> 11) * (1.0 / 9007199254740992.0));
+        }
     }
+    const uint32_t t = hi | (lo != 0 ? 1u : 0u);
+    return (float)t * scale;
+}
+
+// cur: stones of the side to move, opp: the other side's.  Returns -1 / 0 / +1, or 2 when a draw of the
+// uniform rounded up to 1.0f (the caller then replays the playout with exact_playout).  The ply body is free of
+// branches: lanes leave through the loop condition only.
+__device__ __forceinline__ int fast_playout(const Geometry &g, uint64_t cur, uint64_t opp, int turn,
+                                            uint64_t &s0, uint64_t &s1, uint32_t &plies) {
+    BB a, b;
+    a.lo = (uint32_t)cur; a.hi = (uint32_t)(cur >> 32);
+    b.lo = (uint32_t)opp; b.hi = (uint32_t)(opp >> 32);
+    const uint64_t all = cur | opp;
+    uint32_t fills = 0, list = 0;
+    int count = 0;
+    for (int c = 0; c < g.n; c++) {
+        const int h = __popcll(all & g.col_mask(c));
+        fills |= (uint32_t)h << (4 * c);
+        if (h < g.m) { list |= (uint32_t)c << (4 * count); count++; }
+    }
+    if (count == 0) return 0;
+    const int m = g.m, H = g.H;
+    Rng32 r;
+    r.s0l = (uint32_t)s0; r.s0h = (uint32_t)(s0 >> 32); r.s1l = (uint32_t)s1; r.s1h = (uint32_t)(s1 >> 32);
+    int status;  // 0 = game goes on, 1 = mover won, 2 = board full, 3 = ordinal == count
+    uint32_t n = 0;
+    do {
+        uint32_t xl, xh;
+        rng_next32(r, xl, xh);
+        const float u = uniform_from_bits(xl, xh);
+        const int ord = (int)(u * (float)count);  // single-precision product, as the reference's float32 * int16
+        const int sh = ord * 4;
+        const int c = (int)((list >> sh) & 7u);
+        const int c4 = c * 4;
+        const int h = (int)((fills >> c4) & 7u);
+        const int pos = c * H + h;
+        const uint32_t bit = 1u << (pos & 31);
+        a.lo |= (pos < 32) ? bit : 0u;
+        a.hi |= (pos < 32) ? 0u : bit;
+        fills += 1u << c4;
+        const bool full = (h + 1 == m);
+        const uint32_t low = (1u << sh) - 1u;
+        list = full ? ((list & low) | ((list >> 4) & ~low)) : list;  // a full column leaves the ascending list
+        const bool hit = ord >= count;
+        count -= full ? 1 : 0;
+        const bool win = bb_has_four(a, H);
+        status = hit ? 3 : (win ? 1 : (count == 0 ? 2 : 0));
+        n++;
+        const BB t = a; a = b; b = t;
+    } while (status == 0);
+    s0 = ((uint64_t)r.s0h << 32) | r.s0l; s1 = ((uint64_t)r.s1h << 32) | r.s1l;
+    plies += n;
+    const int mover = (n & 1u) ? turn : -turn;  // side that made the last move
+    return status == 1 ? mover : (status == 2 ? 0 : 2);
 }
 
 // ---- kernels ----------------------------------------------------------------------------------------
@@ -244,7 +330,7 @@ __global__ void reset_kernel(const TreeRef *refs, int n_refs, const uint64_t *ro
     for (int i = 0; i < kMaxCols; i++) { h->mail[0][i] = 0; h->mail[1][i] = 0; }
     h->gen = 0; h->plies = 0; h->u1_events = 0;
     h->stat_levels = 0; h->stat_children = 0; h->stat_expanded = 0; h->stat_played = 0;
-    h->t_select = 0; h->t_expand = 0; h->t_playout = 0; h->t_backup = 0;
+    h->t_select = 0; h->t_expand = 0; h->t_playout = 0; h->t_backup = 0; h->t_exchange = 0;
 }
 
 struct LeafInfo {
@@ -328,7 +414,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
     if (!ACP && tid == 0) { e0 = ref.rng_expand[0]; e1 = ref.rng_expand[1]; }
     uint32_t plies = 0, u1 = 0;
     uint32_t st_levels = 0, st_children = 0, st_expanded = 0, st_played = 0;
-    unsigned long long tk_select = 0, tk_expand = 0, tk_playout = 0, tk_backup = 0, tk = 0;
+    unsigned long long tk_select = 0, tk_expand = 0, tk_playout = 0, tk_backup = 0, tk_exchange = 0, tk = 0;
     const bool timing = args.stage_timing != 0 && g == 0;
     const int root_turn = hdr->root_turn;
     uint32_t gen = hdr->gen;  // steps completed since reset
@@ -455,7 +541,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
             const uint64_t s0_start = s0, s1_start = s1;
             const uint32_t plies_start = plies;
             if (tid < P) {
-                outcome = fast_playout(geo, s_nth, pl_cur, pl_opp, pl_turn, s0, s1, plies);
+                outcome = fast_playout(geo, pl_cur, pl_opp, pl_turn, s0, s1, plies);
                 redo = outcome == 2;
             }
             const int par = step & 1;
@@ -516,6 +602,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
             }
             __syncthreads();
             if (s_abort) break;
+            if (timing) tk_exchange += wall_clock64() - tk;
         }
 
         // ================= backup (src/mctsnc.py:2083-2220) on the cached records =================
@@ -663,7 +750,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
         if (st_played) atomicAdd(&hdr->stat_played, (unsigned long long)st_played);
         if (g == 0) {  // identical in every workgroup of the tree
             hdr->stat_levels += st_levels; hdr->stat_children += st_children; hdr->stat_expanded += st_expanded;
-            if (timing) { hdr->t_select += tk_select; hdr->t_expand += tk_expand; hdr->t_playout += tk_playout; hdr->t_backup += tk_backup; }
+            if (timing) { hdr->t_select += tk_select; hdr->t_expand += tk_expand; hdr->t_playout += tk_playout; hdr->t_backup += tk_backup; hdr->t_exchange += tk_exchange; }
         }
     }
 }
@@ -673,7 +760,7 @@ struct TreeDigest {
     int32_t size, root_ns, max_depth, error;
     int64_t depth_sum;
     unsigned long long plies, u1_events, stat_levels, stat_children, stat_expanded, stat_played;
-    unsigned long long t_select, t_expand, t_playout, t_backup;
+    unsigned long long t_select, t_expand, t_playout, t_backup, t_exchange;
     int32_t child_mask;
     int32_t child_ns[kMaxCols], child_wins[kMaxCols];
     int8_t child_terminal[kMaxCols], child_outcome[kMaxCols];
@@ -690,7 +777,7 @@ __global__ void digest_kernel(const TreeRef *refs, int n_refs, TreeDigest *out) 
     d.size = h->size; d.root_ns = h->root_ns; d.max_depth = h->max_depth; d.error = h->error; d.depth_sum = h->depth_sum;
     d.plies = h->plies; d.u1_events = h->u1_events;
     d.stat_levels = h->stat_levels; d.stat_children = h->stat_children; d.stat_expanded = h->stat_expanded; d.stat_played = h->stat_played;
-    d.t_select = h->t_select; d.t_expand = h->t_expand; d.t_playout = h->t_playout; d.t_backup = h->t_backup;
+    d.t_select = h->t_select; d.t_expand = h->t_expand; d.t_playout = h->t_playout; d.t_backup = h->t_backup; d.t_exchange = h->t_exchange;
     d.child_mask = (root->flags & kLeaf) ? 0 : root->child_mask;
     for (int a = 0; a < kMaxCols; a++) {
         d.child_ns[a] = 0; d.child_wins[a] = 0; d.child_terminal[a] = 0; d.child_outcome[a] = 2;

@@ -220,6 +220,7 @@ void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_tu
     const double tick = 1e-8;  // wall_clock64 counts at 100 MHz
     out->time_select = dg[0].t_select * tick; out->time_expand = dg[0].t_expand * tick;
     out->time_playout = dg[0].t_playout * tick; out->time_backup = dg[0].t_backup * tick;
+    out->time_exchange = dg[0].t_exchange * tick;
     for (int t = 0; t < T; t++) {
         out->stat_levels += dg[t].stat_levels; out->stat_children += dg[t].stat_children;
         out->stat_expanded += dg[t].stat_expanded; out->stat_played += dg[t].stat_played;

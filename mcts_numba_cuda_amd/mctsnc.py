@@ -237,6 +237,7 @@ class MCTSNC:
         self.time_reduce_over_actions = 0.0  # both reductions are one pass here
         self.time_select, self.time_expand = res.time_select, res.time_expand
         self.time_playout, self.time_backup = res.time_playout, res.time_backup
+        self.time_exchange = res.time_exchange
         self._root_actions_expanded = np.array(res.root_actions_expanded[:A + 2], dtype=np.int16)
         self._root_ns = np.array(res.root_ns[:A], dtype=np.int64)
         self._actions_ns = np.array(res.actions_ns[:A], dtype=np.int64)
@@ -314,6 +315,7 @@ class MCTSNC:
         times_info["mean_expand"] = ms_factor * self.time_expand / steps
         times_info["mean_playout"] = ms_factor * self.time_playout / steps
         times_info["mean_backup"] = ms_factor * self.time_backup / steps
+        times_info["mean_exchange"] = ms_factor * self.time_exchange / steps  # part of mean_backup
         times_info["device_loop"] = ms_factor * self.time_device_loop
         performance_info["times_[ms]"] = times_info
         trees_info = {}
