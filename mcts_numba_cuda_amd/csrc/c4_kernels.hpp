@@ -240,24 +240,6 @@ __device__ __forceinline__ void rng_next32(Rng32 &r, uint32_t &out_lo, uint32_t 
     r.s1l = __builtin_amdgcn_alignbit(th, tl, 28); r.s1h = __builtin_amdgcn_alignbit(tl, th, 28);
 }
 
-// float32((x >> 11) * 2^-53) without double arithmetic.  Write x >> 11 = hi * 2^21 + f with f < 2^21; the value is
-// (hi + f * 2^-21) * 2^-32.  If hi >= 2^25 the float32 rounding drops at least two bits of hi, so folding "f != 0"
-// into bit 0 of hi (a sticky bit) leaves round-to-nearest-even unchanged.  Smaller values are first shifted left by
-// 7 or 14 bits (exact rescaling); below 2^43 (probability 2^-21) the double path is taken.
-__device__ __forceinline__ float uniform_from_bits(uint32_t lo, uint32_t hi) {
-    lo &= 0xfffff800u;  // the 11 bits that x >> 11 discards
-    float scale = 2.3283064365386963e-10f;  // 2^-32
-    if (__builtin_expect(hi < (1u << 25), 0)) {
-        if (hi >= (1u << 11)) {  // shift left by 14: hi' >= 2^25
-            hi = (hi << 14) | (lo >> 18); lo <<= 14; scale = 1.4210854715202004e-14f;  // 2^-46
-        } else {
-            return (float)((double)(((uint64_t)hi << 32 | lo) >> 11) * (1.0 / 9007199254740992.0));
-        }
-    }
-    const uint32_t t = hi | (lo != 0 ? 1u : 0u);
-    return (float)t * scale;
-}
-
 // cur: stones of the side to move, opp: the other side's.  Returns -1 / 0 / +1, or 2 when a draw of the
 // uniform rounded up to 1.0f (the caller then replays the playout with exact_playout).  The ply body is free of
 // branches: lanes leave through the loop condition only.

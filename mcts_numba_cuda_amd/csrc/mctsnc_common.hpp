@@ -77,6 +77,21 @@ __host__ __device__ inline double det_log(double x) {
 }
 
 #ifdef __HIPCC__
+// float32((x >> 11) * 2^-53) for x = hi * 2^32 + lo, without double arithmetic.  The 11 discarded bits are
+// cleared, the value is shifted left until hi has its top bit at position 25 or above (an exact rescaling), and the
+// bits left in lo are folded into bit 0 of hi as a sticky bit: float32 conversion then drops at least two bits of hi,
+// so round-to-nearest-even sees the same round and sticky information as the exact value.  (If hi was 0, the shift
+// moves all of lo into hi and nothing is left to fold.)
+__device__ __forceinline__ float uniform_from_bits(uint32_t lo, uint32_t hi) {
+    lo &= 0xfffff800u;
+    int sh = (int)__clz((int)hi) - 6;  // __clz(0) = 32
+    sh = sh < 0 ? 0 : sh;
+    const uint32_t hi2 = sh ? __builtin_amdgcn_alignbit(hi, lo, 32 - sh) : hi;
+    const uint32_t lo2 = lo << sh;
+    const uint32_t t = hi2 | (lo2 != 0 ? 1u : 0u);
+    return ldexpf((float)t, -32 - sh);
+}
+
 // UCB of one child with the reference's numba typing (src/mctsnc.py:1337): float64 arithmetic on
 // float32(child_n) and a float32 exploration constant, the sum narrowed to float32.
 __device__ __forceinline__ float ucb_value(int32_t wins, int32_t n, double log_parent_n, float c) {

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "c4_kernels.hpp"
+#include "gomoku_kernels.hpp"
 
 using namespace mctsnc;
 
@@ -91,6 +92,29 @@ struct mctsnc_engine {
     bool has_run = false;
     bool stage_timing = true;
     std::vector<uint64_t> rng_init_playout, rng_init_expand;  // the streams as seeded, kept for reseed()
+    // Gomoku pools
+    gomoku::Node *g_nodes = nullptr;
+    gomoku::Stat *g_stats = nullptr;
+    gomoku::TreeHdr *g_hdrs = nullptr;
+    gomoku::TreeRef *g_refs = nullptr;
+    gomoku::TreeDigest *g_digest = nullptr;
+    int16_t *g_ae = nullptr, *g_root_ae = nullptr;
+    int32_t *g_poc = nullptr, *g_path = nullptr, *g_child_counts = nullptr;
+    int8_t *g_child_info = nullptr;
+    uint32_t *g_root_bb = nullptr;
+    bool is_gomoku() const { return cfg.game == MCTSNC_GAME_GOMOKU; }
+};
+
+// What the final reductions need from one tree, whatever the game.
+struct TreeSummary {
+    int32_t size = 0, root_ns = 0, max_depth = 0;
+    int64_t depth_sum = 0;
+    unsigned long long plies = 0, u1_events = 0, stat_levels = 0, stat_children = 0, stat_expanded = 0, stat_played = 0;
+    unsigned long long t_select = 0, t_expand = 0, t_playout = 0, t_backup = 0, t_exchange = 0;
+    std::vector<int16_t> root_ae;                       // A + 2
+    std::vector<int32_t> child_ns, child_wins;          // per action of the root
+    std::vector<uint8_t> child_exists, child_terminal;
+    std::vector<int8_t> child_outcome;
 };
 
 namespace {
@@ -138,6 +162,11 @@ void free_device(mctsnc_engine *e) {
     if (e->d_root_bb) (void)hipFree(e->d_root_bb);
     if (e->d_root_turns) (void)hipFree(e->d_root_turns);
     if (e->d_abort) (void)hipFree(e->d_abort);
+    void *gp[] = {e->g_nodes, e->g_stats, e->g_hdrs, e->g_refs, e->g_digest, e->g_ae, e->g_root_ae, e->g_poc, e->g_path,
+                  e->g_child_counts, e->g_child_info, e->g_root_bb};
+    for (void *q : gp) if (q) (void)hipFree(q);
+    e->g_nodes = nullptr; e->g_stats = nullptr; e->g_hdrs = nullptr; e->g_refs = nullptr; e->g_digest = nullptr; e->g_ae = nullptr;
+    e->g_root_ae = nullptr; e->g_poc = nullptr; e->g_path = nullptr; e->g_child_counts = nullptr; e->g_child_info = nullptr; e->g_root_bb = nullptr;
     if (e->ev0) (void)hipEventDestroy(e->ev0);
     if (e->ev1) (void)hipEventDestroy(e->ev1);
     if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -173,13 +202,15 @@ struct Budget {
     double steps_limit, time_limit, forced;
 };
 
-// Final reductions over trees and actions (src/mctsnc.py:2222-2375) from the per-tree digests.
-void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_turn, mctsnc_result *out) {
+// Final reductions over trees and actions (src/mctsnc.py:2222-2375) from the per-tree summaries.
+void reduce_result(const mctsnc_engine *e, const TreeSummary *ts, int root_turn, mctsnc_result *out) {
     const mctsnc_config &c = e->cfg;
     const int A = c.max_actions, T = c.n_trees;
-    const int16_t *rae = dg[0].root_ae;
+    const int16_t *rae = ts[0].root_ae.data();
     for (int i = 0; i < A + 2; i++) out->root_actions_expanded[i] = rae[i];
-    const int nb = e->thrifty ? rae[A + 1] : A;
+    int nb = e->thrifty ? rae[A + 1] : A;
+    if (nb < 0) nb = 0;
+    if (nb > A) nb = A;
     out->n_root_entries = nb;
     for (int b = 0; b < A; b++) { out->root_ns[b] = 0; out->actions_ns[b] = 0; out->actions_ns_wins[b] = 0; out->actions_win_flags[b] = 0; }
     for (int b = 0; b < nb; b++) {
@@ -187,11 +218,11 @@ void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_tu
         if (action < 0 || action >= A) continue;
         if (e->thrifty || rae[action] != -1) {
             for (int t = 0; t < T; t++) {
-                out->root_ns[b] += dg[t].root_ns;
-                if ((dg[t].child_mask >> action) & 1) { out->actions_ns[b] += dg[t].child_ns[action]; out->actions_ns_wins[b] += dg[t].child_wins[action]; }
+                out->root_ns[b] += ts[t].root_ns;
+                if (ts[t].child_exists[action]) { out->actions_ns[b] += ts[t].child_ns[action]; out->actions_ns_wins[b] += ts[t].child_wins[action]; }
             }
         }
-        out->actions_win_flags[b] = ((dg[0].child_mask >> action) & 1) && dg[0].child_terminal[action] && dg[0].child_outcome[action] == root_turn;
+        out->actions_win_flags[b] = ts[0].child_exists[action] && ts[0].child_terminal[action] && ts[0].child_outcome[action] == root_turn;
     }
     // strided max-argmax over (win_flag, n, n_wins) with the left slot kept on ties (:2318-2330)
     const int size = next_pow2(A);
@@ -218,21 +249,35 @@ void reduce_result(const mctsnc_engine *e, const c4::TreeDigest *dg, int root_tu
     out->playout_plies = 0; out->u1_events = 0;
     out->stat_levels = out->stat_children = out->stat_expanded = out->stat_played = 0;
     const double tick = 1e-8;  // wall_clock64 counts at 100 MHz
-    out->time_select = dg[0].t_select * tick; out->time_expand = dg[0].t_expand * tick;
-    out->time_playout = dg[0].t_playout * tick; out->time_backup = dg[0].t_backup * tick;
-    out->time_exchange = dg[0].t_exchange * tick;
+    out->time_select = ts[0].t_select * tick; out->time_expand = ts[0].t_expand * tick;
+    out->time_playout = ts[0].t_playout * tick; out->time_backup = ts[0].t_backup * tick;
+    out->time_exchange = ts[0].t_exchange * tick;
     for (int t = 0; t < T; t++) {
-        out->stat_levels += dg[t].stat_levels; out->stat_children += dg[t].stat_children;
-        out->stat_expanded += dg[t].stat_expanded; out->stat_played += dg[t].stat_played;
-        out->depth_sum += dg[t].depth_sum; out->size_sum += dg[t].size;
-        if (dg[t].max_depth > out->max_depth) out->max_depth = dg[t].max_depth;
-        if (dg[t].size > out->max_size) out->max_size = dg[t].size;
-        out->playout_plies += dg[t].plies; out->u1_events += dg[t].u1_events;
+        out->stat_levels += ts[t].stat_levels; out->stat_children += ts[t].stat_children;
+        out->stat_expanded += ts[t].stat_expanded; out->stat_played += ts[t].stat_played;
+        out->depth_sum += ts[t].depth_sum; out->size_sum += ts[t].size;
+        if (ts[t].max_depth > out->max_depth) out->max_depth = ts[t].max_depth;
+        if (ts[t].size > out->max_size) out->max_size = ts[t].size;
+        out->playout_plies += ts[t].plies; out->u1_events += ts[t].u1_events;
     }
 }
 
-int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
-             const Budget &bud, mctsnc_result *out) {
+// Root of a Gomoku search: bitboards with bit = row * n + column; any arrangement of stones is accepted, as in the
+// reference (its outcome test only looks through the last stone placed).
+int gomoku_encode_root(const mctsnc_config &c, const int8_t *board, uint32_t bb[16]) {
+    for (int i = 0; i < 16; i++) bb[i] = 0;
+    for (int cell = 0; cell < c.board_m * c.board_n; cell++) {
+        const int8_t v = board[cell];
+        if (v != -1 && v != 0 && v != 1) return fail(MCTSNC_E_ROOT, "board holds %d at cell %d; cells must be -1, 0 or +1", v, cell);
+        if (v == 1) bb[cell >> 5] |= 1u << (cell & 31);
+        if (v == -1) bb[8 + (cell >> 5)] |= 1u << (cell & 31);
+    }
+    return MCTSNC_OK;
+}
+
+int gomoku_block(const mctsnc_config &c) { return c.n_playouts < 64 ? 64 : (c.n_playouts > gomoku::kMaxThreads ? gomoku::kMaxThreads : c.n_playouts); }
+
+int check_batch(mctsnc_engine **engines, int n, const int32_t *turns) {
     if (n < 1) return fail(MCTSNC_E_INVALID, "no engines given");
     mctsnc_engine *e0 = engines[0];
     for (int i = 0; i < n; i++) {
@@ -244,64 +289,21 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
             return fail(MCTSNC_E_INVALID, "engines of one batch must share their configuration");
         for (int j = 0; j < i; j++)
             if (engines[j] == e) return fail(MCTSNC_E_INVALID, "engine %d appears twice in the batch", i);
-    }
-    const mctsnc_config &c = e0->cfg;
-    const int T = c.n_trees, mn = c.board_m * c.board_n;
-    const int n_refs = n * T;
-    const double t_start = now_s();
-    HIP_TRY(hipSetDevice(c.device));
-
-    for (int i = 0; i < n; i++)
         if (turns[i] != 1 && turns[i] != -1) return fail(MCTSNC_E_ROOT, "root_turn must be -1 or +1");
-    std::vector<uint64_t> bb((size_t)n_refs * 2);
-    std::vector<int32_t> tr((size_t)n_refs);
-    for (int i = 0; i < n; i++) {
-        uint64_t b2[2];
-        int rc = c4_encode_root(c, boards + (size_t)i * mn, extras ? extras + (size_t)i * extra_len : nullptr, extra_len, b2);
-        if (rc) return rc;
-        for (int t = 0; t < T; t++) { bb[2 * ((size_t)i * T + t)] = b2[0]; bb[2 * ((size_t)i * T + t) + 1] = b2[1]; tr[(size_t)i * T + t] = turns[i]; }
     }
+    return MCTSNC_OK;
+}
 
-    // the refs / root / digest buffers of a batch are laid out engine after engine
-    c4::TreeRef *d_refs = e0->d_refs;
-    uint64_t *d_bb = e0->d_root_bb;
-    int32_t *d_turns = e0->d_root_turns;
-    c4::TreeDigest *d_digest = e0->d_digest;
-    bool temp = false;
-    if (n > 1) {
-        temp = true;
-        std::vector<c4::TreeRef> refs((size_t)n_refs);
-        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->d_refs, sizeof(c4::TreeRef) * T, hipMemcpyDeviceToHost));
-        HIP_TRY(hipMalloc(&d_refs, sizeof(c4::TreeRef) * n_refs));
-        HIP_TRY(hipMalloc(&d_bb, sizeof(uint64_t) * 2 * n_refs));
-        HIP_TRY(hipMalloc(&d_turns, sizeof(int32_t) * n_refs));
-        HIP_TRY(hipMalloc(&d_digest, sizeof(c4::TreeDigest) * n_refs));
-        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
-    }
-    auto cleanup = [&]() {
-        if (temp) { (void)hipFree(d_refs); (void)hipFree(d_bb); (void)hipFree(d_turns); (void)hipFree(d_digest); }
-    };
+// The search loop: chunks of steps on the device, the budget checked between chunks.  launch(nsteps) enqueues one
+// launch of the persistent kernel on the engine's stream.
+template <typename Launch>
+int budget_loop(mctsnc_engine *e0, const Budget &bud, Launch launch, int64_t &steps, double &dev_time, double &time_loop) {
     hipStream_t stream = e0->stream;
-    hipError_t herr;
-#define HIP_TRY_C(expr) do { herr = (expr); if (herr != hipSuccess) { cleanup(); return fail(MCTSNC_E_HIP, "%s failed: %s", #expr, hipGetErrorString(herr)); } } while (0)
-    HIP_TRY_C(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
-    HIP_TRY_C(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
-    HIP_TRY_C(hipMemsetAsync(e0->d_abort, 0, sizeof(int32_t), stream));
-    hipLaunchKernelGGL(c4::reset_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_bb, d_turns);
-    HIP_TRY_C(hipGetLastError());
-    HIP_TRY_C(hipStreamSynchronize(stream));
-
-    // ---- the search loop: chunks of steps on the device, the budget checked between chunks ----
-    c4::SearchArgs args;
-    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
-    args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
-    args.stage_timing = e0->stage_timing ? 1 : 0;
-    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
     const bool forced = bud.forced < INFINITY;
     const double step_budget = forced ? bud.forced : bud.steps_limit;
     const double time_budget = forced ? INFINITY : bud.time_limit;
-    int64_t steps = 0;
-    double dev_time = 0.0;
+    steps = 0;
+    dev_time = 0.0;
     const double t_loop = now_s();
     for (;;) {
         const double elapsed = now_s() - t_loop;
@@ -320,39 +322,32 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
             if (by_time < 1.0) by_time = 1.0;
             if (chunk > by_time) chunk = by_time;
         }
-        args.nsteps = (int32_t)chunk;
-        if (args.nsteps < 1) break;
-        HIP_TRY_C(hipEventRecord(e0->ev0, stream));
-        if (e0->acp) {
-            void *kargs[] = {&args};
-            HIP_TRY_C(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, 0, stream));
-        } else {
-            hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, 0, stream, args);
-            HIP_TRY_C(hipGetLastError());
-        }
-        HIP_TRY_C(hipEventRecord(e0->ev1, stream));
-        HIP_TRY_C(hipStreamSynchronize(stream));
+        const int32_t nsteps = (int32_t)chunk;
+        if (nsteps < 1) break;
+        HIP_TRY(hipEventRecord(e0->ev0, stream));
+        int rc = launch(nsteps);
+        if (rc) return rc;
+        HIP_TRY(hipEventRecord(e0->ev1, stream));
+        HIP_TRY(hipStreamSynchronize(stream));
         float ms = 0.f;
-        HIP_TRY_C(hipEventElapsedTime(&ms, e0->ev0, e0->ev1));
+        HIP_TRY(hipEventElapsedTime(&ms, e0->ev0, e0->ev1));
         dev_time += ms * 1e-3;
-        steps += args.nsteps;
+        steps += nsteps;
         int32_t aborted = 0;
-        HIP_TRY_C(hipMemcpy(&aborted, e0->d_abort, sizeof aborted, hipMemcpyDeviceToHost));
-        if (aborted) { cleanup(); return fail(MCTSNC_E_DEVICE_SYNC, "device-side step synchronisation timed out after %lld steps", (long long)steps); }
+        HIP_TRY(hipMemcpy(&aborted, e0->d_abort, sizeof aborted, hipMemcpyDeviceToHost));
+        if (aborted) return fail(MCTSNC_E_DEVICE_SYNC, "device-side step synchronisation timed out after %lld steps", (long long)steps);
     }
-    const double time_loop = now_s() - t_loop;
+    time_loop = now_s() - t_loop;
+    return MCTSNC_OK;
+}
 
-    // ---- final reductions ----
-    const double t_red = now_s();
-    hipLaunchKernelGGL(c4::digest_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_digest);
-    HIP_TRY_C(hipGetLastError());
-    std::vector<c4::TreeDigest> dg((size_t)n_refs);
-    HIP_TRY_C(hipMemcpyAsync(dg.data(), d_digest, sizeof(c4::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
-    HIP_TRY_C(hipStreamSynchronize(stream));
+void finish_results(mctsnc_engine **engines, int n, const std::vector<TreeSummary> &ts, const int32_t *turns, int64_t steps, double t_start,
+                    double t_red, double time_loop, double dev_time, mctsnc_result *out) {
+    const int T = engines[0]->cfg.n_trees;
     for (int i = 0; i < n; i++) {
         mctsnc_result *o = out + i;
         memset(o, 0, sizeof *o);
-        reduce_result(engines[i], dg.data() + (size_t)i * T, turns[i], o);
+        reduce_result(engines[i], ts.data() + (size_t)i * T, turns[i], o);
         o->steps = steps;
         engines[i]->has_run = true;
     }
@@ -360,8 +355,254 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     for (int i = 0; i < n; i++) {
         out[i].time_loop = time_loop; out[i].time_reduce = t_end - t_red; out[i].time_total = t_end - t_start; out[i].time_device_loop = dev_time;
     }
-    cleanup();
-#undef HIP_TRY_C
+}
+
+// RAII holder for the temporary device buffers of a batched run
+struct TempBuffers {
+    std::vector<void *> ptrs;
+    ~TempBuffers() { for (void *p : ptrs) (void)hipFree(p); }
+    template <typename T> int alloc(T **out, size_t count) {
+        void *p = nullptr;
+        hipError_t err = hipMalloc(&p, sizeof(T) * count);
+        if (err != hipSuccess) return fail(MCTSNC_E_HIP, "hipMalloc of a batch buffer failed: %s", hipGetErrorString(err));
+        ptrs.push_back(p);
+        *out = static_cast<T *>(p);
+        return MCTSNC_OK;
+    }
+};
+
+int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
+                const Budget &bud, mctsnc_result *out) {
+    mctsnc_engine *e0 = engines[0];
+    const mctsnc_config &c = e0->cfg;
+    const int T = c.n_trees, mn = c.board_m * c.board_n, A = c.max_actions;
+    const int n_refs = n * T;
+    const double t_start = now_s();
+    std::vector<uint64_t> bb((size_t)n_refs * 2);
+    std::vector<int32_t> tr((size_t)n_refs);
+    for (int i = 0; i < n; i++) {
+        uint64_t b2[2];
+        int rc = c4_encode_root(c, boards + (size_t)i * mn, extras ? extras + (size_t)i * extra_len : nullptr, extra_len, b2);
+        if (rc) return rc;
+        for (int t = 0; t < T; t++) { bb[2 * ((size_t)i * T + t)] = b2[0]; bb[2 * ((size_t)i * T + t) + 1] = b2[1]; tr[(size_t)i * T + t] = turns[i]; }
+    }
+    // the refs / root / digest buffers of a batch are laid out engine after engine
+    c4::TreeRef *d_refs = e0->d_refs;
+    uint64_t *d_bb = e0->d_root_bb;
+    int32_t *d_turns = e0->d_root_turns;
+    c4::TreeDigest *d_digest = e0->d_digest;
+    TempBuffers tmp;
+    if (n > 1) {
+        std::vector<c4::TreeRef> refs((size_t)n_refs);
+        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->d_refs, sizeof(c4::TreeRef) * T, hipMemcpyDeviceToHost));
+        int rc;
+        if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 2 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) || (rc = tmp.alloc(&d_digest, n_refs))) return rc;
+        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
+    }
+    hipStream_t stream = e0->stream;
+    HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY(hipMemsetAsync(e0->d_abort, 0, sizeof(int32_t), stream));
+    hipLaunchKernelGGL(c4::reset_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_bb, d_turns);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize(stream));
+
+    c4::SearchArgs args;
+    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
+    args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
+    args.stage_timing = e0->stage_timing ? 1 : 0;
+    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    int64_t steps; double dev_time, time_loop;
+    int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
+        args.nsteps = nsteps;
+        if (e0->acp) {
+            void *kargs[] = {&args};
+            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, 0, stream));
+        } else {
+            hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, 0, stream, args);
+            HIP_TRY(hipGetLastError());
+        }
+        return MCTSNC_OK;
+    }, steps, dev_time, time_loop);
+    if (rc) return rc;
+
+    const double t_red = now_s();
+    hipLaunchKernelGGL(c4::digest_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_digest);
+    HIP_TRY(hipGetLastError());
+    std::vector<c4::TreeDigest> dg((size_t)n_refs);
+    HIP_TRY(hipMemcpyAsync(dg.data(), d_digest, sizeof(c4::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    std::vector<TreeSummary> ts((size_t)n_refs);
+    for (int r = 0; r < n_refs; r++) {
+        const c4::TreeDigest &d = dg[r];
+        TreeSummary &t = ts[r];
+        t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
+        t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
+        t.stat_expanded = d.stat_expanded; t.stat_played = d.stat_played;
+        t.t_select = d.t_select; t.t_expand = d.t_expand; t.t_playout = d.t_playout; t.t_backup = d.t_backup; t.t_exchange = d.t_exchange;
+        t.root_ae.assign(d.root_ae, d.root_ae + A + 2);
+        t.child_ns.resize(A); t.child_wins.resize(A); t.child_exists.resize(A); t.child_terminal.resize(A); t.child_outcome.resize(A);
+        for (int a = 0; a < A; a++) {
+            t.child_exists[a] = (d.child_mask >> a) & 1; t.child_ns[a] = d.child_ns[a]; t.child_wins[a] = d.child_wins[a];
+            t.child_terminal[a] = d.child_terminal[a]; t.child_outcome[a] = d.child_outcome[a];
+        }
+    }
+    finish_results(engines, n, ts, turns, steps, t_start, t_red, time_loop, dev_time, out);
+    return MCTSNC_OK;
+}
+
+int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const int32_t *turns, const Budget &bud, mctsnc_result *out) {
+    mctsnc_engine *e0 = engines[0];
+    const mctsnc_config &c = e0->cfg;
+    const int T = c.n_trees, cells = c.board_m * c.board_n, A = c.max_actions;
+    const int n_refs = n * T;
+    const double t_start = now_s();
+    std::vector<uint32_t> bb((size_t)n_refs * 16);
+    std::vector<int32_t> tr((size_t)n_refs);
+    for (int i = 0; i < n; i++) {
+        uint32_t b16[16];
+        int rc = gomoku_encode_root(c, boards + (size_t)i * cells, b16);
+        if (rc) return rc;
+        for (int t = 0; t < T; t++) { memcpy(&bb[16 * ((size_t)i * T + t)], b16, sizeof b16); tr[(size_t)i * T + t] = turns[i]; }
+    }
+    gomoku::TreeRef *d_refs = e0->g_refs;
+    uint32_t *d_bb = e0->g_root_bb;
+    int32_t *d_turns = e0->d_root_turns;
+    gomoku::TreeDigest *d_digest = e0->g_digest;
+    int32_t *d_counts = e0->g_child_counts;
+    int8_t *d_info = e0->g_child_info;
+    TempBuffers tmp;
+    if (n > 1) {
+        std::vector<gomoku::TreeRef> refs((size_t)n_refs);
+        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->g_refs, sizeof(gomoku::TreeRef) * T, hipMemcpyDeviceToHost));
+        int rc;
+        if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 16 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) ||
+            (rc = tmp.alloc(&d_digest, n_refs)) || (rc = tmp.alloc(&d_counts, (size_t)n_refs * A * 2)) || (rc = tmp.alloc(&d_info, (size_t)n_refs * A * 3))) return rc;
+        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(gomoku::TreeRef) * n_refs, hipMemcpyHostToDevice));
+    }
+    hipStream_t stream = e0->stream;
+    HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint32_t) * 16 * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY(hipMemsetAsync(e0->d_abort, 0, sizeof(int32_t), stream));
+    hipLaunchKernelGGL(gomoku::reset_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_bb, d_turns);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize(stream));
+
+    gomoku::SearchArgs args;
+    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
+    args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
+    args.stage_timing = e0->stage_timing ? 1 : 0;
+    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->block);
+    int64_t steps; double dev_time, time_loop;
+    int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
+        args.nsteps = nsteps;
+        if (e0->acp) {
+            void *kargs[] = {&args};
+            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+        } else {
+            hipLaunchKernelGGL(gomoku::search_kernel<false>, grid, block, lds, stream, args);
+            HIP_TRY(hipGetLastError());
+        }
+        return MCTSNC_OK;
+    }, steps, dev_time, time_loop);
+    if (rc) return rc;
+
+    const double t_red = now_s();
+    hipLaunchKernelGGL(gomoku::digest_kernel, dim3(n_refs), dim3(256), 0, stream, d_refs, n_refs, cells, d_digest, d_counts, d_info);
+    HIP_TRY(hipGetLastError());
+    std::vector<gomoku::TreeDigest> dg((size_t)n_refs);
+    std::vector<int32_t> counts((size_t)n_refs * A * 2);
+    std::vector<int8_t> info((size_t)n_refs * A * 3);
+    std::vector<int16_t> rae((size_t)(A + 2));
+    HIP_TRY(hipMemcpyAsync(dg.data(), d_digest, sizeof(gomoku::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipMemcpyAsync(counts.data(), d_counts, counts.size() * sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipMemcpyAsync(info.data(), d_info, info.size(), hipMemcpyDeviceToHost, stream));
+    HIP_TRY(hipStreamSynchronize(stream));
+    std::vector<TreeSummary> ts((size_t)n_refs);
+    for (int r = 0; r < n_refs; r++) {
+        const gomoku::TreeDigest &d = dg[r];
+        TreeSummary &t = ts[r];
+        t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
+        t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
+        t.stat_expanded = d.stat_expanded; t.stat_played = d.stat_played;
+        t.t_select = d.t_select; t.t_expand = d.t_expand; t.t_playout = d.t_playout; t.t_backup = d.t_backup; t.t_exchange = d.t_exchange;
+        t.root_ae.assign((size_t)A + 2, 0);
+        if (r % T == 0) {  // only tree 0 of an engine holds the memorised row the reductions use
+            HIP_TRY(hipMemcpy(t.root_ae.data(), engines[r / T]->g_root_ae, sizeof(int16_t) * (A + 2), hipMemcpyDeviceToHost));
+        }
+        t.child_ns.resize(A); t.child_wins.resize(A); t.child_exists.resize(A); t.child_terminal.resize(A); t.child_outcome.resize(A);
+        for (int a = 0; a < A; a++) {
+            t.child_ns[a] = counts[((size_t)r * A + a) * 2]; t.child_wins[a] = counts[((size_t)r * A + a) * 2 + 1];
+            t.child_exists[a] = (uint8_t)info[((size_t)r * A + a) * 3]; t.child_terminal[a] = (uint8_t)info[((size_t)r * A + a) * 3 + 1];
+            t.child_outcome[a] = info[((size_t)r * A + a) * 3 + 2];
+        }
+    }
+    finish_results(engines, n, ts, turns, steps, t_start, t_red, time_loop, dev_time, out);
+    return MCTSNC_OK;
+}
+
+int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
+             const Budget &bud, mctsnc_result *out) {
+    int rc = check_batch(engines, n, turns);
+    if (rc) return rc;
+    HIP_TRY(hipSetDevice(engines[0]->cfg.device));
+    if (engines[0]->is_gomoku()) return run_many_gomoku(engines, n, boards, turns, bud, out);
+    return run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out);
+}
+
+int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t need) {
+    const mctsnc_config &c = e->cfg;
+    const int A = c.max_actions, m = c.board_m, n = c.board_n, E = c.extra_info_memory;
+    gomoku::TreeHdr h;
+    HIP_TRY(hipMemcpy(&h, e->g_hdrs + tree, sizeof h, hipMemcpyDeviceToHost));
+    switch (array_id) {
+        case MCTSNC_ARR_SELECTED_PATH: if (need) HIP_TRY(hipMemcpy(dst, e->g_path + (size_t)tree * gomoku::kMaxPath, need, hipMemcpyDeviceToHost)); return MCTSNC_OK;
+        case MCTSNC_ARR_ACTIONS_EXPANDED: HIP_TRY(hipMemcpy(dst, e->g_ae + (size_t)tree * (A + 2), need, hipMemcpyDeviceToHost)); return MCTSNC_OK;
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES: { int32_t v[2] = {h.po_neg, h.po_pos}; memcpy(dst, v, 8); return MCTSNC_OK; }
+        case MCTSNC_ARR_PLAYOUT_OUTCOMES_CHILDREN: HIP_TRY(hipMemcpy(dst, e->g_poc + (size_t)tree * 2 * A, need, hipMemcpyDeviceToHost)); return MCTSNC_OK;
+        case MCTSNC_ARR_NODE_SELECTED: memcpy(dst, &h.selected, 4); return MCTSNC_OK;
+        default: break;
+    }
+    const int64_t sz = h.size;
+    const size_t S = (size_t)c.max_tree_size;
+    std::vector<gomoku::Node> nd((size_t)sz);
+    std::vector<gomoku::Stat> st((size_t)sz);
+    HIP_TRY(hipMemcpy(nd.data(), e->g_nodes + (size_t)tree * S, sizeof(gomoku::Node) * (size_t)sz, hipMemcpyDeviceToHost));
+    if (array_id == MCTSNC_ARR_NS || array_id == MCTSNC_ARR_NS_WINS)
+        HIP_TRY(hipMemcpy(st.data(), e->g_stats + (size_t)tree * S, sizeof(gomoku::Stat) * (size_t)sz, hipMemcpyDeviceToHost));
+    for (int64_t i = 0; i < sz; i++) {
+        const gomoku::Node &x = nd[(size_t)i];
+        switch (array_id) {
+            case MCTSNC_ARR_TREES: {
+                int32_t *row = (int32_t *)dst + i * (1 + A);
+                row[0] = x.parent;
+                int rank = 0;
+                const bool expanded = !(x.flags & gomoku::kLeaf);
+                for (int a = 0; a < A; a++) {
+                    const bool empty = !((x.bb_pos[a >> 5] | x.bb_neg[a >> 5]) >> (a & 31) & 1u);
+                    row[1 + a] = (expanded && empty && rank < x.n_children) ? x.child_base + rank : -1;
+                    if (empty) rank++;
+                }
+                break;
+            }
+            case MCTSNC_ARR_DEPTHS: ((int16_t *)dst)[i] = x.depth; break;
+            case MCTSNC_ARR_TURNS: ((int8_t *)dst)[i] = x.turn; break;
+            case MCTSNC_ARR_LEAVES: ((uint8_t *)dst)[i] = (x.flags & gomoku::kLeaf) ? 1 : 0; break;
+            case MCTSNC_ARR_TERMINALS: ((uint8_t *)dst)[i] = (x.flags & gomoku::kTerminal) ? 1 : 0; break;
+            case MCTSNC_ARR_OUTCOMES: ((int8_t *)dst)[i] = x.outcome; break;
+            case MCTSNC_ARR_NS: ((int32_t *)dst)[i] = st[(size_t)i].ns; break;
+            case MCTSNC_ARR_NS_WINS: ((int32_t *)dst)[i] = st[(size_t)i].wins; break;
+            case MCTSNC_ARR_BOARDS: {
+                int8_t *b = (int8_t *)dst + i * m * n;
+                for (int cell = 0; cell < m * n; cell++)
+                    b[cell] = ((x.bb_pos[cell >> 5] >> (cell & 31)) & 1u) ? 1 : (((x.bb_neg[cell >> 5] >> (cell & 31)) & 1u) ? -1 : 0);
+                break;
+            }
+            case MCTSNC_ARR_EXTRA_INFOS: memset((int8_t *)dst + i * E, 0, (size_t)E); break;
+            default: return fail(MCTSNC_E_INVALID, "unknown array id %d", array_id);
+        }
+    }
     return MCTSNC_OK;
 }
 
@@ -374,11 +615,18 @@ const char *mctsnc_last_error(void) { return g_error.c_str(); }
 int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
     if (!cfg || !out) return fail(MCTSNC_E_INVALID, "null argument");
     const mctsnc_config &c = *cfg;
-    if (c.game != MCTSNC_GAME_C4) return fail(MCTSNC_E_INVALID, "game %d is not available in this build (Connect 4 only)", c.game);
-    if (c.board_m < 1 || c.board_n < 1 || c.board_n > c4::kMaxCols || (c.board_m + 1) * c.board_n > 64)
-        return fail(MCTSNC_E_INVALID, "Connect 4 board %dx%d unsupported: needs columns <= %d and (rows + 1) * columns <= 64", c.board_m, c.board_n, c4::kMaxCols);
-    if (c.max_actions != c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 has one action per column (%d), got max_actions = %d", c.board_n, c.max_actions);
-    if (c.extra_info_memory < c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 keeps the column fills in extra_info: needs >= %d bytes", c.board_n);
+    if (c.game != MCTSNC_GAME_C4 && c.game != MCTSNC_GAME_GOMOKU) return fail(MCTSNC_E_INVALID, "unknown game %d", c.game);
+    if (c.game == MCTSNC_GAME_C4) {
+        if (c.board_m < 1 || c.board_n < 1 || c.board_n > c4::kMaxCols || (c.board_m + 1) * c.board_n > 64)
+            return fail(MCTSNC_E_INVALID, "Connect 4 board %dx%d unsupported: needs columns <= %d and (rows + 1) * columns <= 64", c.board_m, c.board_n, c4::kMaxCols);
+        if (c.max_actions != c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 has one action per column (%d), got max_actions = %d", c.board_n, c.max_actions);
+        if (c.extra_info_memory < c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 keeps the column fills in extra_info: needs >= %d bytes", c.board_n);
+    } else {
+        if (c.board_m < 5 || c.board_n < 5 || c.board_m > 16 || c.board_n > 16)
+            return fail(MCTSNC_E_INVALID, "Gomoku board %dx%d unsupported: sides must be in [5, 16]", c.board_m, c.board_n);
+        if (c.max_actions != c.board_m * c.board_n) return fail(MCTSNC_E_INVALID, "Gomoku has one action per cell (%d), got max_actions = %d", c.board_m * c.board_n, c.max_actions);
+        if (c.extra_info_memory < 1) return fail(MCTSNC_E_INVALID, "extra_info_memory must be >= 1");
+    }
     if (c.n_trees < 1 || c.n_trees > 512) return fail(MCTSNC_E_INVALID, "n_trees must be in [1, 512]");
     if (c.n_playouts < 1 || c.n_playouts > 512 || (c.n_playouts & (c.n_playouts - 1))) return fail(MCTSNC_E_INVALID, "n_playouts must be a power of two <= 512");
     if (c.variant < MCTSNC_OCP_THRIFTY || c.variant > MCTSNC_ACP_PRODIGAL) return fail(MCTSNC_E_INVALID, "unknown variant %d", c.variant);
@@ -388,8 +636,13 @@ int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
     e->cfg = c;
     e->acp = c.variant >= MCTSNC_ACP_THRIFTY;
     e->thrifty = (c.variant == MCTSNC_OCP_THRIFTY || c.variant == MCTSNC_ACP_THRIFTY);
-    e->G = e->acp ? c.board_n : 1;
-    e->block = c.n_playouts < 64 ? 64 : c.n_playouts;
+    if (c.game == MCTSNC_GAME_C4) {
+        e->G = e->acp ? c.board_n : 1;
+        e->block = c.n_playouts < 64 ? 64 : c.n_playouts;
+    } else {
+        e->G = e->acp ? (c.max_actions < 32 ? c.max_actions : 32) : 1;  // workgroups per tree; each takes every G-th child
+        e->block = gomoku_block(c);
+    }
     // tpb table of src/mctsnc.py:360-365 with cuda_tpb_default = 512: fixes which expand generators OCP uses
     const int tpb_board = next_pow2(c.board_m * c.board_n), tpb_extra = next_pow2(c.extra_info_memory), tpb_actions = next_pow2(c.max_actions);
     int tpb_r = tpb_board > tpb_extra ? tpb_board : tpb_extra; if (tpb_r > 512) tpb_r = 512;
@@ -414,26 +667,64 @@ int mctsnc_init_device(mctsnc_engine *e) {
     HIP_TRY(hipStreamCreate(&e->stream));
     HIP_TRY(hipEventCreate(&e->ev0));
     HIP_TRY(hipEventCreate(&e->ev1));
-    HIP_TRY(hipMalloc(&e->d_nodes, sizeof(c4::Node) * S * T));
-    HIP_TRY(hipMalloc(&e->d_hdrs, sizeof(c4::TreeHdr) * T));
-    HIP_TRY(hipMemset(e->d_hdrs, 0, sizeof(c4::TreeHdr) * T));
     e->n_rng_playout = e->acp ? (int64_t)T * c.max_actions * c.n_playouts : (int64_t)T * c.n_playouts;
     e->n_rng_expand = e->acp ? 0 : T;
     HIP_TRY(hipMalloc(&e->d_rng_playout, sizeof(uint64_t) * 2 * e->n_rng_playout));
     if (!e->acp) HIP_TRY(hipMalloc(&e->d_rng_expand, sizeof(uint64_t) * 2 * T));
-    HIP_TRY(hipMalloc(&e->d_refs, sizeof(c4::TreeRef) * T));
-    HIP_TRY(hipMalloc(&e->d_digest, sizeof(c4::TreeDigest) * T));
-    HIP_TRY(hipMalloc(&e->d_root_bb, sizeof(uint64_t) * 2 * T));
     HIP_TRY(hipMalloc(&e->d_root_turns, sizeof(int32_t) * T));
     HIP_TRY(hipMalloc(&e->d_abort, sizeof(int32_t)));
-    std::vector<c4::TreeRef> refs((size_t)T);
-    for (int t = 0; t < T; t++) {
-        refs[t].nodes = e->d_nodes + (size_t)t * S;
-        refs[t].hdr = e->d_hdrs + t;
-        refs[t].rng_playout = e->d_rng_playout + 2 * (size_t)t * (e->acp ? c.max_actions * c.n_playouts : c.n_playouts);
-        refs[t].rng_expand = e->acp ? nullptr : e->d_rng_expand + 2 * (size_t)t;
+    const size_t rng_per_tree = (size_t)(e->acp ? c.max_actions * c.n_playouts : c.n_playouts);
+    if (!e->is_gomoku()) {
+        HIP_TRY(hipMalloc(&e->d_nodes, sizeof(c4::Node) * S * T));
+        HIP_TRY(hipMalloc(&e->d_hdrs, sizeof(c4::TreeHdr) * T));
+        HIP_TRY(hipMemset(e->d_hdrs, 0, sizeof(c4::TreeHdr) * T));
+        HIP_TRY(hipMalloc(&e->d_refs, sizeof(c4::TreeRef) * T));
+        HIP_TRY(hipMalloc(&e->d_digest, sizeof(c4::TreeDigest) * T));
+        HIP_TRY(hipMalloc(&e->d_root_bb, sizeof(uint64_t) * 2 * T));
+        std::vector<c4::TreeRef> refs((size_t)T);
+        for (int t = 0; t < T; t++) {
+            refs[t].nodes = e->d_nodes + (size_t)t * S;
+            refs[t].hdr = e->d_hdrs + t;
+            refs[t].rng_playout = e->d_rng_playout + 2 * (size_t)t * rng_per_tree;
+            refs[t].rng_expand = e->acp ? nullptr : e->d_rng_expand + 2 * (size_t)t;
+        }
+        HIP_TRY(hipMemcpy(e->d_refs, refs.data(), sizeof(c4::TreeRef) * T, hipMemcpyHostToDevice));
+    } else {
+        const int A = c.max_actions;
+        HIP_TRY(hipMalloc(&e->g_nodes, sizeof(gomoku::Node) * S * T));
+        HIP_TRY(hipMalloc(&e->g_stats, sizeof(gomoku::Stat) * S * T));
+        HIP_TRY(hipMalloc(&e->g_hdrs, sizeof(gomoku::TreeHdr) * T));
+        HIP_TRY(hipMemset(e->g_hdrs, 0, sizeof(gomoku::TreeHdr) * T));
+        HIP_TRY(hipMalloc(&e->g_refs, sizeof(gomoku::TreeRef) * T));
+        HIP_TRY(hipMalloc(&e->g_digest, sizeof(gomoku::TreeDigest) * T));
+        HIP_TRY(hipMalloc(&e->g_ae, sizeof(int16_t) * (A + 2) * T));
+        HIP_TRY(hipMemset(e->g_ae, 0, sizeof(int16_t) * (A + 2) * T));
+        HIP_TRY(hipMalloc(&e->g_root_ae, sizeof(int16_t) * (A + 2) * T));
+        HIP_TRY(hipMemset(e->g_root_ae, 0, sizeof(int16_t) * (A + 2) * T));
+        HIP_TRY(hipMalloc(&e->g_poc, sizeof(int32_t) * 2 * A * T));
+        HIP_TRY(hipMemset(e->g_poc, 0, sizeof(int32_t) * 2 * A * T));
+        HIP_TRY(hipMalloc(&e->g_path, sizeof(int32_t) * gomoku::kMaxPath * T));
+        HIP_TRY(hipMalloc(&e->g_child_counts, sizeof(int32_t) * 2 * A * T));
+        HIP_TRY(hipMalloc(&e->g_child_info, (size_t)3 * A * T));
+        HIP_TRY(hipMalloc(&e->g_root_bb, sizeof(uint32_t) * 16 * T));
+        std::vector<gomoku::TreeRef> refs((size_t)T);
+        for (int t = 0; t < T; t++) {
+            refs[t].nodes = e->g_nodes + (size_t)t * S;
+            refs[t].stats = e->g_stats + (size_t)t * S;
+            refs[t].hdr = e->g_hdrs + t;
+            refs[t].rng_playout = e->d_rng_playout + 2 * (size_t)t * rng_per_tree;
+            refs[t].rng_expand = e->acp ? nullptr : e->d_rng_expand + 2 * (size_t)t;
+            refs[t].ae = e->g_ae + (size_t)t * (A + 2);
+            refs[t].root_ae = e->g_root_ae + (size_t)t * (A + 2);
+            refs[t].poc = e->g_poc + (size_t)t * 2 * A;
+            refs[t].path = e->g_path + (size_t)t * gomoku::kMaxPath;
+        }
+        HIP_TRY(hipMemcpy(e->g_refs, refs.data(), sizeof(gomoku::TreeRef) * T, hipMemcpyHostToDevice));
+        // the playout state of a workgroup can need more LDS than the default limit allows
+        const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->block);
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     }
-    HIP_TRY(hipMemcpy(e->d_refs, refs.data(), sizeof(c4::TreeRef) * T, hipMemcpyHostToDevice));
     int rc = upload_rng(e);
     if (rc) return rc;
     if (e->acp) {
@@ -488,9 +779,16 @@ int64_t mctsnc_read_size(mctsnc_engine *e, int32_t array_id, int32_t tree) {
     if (tree < 0 || tree >= c.n_trees) return fail(MCTSNC_E_INVALID, "tree %d out of range", tree);
     if (!e->has_run) return fail(MCTSNC_E_STATE, "no search has run yet");
     if (hipSetDevice(c.device) != hipSuccess) return fail(MCTSNC_E_HIP, "hipSetDevice failed");
-    c4::TreeHdr h;
-    if (hipMemcpy(&h, e->d_hdrs + tree, sizeof h, hipMemcpyDeviceToHost) != hipSuccess) return fail(MCTSNC_E_HIP, "header copy failed");
-    const int64_t sz = h.size;
+    int64_t sz, path_len;
+    if (e->is_gomoku()) {
+        gomoku::TreeHdr h;
+        if (hipMemcpy(&h, e->g_hdrs + tree, sizeof h, hipMemcpyDeviceToHost) != hipSuccess) return fail(MCTSNC_E_HIP, "header copy failed");
+        sz = h.size; path_len = h.path_len;
+    } else {
+        c4::TreeHdr h;
+        if (hipMemcpy(&h, e->d_hdrs + tree, sizeof h, hipMemcpyDeviceToHost) != hipSuccess) return fail(MCTSNC_E_HIP, "header copy failed");
+        sz = h.size; path_len = h.path_len;
+    }
     switch (array_id) {
         case MCTSNC_ARR_TREES: return sz * (1 + A) * 4;
         case MCTSNC_ARR_DEPTHS: return sz * 2;
@@ -498,7 +796,7 @@ int64_t mctsnc_read_size(mctsnc_engine *e, int32_t array_id, int32_t tree) {
         case MCTSNC_ARR_NS: case MCTSNC_ARR_NS_WINS: return sz * 4;
         case MCTSNC_ARR_BOARDS: return sz * c.board_m * c.board_n;
         case MCTSNC_ARR_EXTRA_INFOS: return sz * c.extra_info_memory;
-        case MCTSNC_ARR_SELECTED_PATH: return (int64_t)h.path_len * 4;
+        case MCTSNC_ARR_SELECTED_PATH: return path_len * 4;
         case MCTSNC_ARR_ACTIONS_EXPANDED: return (A + 2) * 2;
         case MCTSNC_ARR_PLAYOUT_OUTCOMES: return 8;
         case MCTSNC_ARR_PLAYOUT_OUTCOMES_CHILDREN: return A * 8;
@@ -515,6 +813,7 @@ int mctsnc_read(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, siz
     const int A = c.max_actions, m = c.board_m, n = c.board_n, H = m + 1, E = c.extra_info_memory;
     if (array_id == MCTSNC_ARR_RNG_PLAYOUT) { HIP_TRY(hipMemcpy(dst, e->d_rng_playout, (size_t)need, hipMemcpyDeviceToHost)); return MCTSNC_OK; }
     if (array_id == MCTSNC_ARR_RNG_EXPAND) { if (need) HIP_TRY(hipMemcpy(dst, e->d_rng_expand, (size_t)need, hipMemcpyDeviceToHost)); return MCTSNC_OK; }
+    if (e->is_gomoku()) return read_gomoku(e, array_id, tree, dst, (size_t)need);
     c4::TreeHdr h;
     HIP_TRY(hipMemcpy(&h, e->d_hdrs + tree, sizeof h, hipMemcpyDeviceToHost));
     switch (array_id) {

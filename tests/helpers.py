@@ -103,3 +103,14 @@ def compare_with_oracle(e, o, board, fills, turn, steps):
     np.testing.assert_array_equal(e._actions_ns_wins, o.result("actions_ns_wins"))
     np.testing.assert_array_equal(e._actions_win_flags.astype(np.uint8), o.result("actions_win_flags"))
     np.testing.assert_array_equal(e.read_array("rng_playout"), o.rng_states("playout"))
+
+
+def random_gomoku_root(rng, m, n, stones):
+    """`stones` stones placed alternately on distinct random cells (no rule check: the engine, like the reference,
+    only tests lines through the last stone placed)."""
+    board = np.zeros((m, n), np.int8)
+    turn = 1
+    for c in rng.permutation(m * n)[:stones]:
+        board[c // n, c % n] = turn
+        turn = -turn
+    return board, turn

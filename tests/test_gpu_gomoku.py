@@ -1,0 +1,59 @@
+"""GPU parity of the Gomoku engine against the CPU oracle (the reference's Gomoku archives are missing from its
+checkout, so the oracle -- pinned on Connect 4 and, for the Gomoku rules, by brute-force checks -- is the only
+reference here: "oracle-pinned")."""
+import numpy as np
+import pytest
+
+from helpers import compare_with_oracle, make_engine, random_gomoku_root
+
+pytestmark = pytest.mark.gpu
+
+
+def engines(variant, T, P, m, n, seed=3, device_memory=0.5, **okw):
+    from oracle.oracle import Oracle
+    params = dict(n_trees=T, n_playouts=P, variant=variant, device_memory=device_memory, ucb_c=2.0, seed=seed)
+    e = make_engine(params, board_shape=(m, n), extra=0, actions=m * n, game="gomoku")
+    o = Oracle("gomoku", (m, n), 0, m * n, T, P, variant, ucb_c=2.0, seed=seed, device_memory=device_memory, threads=8, **okw)
+    return e, o
+
+
+@pytest.mark.parametrize("variant,T,P,steps", [("ocp_thrifty", 4, 128, 60), ("ocp_prodigal", 2, 64, 80),
+                                               ("acp_thrifty", 2, 64, 6), ("acp_prodigal", 1, 128, 5)])
+def test_gomoku_15x15_full_state(variant, T, P, steps):
+    """Two consecutive searches on 15x15 (random streams carried over): every per-node array, the step scratch,
+    the reduced root table and the generator states must equal the oracle's."""
+    rng = np.random.default_rng(11)
+    e, o = engines(variant, T, P, 15, 15)
+    for stones in (0, 12):
+        board, turn = random_gomoku_root(rng, 15, 15, stones)
+        compare_with_oracle(e, o, board, None, turn, steps)
+
+
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
+def test_gomoku_small_boards_deep_trees(variant):
+    """Small boards give deep trees, draws, terminal selections and, on 5x5, frequent exactly-five wins."""
+    rng = np.random.default_rng(12)
+    for (m, n), steps in (((6, 6), 250), ((5, 7), 150), ((8, 5), 100)):
+        e, o = engines(variant, 2, 64, m, n)
+        board, turn = random_gomoku_root(rng, m, n, 4)
+        compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else steps // 3)
+
+
+def test_gomoku_tree_full_path():
+    from mcts_numba_cuda_amd import MCTSNC
+    from oracle.oracle import Oracle
+    for variant in ("ocp_prodigal", "acp_thrifty"):
+        e = MCTSNC((6, 6), 0, 36, search_time_limit=np.inf, n_trees=2, n_playouts=64, variant=variant, seed=5, verbose_info=False, game="gomoku")
+        e.device_memory = float(2 * 194 * 80 + 2 * 8500)
+        e.init_device_side_arrays()
+        assert 40 < e.max_tree_size < 120
+        o = Oracle("gomoku", (6, 6), 0, 36, 2, 64, variant, seed=5, max_tree_size_override=e.max_tree_size, threads=4)
+        board, turn = random_gomoku_root(np.random.default_rng(1), 6, 6, 3)
+        compare_with_oracle(e, o, board, None, turn, 40)
+
+
+def test_gomoku_large_playout_count_runs_in_rounds():
+    """n_playouts = 512 exceeds the 256 threads of a workgroup; the playouts then run in two rounds."""
+    e, o = engines("ocp_thrifty", 1, 512, 15, 15)
+    board, turn = random_gomoku_root(np.random.default_rng(2), 15, 15, 8)
+    compare_with_oracle(e, o, board, None, turn, 12)
