@@ -1,4 +1,5 @@
-"""Builds libmctsnc_hip.so for gfx950 with hipcc (in-tree, next to this file)."""
+"""Builds libmctsnc_hip.so (search engine) and libpuct_hip.so (PUCT select/backup) for gfx950 with hipcc, in-tree,
+next to this file."""
 import os
 import subprocess
 import sys
@@ -6,7 +7,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmctsnc_hip.so")
-SOURCES = ["mctsnc_engine.hip"]
+PUCT_LIB = os.path.join(HERE, "libpuct_hip.so")
+LIBRARIES = {LIB: ["mctsnc_engine.hip"], PUCT_LIB: ["puct_kernels.hip"]}
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                # UCB values must be bit-reproducible: no fused multiply-add contraction anywhere
                "-ffp-contract=off",
@@ -14,9 +16,9 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                "-Wno-unknown-warning-option"]
 
 
-def build(verbose=False):
+def build_one(lib, sources, verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-o", lib] + [os.path.join(CSRC, s) for s in sources]
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -25,6 +27,14 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+    return lib
+
+
+def build(verbose=False, only=None):
+    """Compiles every library (or the one whose path is `only`); returns the search engine's path."""
+    for lib, sources in LIBRARIES.items():
+        if only is None or only == lib:
+            build_one(lib, sources, verbose)
     return LIB
 
 

@@ -19,8 +19,10 @@ MAX_TREE_DEPTH = 2048
 
 def build(force=False):
     """Compiles the oracle with gcc through its Makefile."""
-    if force and os.path.exists(_LIB_PATH):
-        os.remove(_LIB_PATH)
+    if force:
+        for path in (_LIB_PATH, os.path.join(_HERE, "libpuct_oracle.so")):
+            if os.path.exists(path):
+                os.remove(path)
     subprocess.check_call(["make", "-s", "-C", _HERE])
     return _LIB_PATH
 

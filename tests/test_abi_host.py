@@ -117,3 +117,23 @@ def test_replay_helpers_reconstruct_positions(archives):
             pos.play(ev["action"])
     from helpers import c4_has_four
     assert game["outcome"] == "WHITE WINS" and c4_has_four(pos.board, -1) and not c4_has_four(pos.board, 1)
+
+
+def test_puct_library_exports_every_declared_symbol(tmp_path):
+    """libpuct_hip.so loads without a GPU and exports what include/puct_select.h declares, including the two symbols
+    the reference's binding resolves by name (src/puct/puct_gpu_v3_cpp.py:88-113); the header is valid C."""
+    from mcts_numba_cuda_amd import build, puct
+    if not os.path.exists(puct.LIB_PATH):
+        build.build(only=build.PUCT_LIB)
+    lib = puct._lib()
+    header = os.path.join(ROOT, "include", "puct_select.h")
+    text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(puct_[a-z_]+)\s*\(", text)))
+    assert {"puct_select_winner_recalc_launch", "puct_cpp_cuda_error_string", "puct_edge_backup_launch",
+            "puct_node_backup_launch"} == set(names)
+    for name in names:
+        assert hasattr(lib, name), name
+    src = tmp_path / "probe.c"
+    src.write_text(f'#include "{header}"\nint main(void) {{ return PUCT_SELECT_BUSY == 4 ? 0 : 1; }}\n')
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-c", "-o", str(tmp_path / "probe.o"), str(src)])
+    assert (puct.PACKED_KIND_SHIFT, puct.PACKED_SLOT_SHIFT, puct.PACKED_REASON_SHIFT) == (22, 14, 25)
