@@ -31,8 +31,9 @@ M, N, A = 6, 7, 7
 T, P, STEPS, DEVICE_MEMORY = 4, 256, 5000, 2.0
 N_ROOTS = 64
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per search-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or None until measured
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per search-kernel launch from rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy gives) and WRITE_SIZE
+# (x1), averaged over the first four roots: (5044.8 * 2 + 23530.4) KiB
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 34427000
 
 
 def has_four(board, token):
@@ -98,10 +99,23 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-batched", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
+                         "WRITE_SIZE readings are scaled by) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (trees are independent and would shard over GPUs with one "
                  "final all-reduce of the root table, but no multi-GPU path is part of it); run with --gpus 1")
+
+    if args.copy_calibration:
+        import torch
+        src = torch.arange(1 << 28, dtype=torch.int32, device="cuda")   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "copies": 4}))
+        return
 
     import contextlib
     import io
@@ -165,7 +179,10 @@ def main():
                 n_searches = (min(args.steps, len(roots)) // nb) * nb
                 batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": n_searches / bt,
                            "mcts_steps_per_s_all_roots": n_searches * STEPS / bt}
+            for e in engines[1:]:
+                e._release()
             del engines
+        eng._release()      # free the pools now rather than at interpreter exit, after the HIP runtime has shut down
 
     value = playouts / elapsed
     launches = args.steps  # one search kernel launch per search at a fixed step budget
@@ -176,7 +193,7 @@ def main():
                 "avg_launch_ms": dev_time / launches * 1e3,
                 "stage_bytes_per_launch": {k: v / launches for k, v in alg.items() if k != "total"},
                 "playout_plies_per_s": plies / dev_time,
-                "note": "latency-bound pointer chasing plus integer playouts on 28 workgroups: a few KB of tree data per step; see DESIGN.md"}
+                "note": "latency-bound pointer chasing plus integer playouts on 28 workgroups: a few KB of tree data per step"}
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
