@@ -164,21 +164,22 @@ def main():
 
         batched = None
         if not args.no_batched:
-            nb = 16
+            # the same 64 searches, all handed to the device at once (the engine runs them in as few fully resident
+            # groups as the device allows); results are identical to the sequential runs
+            nb = min(len(roots), max(args.steps, 1))
             engines = [eng] + [new_engine() for _ in range(nb - 1)]
-            bt, bp = 0.0, 0
-            for start in range(0, min(args.steps, len(roots)) - nb + 1, nb):
-                chunk = roots[start:start + nb]
+            chunk = roots[:nb]
+            for rep in range(2):    # first pass warms the pools up
                 for e in engines:
                     e.reseed()
                 t1 = time.perf_counter()
                 run_batch(engines, [c[0] for c in chunk], [c[1] for c in chunk], [c[2] for c in chunk])
-                bt += time.perf_counter() - t1
-                bp += sum(e.performance_info["playouts"] for e in engines)
-            if bt > 0:
-                n_searches = (min(args.steps, len(roots)) // nb) * nb
-                batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": n_searches / bt,
-                           "mcts_steps_per_s_all_roots": n_searches * STEPS / bt}
+                bt = time.perf_counter() - t1
+            bp = sum(e.performance_info["playouts"] for e in engines)
+            bbytes = sum(algorithmic_bytes(e._result, e.steps * T)["total"] for e in engines)
+            batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": nb / bt,
+                       "mcts_steps_per_s_all_roots": nb * STEPS / bt, "ms_per_pass": bt * 1e3,
+                       "algorithmic_GB_per_s": bbytes / bt / 1e9, "hbm_frac": bbytes / bt / 1e9 / HBM_PEAK_GBS}
             for e in engines[1:]:
                 e._release()
             del engines

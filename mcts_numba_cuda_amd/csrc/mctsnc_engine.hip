@@ -546,9 +546,36 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
              const Budget &bud, mctsnc_result *out) {
     int rc = check_batch(engines, n, turns);
     if (rc) return rc;
-    HIP_TRY(hipSetDevice(engines[0]->cfg.device));
-    if (engines[0]->is_gomoku()) return run_many_gomoku(engines, n, boards, turns, bud, out);
-    return run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out);
+    mctsnc_engine *e0 = engines[0];
+    const mctsnc_config &c = e0->cfg;
+    HIP_TRY(hipSetDevice(c.device));
+    // The all-children-playouts kernels synchronise workgroups of one tree with each other, so a launch must be fully
+    // resident: a batch whose grid exceeds what the device holds at once runs as consecutive groups of searches, each
+    // with the whole budget.
+    int group = n;
+    if (e0->acp && n > 1) {
+        int per_cu = 0, cus = 0;
+        if (e0->is_gomoku())
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
+                                                                 gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
+        else
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, 0));
+        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
+        const int64_t max_refs = (int64_t)per_cu * cus / (8 * e0->G) * 8;   // the grid is 8 * G * ceil(refs / 8) workgroups
+        group = (int)std::max<int64_t>(1, std::min<int64_t>(n, max_refs / c.n_trees));
+    }
+    const size_t cells = (size_t)c.board_m * c.board_n;
+    for (int start = 0; start < n; start += group) {
+        const int k = std::min(group, n - start);
+        const int8_t *b = boards + (size_t)start * cells;
+        if (e0->is_gomoku())
+            rc = run_many_gomoku(engines + start, k, b, turns + start, bud, out + start);
+        else
+            rc = run_many_c4(engines + start, k, b, extras ? extras + (size_t)start * extra_len : nullptr, extra_len, turns + start, bud,
+                             out + start);
+        if (rc) return rc;
+    }
+    return MCTSNC_OK;
 }
 
 int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t need) {

@@ -105,6 +105,25 @@ def test_run_batch_equals_single_runs():
             np.testing.assert_array_equal(eb.read_array("rng_playout"), es.read_array("rng_playout"))
 
 
+def test_run_batch_larger_than_the_device_runs_in_groups():
+    """A batch whose workgroups cannot all be resident at once (48 searches x 4 trees x 7 columns = 1344 workgroups of
+    256 threads) is split into consecutive groups; every search still ends exactly where a separate run ends."""
+    from mcts_numba_cuda_amd import run_batch
+    rng = np.random.default_rng(17)
+    params = dict(n_trees=4, n_playouts=256, variant="acp_thrifty", device_memory=0.02, ucb_c=2.0, seed=3)
+    roots = [random_c4_root(rng, int(rng.integers(0, 24))) for _ in range(48)]
+    batch = [make_engine(params) for _ in roots]
+    run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=120)
+    single = make_engine(params)
+    for k in (0, 7, 31, 32, 33, 47):
+        single.reseed()
+        single.run(*roots[k], forced_search_steps_limit=120)
+        assert batch[k].actions_info == single.actions_info
+        for ti in range(4):
+            for name in ("trees", "ns", "ns_wins"):
+                np.testing.assert_array_equal(batch[k].read_array(name, ti), single.read_array(name, ti))
+
+
 def test_time_limited_run_and_chunking():
     """A time budget is honoured within a few percent and splitting a search over several kernel launches changes
     nothing: the same number of steps in one launch gives the identical tree."""
