@@ -1,0 +1,100 @@
+/*
+ * C ABI of the Gomoku PUCT search loop with virtual loss (part of libpuct_hip.so, gfx950).
+ *
+ * The reference has no such loop: its PUCT kernels stop at selection (src/puct/puct_gpu_v3_cpp.cu:277-448) and backup
+ * (src/puct/puct_gpu_v2.py:847-927) on synthetic trees.  This engine puts the step between them — committing the
+ * claimed expansion slot, creating the child position, evaluating it — around those two kernels, for Gomoku with the
+ * rules of the reference's game plugin (five in a row exactly, src/mctsnc_game_mechanics.py:181-280), a synthetic
+ * evaluator (Dirichlet priors over the legal cells and a value, both pure functions of the position) and the
+ * reference's array layout and sizes (src/puct/puct_gpu_v2.py:69-103: [trees, nodes, edges] arrays, nodes <= 16384,
+ * edges <= 256).
+ *
+ * One step = every tree runs `traversals` selections at once (one 64-lane wavefront each, virtual loss between
+ * them), then expands / evaluates the selected leaves, then backs the values up.  All steps of a search run inside one
+ * kernel launch, one workgroup per tree.
+ *
+ * All functions return 0 on success or a negative error code; puct_gomoku_last_error() describes the last failure
+ * of the calling thread.  Host pointers only; the engine owns its device memory.
+ */
+#ifndef PUCT_GOMOKU_H
+#define PUCT_GOMOKU_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PUCT_GOMOKU_OK 0
+#define PUCT_GOMOKU_E_INVALID (-1)
+#define PUCT_GOMOKU_E_HIP (-2)
+#define PUCT_GOMOKU_E_ROOT (-3)
+
+typedef struct {
+    int32_t board_m, board_n;  /* rows, columns; m * n <= 256 */
+    int32_t trees;             /* independent trees on the same root, each with its own synthetic evaluator */
+    int32_t traversals;        /* concurrent selections per tree and step, 1..16 */
+    int32_t max_nodes;         /* node capacity per tree, 2..16384 */
+    int32_t path_depth;        /* longest path a selection may take, 1..1024 */
+    float cpuct, c_pw, alpha_pw;
+    int32_t soft_winner;
+    float dirichlet_alpha;     /* in (0, 1) */
+    uint64_t seed;
+    int32_t device;
+} puct_gomoku_config;
+
+typedef struct {
+    int64_t steps;
+    int32_t best_action;             /* cell with the most root visits over all trees (smallest index on ties), -1 if none */
+    int64_t best_n;
+    int64_t root_n[256];             /* visits per cell, summed over trees */
+    double root_w[256];              /* value sums per cell (for the player to move at the root), summed over trees */
+    int64_t selections[5];           /* per kind: invalid, expand, terminal, depth limit, busy */
+    int64_t expansions_committed;    /* children created */
+    int64_t nodes_total;             /* nodes over all trees after the search */
+    int32_t max_nodes_in_tree;
+    double time_total, time_device;  /* seconds */
+} puct_gomoku_result;
+
+typedef struct puct_gomoku_engine puct_gomoku_engine;
+
+int puct_gomoku_create(const puct_gomoku_config *config, puct_gomoku_engine **out);
+void puct_gomoku_destroy(puct_gomoku_engine *engine);
+
+/* Searches from `board` (int8 [m, n]: 0 empty, +1 / -1 stones) with `turn` (+1 / -1) to move for `steps` steps.
+ * fused != 0: one kernel launch for the whole search; fused == 0: three launches per step (the selection of
+ * puct_select_winner_recalc_launch, expansion / evaluation, the backup of puct_edge_backup_launch) — same results
+ * whenever the selections of a step do not race (traversals == 1).  Selection differs from the plain launcher in one
+ * point: progressive widening is capped by the node's number of empty cells instead of by the edge dimension, so a
+ * fully expanded node is descended through rather than asked for another slot. */
+int puct_gomoku_run(puct_gomoku_engine *engine, const int8_t *board, int32_t turn, int32_t steps, int32_t fused,
+                    puct_gomoku_result *result);
+
+/* Copies one device array of the last search to the host.  Shapes (T trees, N = max_nodes, E = 256, W traversals,
+ * D = path_depth): see the ids below.  `bytes` must equal the array's size. */
+#define PUCT_GOMOKU_ARR_EDGE_CHILD 0       /* int32 [T, N, E] */
+#define PUCT_GOMOKU_ARR_EDGE_PRIOR 1       /* float32 [T, N, E] */
+#define PUCT_GOMOKU_ARR_EDGE_W 2           /* float32 [T, N, E] */
+#define PUCT_GOMOKU_ARR_EDGE_N 3           /* int32 [T, N, E] */
+#define PUCT_GOMOKU_ARR_EDGE_INFLIGHT 4    /* int32 [T, N, E] */
+#define PUCT_GOMOKU_ARR_EDGE_ACTION 5      /* uint8 [T, N, E] */
+#define PUCT_GOMOKU_ARR_NODE_EXPANDED 6    /* int32 [T, N] */
+#define PUCT_GOMOKU_ARR_NODE_EXPAND_INFLIGHT 7 /* int32 [T, N] */
+#define PUCT_GOMOKU_ARR_NODE_COUNT 8       /* int32 [T] */
+#define PUCT_GOMOKU_ARR_NODE_BOARD 9       /* uint32 [T, N, 16]: words 0..7 stones of +1, 8..15 stones of -1 */
+#define PUCT_GOMOKU_ARR_NODE_TURN 10       /* int8 [T, N] */
+#define PUCT_GOMOKU_ARR_NODE_VALUE 11      /* float32 [T, N]: value of a terminal node for its player to move */
+#define PUCT_GOMOKU_ARR_OUT_SELECTED 12    /* int32 [T, W]: last step */
+#define PUCT_GOMOKU_ARR_OUT_PATH 13        /* int32 [T, W, D]: last step */
+#define PUCT_GOMOKU_ARR_OUT_LEN 14         /* int32 [T, W]: last step */
+#define PUCT_GOMOKU_ARR_PATH_VALUES 15     /* float32 [T, W, D]: last step */
+#define PUCT_GOMOKU_ARR_NODE_LEGAL 16      /* int32 [T, N]: empty cells of the node's position = most children it can have */
+int64_t puct_gomoku_array_bytes(puct_gomoku_engine *engine, int32_t array_id);
+int puct_gomoku_read(puct_gomoku_engine *engine, int32_t array_id, void *dst, size_t bytes);
+
+const char *puct_gomoku_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmctsnc_hip.so")
 PUCT_LIB = os.path.join(HERE, "libpuct_hip.so")
-LIBRARIES = {LIB: ["mctsnc_engine.hip"], PUCT_LIB: ["puct_kernels.hip"]}
+LIBRARIES = {LIB: ["mctsnc_engine.hip"], PUCT_LIB: ["puct_kernels.hip", "puct_gomoku.hip"]}
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                # UCB values must be bit-reproducible: no fused multiply-add contraction anywhere
                "-ffp-contract=off",

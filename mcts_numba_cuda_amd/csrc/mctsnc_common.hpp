@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "det_math.h"
+
 namespace mctsnc {
 
 constexpr int kWave = 64;
@@ -33,48 +35,7 @@ __host__ __device__ __forceinline__ float rng_uniform(uint64_t &s0, uint64_t &s1
 // x = 2^k (1 + f), s = f / (2 + f), log(1 + f) = f - hfsq + s (hfsq + R(s^2)); error below 1 ulp.
 // Valid for positive normal x (the callers pass visit counts >= 1).
 // ------------------------------------------------------------------------------------------------
-__host__ __device__ inline double det_log(double x) {
-    const double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10;
-    const double Lg1 = 6.666666666666735130e-01, Lg2 = 3.999999999940941908e-01, Lg3 = 2.857142874366239149e-01,
-                 Lg4 = 2.222219843214978396e-01, Lg5 = 1.818357216161805012e-01, Lg6 = 1.531383769920937332e-01,
-                 Lg7 = 1.479819860511658591e-01;
-    union { double d; uint64_t u; } v;
-    v.d = x;
-    int32_t hx = (int32_t)(v.u >> 32);
-    const uint32_t lx = (uint32_t)v.u;
-    int32_t k = (hx >> 20) - 1023;
-    hx &= 0x000fffff;
-    int32_t i = (hx + 0x95f64) & 0x100000;
-    v.u = ((uint64_t)(uint32_t)(hx | (i ^ 0x3ff00000)) << 32) | lx;  // normalise x or x/2
-    k += (i >> 20);
-    const double f = v.d - 1.0;
-    const double dk = (double)k;
-    if ((0x000fffff & (2 + hx)) < 3) {  // |f| < 2^-20
-        if (f == 0.0) {
-            if (k == 0) return 0.0;
-            return dk * ln2_hi + dk * ln2_lo;
-        }
-        const double R = f * f * (0.5 - 0.33333333333333333 * f);
-        if (k == 0) return f - R;
-        return dk * ln2_hi - ((R - dk * ln2_lo) - f);
-    }
-    const double s = f / (2.0 + f);
-    const double z = s * s;
-    i = hx - 0x6147a;
-    const double w = z * z;
-    const int32_t j = 0x6b851 - hx;
-    const double t1 = w * (Lg2 + w * (Lg4 + w * Lg6));
-    const double t2 = z * (Lg1 + w * (Lg3 + w * (Lg5 + w * Lg7)));
-    i |= j;
-    const double R = t2 + t1;
-    if (i > 0) {
-        const double hfsq = 0.5 * f * f;
-        if (k == 0) return f - (hfsq - s * (hfsq + R));
-        return dk * ln2_hi - ((hfsq - (s * (hfsq + R) + dk * ln2_lo)) - f);
-    }
-    if (k == 0) return f - s * (f - R);
-    return dk * ln2_hi - ((s * (f - R) - dk * ln2_lo) - f);
-}
+__host__ __device__ inline double det_log(double x) { return detm_log(x); }
 
 #ifdef __HIPCC__
 // float32((x >> 11) * 2^-53) for x = hi * 2^32 + lo, without double arithmetic.  The 11 discarded bits are

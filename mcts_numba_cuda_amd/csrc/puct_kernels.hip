@@ -1,378 +1,20 @@
-// PUCT selection and backup with virtual loss for gfx950 (wave64): one 64-lane wavefront per traversal.
-//
-// Semantics follow src/puct/puct_gpu_v3_cpp.cu:38-448 (selection) and src/puct/puct_gpu_v2.py:847-927 (backup); the
-// wavefront-level organisation is this library's own:
-//   * the first 64 edges of a node (all of them for almost every node under progressive widening) are loaded once,
-//     together with the node's own words, before anything about the node is known, so a level costs one round of
-//     loads and one claim instead of a chain of dependent loads;
-//   * the reference's total order on edges (score descending, rotated edge index ascending) is folded into one 64-bit
-//     key, so the arg-max is a single max-reduction over DPP row operations and four lane reads.
-#include <hip/hip_runtime.h>
-#include <float.h>
-#include <stdint.h>
-
-#include "../../include/puct_select.h"
+// Kernels and C ABI of PUCT selection and backup with virtual loss (device code: puct_device.hpp).
+#include "puct_device.hpp"
 
 namespace {
-
-constexpr int kWave = 64;
-constexpr int kMaxWavesPerBlock = 16;
-constexpr int kRecalcAttempts = 2;  // MAX_RECALC_RETRY, src/puct/puct_gpu_v3_cpp.cu:36
-constexpr int kNoEdge = 0x7fffffff;
-
-struct SelectArgs {
-    float cpuct, c_pw, alpha_pw;
-    int soft_winner;
-    const int *edge_child_id;
-    const float *edge_prior;
-    const float *edge_W;
-    const int *edge_N;
-    int *edge_inflight;
-    int *node_expand_inflight;
-    const int *node_expanded;
-    const int *tree_nodes;
-    int *out_selected_node;
-    int *out_path_eids;
-    int *out_path_len;
-    int trees, nodes, edges, warps, path_depth;
-};
-
-// ---- cross-lane reductions -------------------------------------------------------------------------------------
-// DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror.  After the four steps every
-// lane holds the reduction of its 16-lane row; the four rows are combined through lane reads.
-template <int CTRL>
-__device__ __forceinline__ int dpp(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
-}
-
-__device__ __forceinline__ int wave_sum(int v) {
-    v += dpp<0xB1>(v);
-    v += dpp<0x4E>(v);
-    v += dpp<0x141>(v);
-    v += dpp<0x140>(v);
-    return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
-           __builtin_amdgcn_readlane(v, 48);
-}
-
-template <int CTRL>
-__device__ __forceinline__ uint64_t dpp_max64(uint64_t v) {
-    const uint32_t lo = (uint32_t)dpp<CTRL>((int)(uint32_t)v);
-    const uint32_t hi = (uint32_t)dpp<CTRL>((int)(uint32_t)(v >> 32));
-    const uint64_t o = ((uint64_t)hi << 32) | lo;
-    return o > v ? o : v;
-}
-
-__device__ __forceinline__ uint64_t read_lane64(uint64_t v, int lane) {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, lane);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), lane);
-    return ((uint64_t)hi << 32) | lo;
-}
-
-__device__ __forceinline__ uint64_t wave_max(uint64_t v) {
-    v = dpp_max64<0xB1>(v);
-    v = dpp_max64<0x4E>(v);
-    v = dpp_max64<0x141>(v);
-    v = dpp_max64<0x140>(v);
-    const uint64_t a = read_lane64(v, 0), b = read_lane64(v, 16), c = read_lane64(v, 32), d = read_lane64(v, 48);
-    const uint64_t ab = a > b ? a : b, cd = c > d ? c : d;
-    return ab > cd ? ab : cd;
-}
-
-__device__ __forceinline__ int load_relaxed(const int *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// ---- selection ---------------------------------------------------------------------------------------------------
-__device__ __forceinline__ int pack_selection(int kind, int node, int slot, int reason) {
-    return (reason << PUCT_PACKED_REASON_SHIFT) | (kind << PUCT_PACKED_KIND_SHIFT) | (slot << PUCT_PACKED_SLOT_SHIFT) |
-           node;
-}
-
-// src/puct/puct_gpu_v3_cpp.cu:43-49
-__device__ __forceinline__ bool valid_select_shape(int path_depth, int nodes, int node_cnt, int edges) {
-    return path_depth >= 1 && nodes > 0 && node_cnt > 0 && node_cnt <= nodes && node_cnt <= PUCT_PACKED_NODE_LIMIT &&
-           edges > 0 && edges <= PUCT_PACKED_EDGE_MASK + 1;
-}
-
-// Progressive widening, src/puct/puct_gpu_v3_cpp.cu:150-157.
-__device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int n_node, int edges) {
-    const float val = (alpha_pw == 0.5f) ? c_pw * sqrtf((float)n_node) : c_pw * powf((float)n_node, alpha_pw);
-    if (val >= (float)edges) return edges;
-    const int allowed = (int)ceilf(val);
-    return allowed > 1 ? allowed : 1;
-}
-
-// src/puct/puct_gpu_v3_cpp.cu:171-180
-__device__ __forceinline__ float puct_score(float cpuct, float prior, float w, int n, int inflight, float sqrt_parent) {
-    const float q = n > 0 ? w / (float)n : 0.0f;
-    const float u = cpuct * prior * sqrt_parent / (float)(n + inflight + 1);
-    return q + u;
-}
-
-// One 64-bit key per candidate edge whose unsigned order is the reference's order "higher score first, then smaller
-// rotated edge index" (src/puct/puct_gpu_v3_cpp.cu:51-71).  0 means "not a candidate": the reference starts from
-// (-FLT_MAX, no edge) and accepts a score that is greater than or equal to it, so NaN and -inf never win.  -0.0f is
-// made +0.0f because the reference compares floats, for which the two are equal.
-__device__ __forceinline__ uint64_t candidate_key(float score, int eid, int tie_offset, int span) {
-    if (!(score >= -FLT_MAX)) return 0;
-    const uint32_t b = __float_as_uint(score + 0.0f);
-    const uint32_t ordered = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-    int key = eid - tie_offset;
-    if (key < 0) key += span;
-    return ((uint64_t)ordered << 32) | ((uint32_t)(0xFFFF - key) << 16) | (uint32_t)eid;
-}
-
-// Takes back the virtual loss of the first `depth` path entries (src/puct/puct_gpu_v3_cpp.cu:206-217).  The entries
-// were stored by lane 0 of this wavefront; the fence completes those stores before other lanes read them back.
-__device__ __forceinline__ void rollback_path(const SelectArgs &a, const int *path, int tree, int depth, int lane,
-                                              int node_cnt) {
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
-    for (int d = lane; d < depth; d += kWave) {
-        const int encoded = load_relaxed(path + d);
-        const int parent = encoded >> 8, slot = encoded & 0xFF;
-        if (parent >= 0 && parent < node_cnt && slot < a.edges)
-            atomicSub(&a.edge_inflight[((size_t)tree * a.nodes + parent) * a.edges + slot], 1);
-    }
-}
+using namespace puct;
 
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_kernel(const SelectArgs a) {
-    const int tree = blockIdx.x;
-    const int lane = threadIdx.x & (kWave - 1);
     const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (wid >= a.warps) return;
-
-    const size_t out = (size_t)tree * a.warps + wid;
-    int *path = a.out_path_eids + out * a.path_depth;
-    const int node_cnt = a.tree_nodes[tree];
-    const int nodes = a.nodes, edges = a.edges;
-
-    int final_packed = pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_UNKNOWN);
-    int final_len = 0;
-
-    if (!valid_select_shape(a.path_depth, nodes, node_cnt, edges)) {
-        final_packed = pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_SHAPE);
-    } else {
-        int node = 0, depth = 0;
-        while (true) {
-            const size_t nrow = (size_t)tree * nodes + node;
-            const size_t erow = nrow * edges;
-
-            // Everything a level can need from the first 64 edges, requested in one go.
-            int n0 = 0, f0 = 0, c0 = -1;
-            float p0 = 0.0f, w0 = 0.0f;
-            if (lane < edges) {
-                n0 = a.edge_N[erow + lane];
-                f0 = load_relaxed(a.edge_inflight + erow + lane);
-                p0 = a.edge_prior[erow + lane];
-                w0 = a.edge_W[erow + lane];
-                c0 = a.edge_child_id[erow + lane];
-            }
-            const int node_info = a.node_expanded[nrow];
-            const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
-
-            if (node_info == PUCT_NODE_EXPANDED_TERMINAL) {
-                final_packed = pack_selection(PUCT_SELECT_TERMINAL, node, 0, PUCT_REASON_OK_TERMINAL);
-                final_len = depth + 1;
-                break;
-            }
-            if (node_info < 0 || node_info > edges) {
-                rollback_path(a, path, tree, depth, lane, node_cnt);
-                final_packed =
-                    pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NODE_INFO);
-                break;
-            }
-            if (depth >= a.path_depth) {
-                final_packed = pack_selection(PUCT_SELECT_DEPTH_LIMIT, node, 0, PUCT_REASON_OK_DEPTH_LIMIT);
-                final_len = depth + 1;
-                break;
-            }
-
-            const int cur_expanded = node_info;
-            int parent_eff = 1, allowed = 1;
-            if (cur_expanded != 1 || a.c_pw != 0.0f) {
-                int total = lane < cur_expanded ? n0 + f0 : 0;
-                for (int eid = lane + kWave; eid < cur_expanded; eid += kWave)
-                    total += a.edge_N[erow + eid] + load_relaxed(a.edge_inflight + erow + eid);
-                total = wave_sum(total);
-                parent_eff = total > 1 ? total : 1;
-                allowed = allowed_children(a.c_pw, a.alpha_pw, parent_eff, edges);
-            }
-
-            if (allowed > cur_expanded) {
-                // Expansion ticket, src/puct/puct_gpu_v3_cpp.cu:219-233.
-                int expand_slot = -1;
-                if (cur_expanded + expand_inflight < allowed) {
-                    if (lane == 0) {
-                        const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
-                        if (slot < allowed)
-                            expand_slot = slot;
-                        else
-                            atomicSub(&a.node_expand_inflight[nrow], 1);
-                    }
-                    expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
-                }
-                if (expand_slot >= 0) {
-                    final_packed = pack_selection(PUCT_SELECT_EXPAND, node, expand_slot, PUCT_REASON_OK_EXPAND);
-                    final_len = depth + 1;
-                    break;
-                }
-                if (cur_expanded == 0) {
-                    rollback_path(a, path, tree, depth, lane, node_cnt);
-                    final_packed = pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_EXPAND_INFLIGHT);
-                    break;
-                }
-            }
-
-            int tie_offset = wid;
-            if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
-
-            int best_eid = 0, held = 0;
-            if (cur_expanded == 1) {
-                if (lane == 0) atomicAdd(&a.edge_inflight[erow], 1);
-                held = 1;
-            } else {
-                // Winner-recalc claim, src/puct/puct_gpu_v3_cpp.cu:235-275: score all edges, try to move the winner's
-                // in-flight count from the value the score was computed with to that value plus one, rescore once if
-                // another traversal got there first.
-                const float sqrt_parent = sqrtf((float)parent_eff);
-                best_eid = kNoEdge;
-                for (int attempt = 0; attempt < kRecalcAttempts; ++attempt) {
-                    uint64_t key = 0;
-                    int my_inflight = 0;
-                    if (lane < cur_expanded) {
-                        my_inflight = attempt == 0 ? f0 : load_relaxed(a.edge_inflight + erow + lane);
-                        key = candidate_key(puct_score(a.cpuct, p0, w0, n0, my_inflight, sqrt_parent), lane,
-                                            tie_offset, cur_expanded);
-                    }
-                    for (int eid = lane + kWave; eid < cur_expanded; eid += kWave) {
-                        const int f = load_relaxed(a.edge_inflight + erow + eid);
-                        const uint64_t k = candidate_key(
-                            puct_score(a.cpuct, a.edge_prior[erow + eid], a.edge_W[erow + eid], a.edge_N[erow + eid], f,
-                                       sqrt_parent),
-                            eid, tie_offset, cur_expanded);
-                        if (k > key) {
-                            key = k;
-                            my_inflight = f;
-                        }
-                    }
-                    const uint64_t best = wave_max(key);
-                    if (best == 0) {
-                        best_eid = kNoEdge;
-                        break;
-                    }
-                    best_eid = (int)(best & 0xFFFFu);
-                    const int best_inflight = __builtin_amdgcn_readlane(my_inflight, best_eid & (kWave - 1));
-                    int got = 0;
-                    if (lane == 0) {
-                        const int prev = atomicCAS(&a.edge_inflight[erow + best_eid], best_inflight, best_inflight + 1);
-                        got = prev == best_inflight ? 1 : 0;
-                    }
-                    held = __builtin_amdgcn_readfirstlane(got);
-                    if (held) break;
-                }
-                if (a.soft_winner != 0 && held == 0 && best_eid != kNoEdge) {
-                    if (lane == 0) atomicAdd(&a.edge_inflight[erow + best_eid], 1);
-                    held = 1;
-                }
-            }
-
-            if (held == 0) {
-                rollback_path(a, path, tree, depth, lane, node_cnt);
-                final_packed =
-                    best_eid == kNoEdge
-                        ? pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NO_VALID_EDGE)
-                        : pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_WINNER_RECALC);
-                break;
-            }
-
-            const int best_child =
-                best_eid < kWave ? __builtin_amdgcn_readlane(c0, best_eid) : a.edge_child_id[erow + best_eid];
-            if (best_child < 0 || best_child >= node_cnt) {
-                if (lane == 0) atomicSub(&a.edge_inflight[erow + best_eid], 1);
-                rollback_path(a, path, tree, depth, lane, node_cnt);
-                final_packed =
-                    pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_CHILD_OOB);
-                break;
-            }
-
-            if (lane == 0) path[depth] = (node << 8) | best_eid;
-            node = best_child;
-            depth += 1;
-        }
-    }
-
-    if (lane == 0) {
-        a.out_selected_node[out] = final_packed;
-        a.out_path_len[out] = final_len;
-    }
+    select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
-// ---- backup --------------------------------------------------------------------------------------------------------
-struct BackupArgs {
-    int virtual_loss;
-    const int *edge_child_id;
-    float *edge_W;
-    int *edge_N;
-    int *edge_inflight;
-    int *node_inflight;
-    int *node_expand_inflight;
-    const int *node_count;
-    const int *out_selected_node;
-    const int *out_path_eids;
-    const int *out_path_len;
-    const float *path_edge_values;
-    int trees, nodes, edges, warps, path_depth;
-};
-
-// NODE_LEVEL = true: src/puct/puct_gpu_v2.py:847-927 as written (virtual loss lives in node_inflight[child], the
-// selection word has no reason field).  NODE_LEVEL = false: the same conversion of virtual visits into real ones for
-// the edge-level virtual loss of select_kernel; BUSY selections hold nothing and are skipped, as in
-// src/puct/test_puct_gpu_v3.py:297-302.
 template <bool NODE_LEVEL>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_kernel(const BackupArgs a) {
-    const int tree = blockIdx.x;
-    const int lane = threadIdx.x & (kWave - 1);
     const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (wid >= a.warps) return;
-
-    const int node_limit = a.node_count[tree];
-    if (node_limit <= 0 || node_limit > a.nodes || node_limit > PUCT_PACKED_NODE_LIMIT) return;
-
-    const size_t out = (size_t)tree * a.warps + wid;
-    const int raw = a.out_selected_node[out];
-    if (raw < 0) return;
-    const int kind = NODE_LEVEL ? raw >> PUCT_PACKED_KIND_SHIFT : (raw >> PUCT_PACKED_KIND_SHIFT) & PUCT_PACKED_KIND_MASK;
-    if (kind == PUCT_SELECT_INVALID) return;
-    if (!NODE_LEVEL && kind == PUCT_SELECT_BUSY) return;
-    const int plen = a.out_path_len[out];
-    if (plen <= 0) return;
-
-    int edge_count = plen - 1;
-    if (edge_count > a.path_depth) edge_count = a.path_depth;
-    const int *path = a.out_path_eids + out * a.path_depth;
-    for (int d = lane; d < edge_count; d += kWave) {
-        const int encoded = path[d];
-        if (encoded < 0) continue;
-        const int parent = encoded >> 8, slot = encoded & 0xFF;
-        if (parent >= node_limit || slot >= a.edges) continue;
-        const size_t e = ((size_t)tree * a.nodes + parent) * a.edges + slot;
-        if (NODE_LEVEL) {
-            const int child = a.edge_child_id[e];
-            if (child >= 0 && child < node_limit)
-                atomicSub(&a.node_inflight[(size_t)tree * a.nodes + child], a.virtual_loss);
-        } else {
-            atomicSub(&a.edge_inflight[e], a.virtual_loss);
-        }
-        if (a.path_edge_values != nullptr) {
-            atomicAdd(&a.edge_N[e], 1);
-            unsafeAtomicAdd(&a.edge_W[e], a.path_edge_values[out * a.path_depth + d]);
-        }
-    }
-
-    if (lane == 0 && kind == PUCT_SELECT_EXPAND) {
-        const int leaf = raw & PUCT_PACKED_NODE_MASK;
-        if (leaf < node_limit) atomicSub(&a.node_expand_inflight[(size_t)tree * a.nodes + leaf], 1);
-    }
+    backup_traversal<NODE_LEVEL>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
 // One wavefront per traversal; a tree with more than 16 traversals is spread over several workgroups.

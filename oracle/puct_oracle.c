@@ -72,7 +72,8 @@ static void rollback(int *edge_inflight, const int *path, int depth, size_t tree
 static void select_one(float cpuct, float c_pw, float alpha_pw, int soft_winner, const int *edge_child_id,
                        const float *edge_prior, const float *edge_W, const int *edge_N, int *edge_inflight,
                        int *node_expand_inflight, const int *node_expanded, int node_cnt, int *out_selected,
-                       int *path, int *out_len, int tree, int wid, int nodes, int edges, int path_depth) {
+                       int *path, int *out_len, int tree, int wid, int nodes, int edges, int path_depth,
+                       const int *node_capacity) {
     (void)soft_winner; /* a sequential claim never loses its compare-and-swap, so the soft fallback cannot trigger */
     *out_selected = pack(K_INVALID, NODE_MASK, 0, R_UNSET);
     *out_len = 0;
@@ -107,7 +108,7 @@ static void select_one(float cpuct, float c_pw, float alpha_pw, int soft_winner,
             int total = 0;
             for (int e = 0; e < expanded; ++e) total += edge_N[erow + e] + edge_inflight[erow + e];
             parent_eff = total > 1 ? total : 1;
-            allowed = allowed_children(c_pw, alpha_pw, parent_eff, edges);
+            allowed = allowed_children(c_pw, alpha_pw, parent_eff, node_capacity ? node_capacity[nrow] : edges);
         }
         if (allowed > expanded) {
             int slot = -1;
@@ -172,17 +173,29 @@ static void select_one(float cpuct, float c_pw, float alpha_pw, int soft_winner,
     *out_len = len;
 }
 
-void po_select(float cpuct, float c_pw, float alpha_pw, int soft_winner, const int *edge_child_id,
-               const float *edge_prior, const float *edge_W, const int *edge_N, int *edge_inflight,
-               int *node_expand_inflight, const int *node_expanded, const int *tree_nodes, int *out_selected_node,
-               int *out_path_eids, int *out_path_len, int trees, int nodes, int edges, int warps, int path_depth) {
+/* node_capacity: optional int32 [trees, nodes] limit on the children of each node (NULL = `edges`, the reference). */
+static void select_all(float cpuct, float c_pw, float alpha_pw, int soft_winner, const int *edge_child_id,
+                       const float *edge_prior, const float *edge_W, const int *edge_N, int *edge_inflight,
+                       int *node_expand_inflight, const int *node_expanded, const int *tree_nodes,
+                       int *out_selected_node, int *out_path_eids, int *out_path_len, int trees, int nodes, int edges,
+                       int warps, int path_depth, const int *node_capacity) {
     for (int tree = 0; tree < trees; ++tree)
         for (int wid = 0; wid < warps; ++wid) {
             const size_t out = (size_t)tree * warps + wid;
             select_one(cpuct, c_pw, alpha_pw, soft_winner, edge_child_id, edge_prior, edge_W, edge_N, edge_inflight,
                        node_expand_inflight, node_expanded, tree_nodes[tree], out_selected_node + out,
-                       out_path_eids + out * path_depth, out_path_len + out, tree, wid, nodes, edges, path_depth);
+                       out_path_eids + out * path_depth, out_path_len + out, tree, wid, nodes, edges, path_depth,
+                       node_capacity);
         }
+}
+
+void po_select(float cpuct, float c_pw, float alpha_pw, int soft_winner, const int *edge_child_id,
+               const float *edge_prior, const float *edge_W, const int *edge_N, int *edge_inflight,
+               int *node_expand_inflight, const int *node_expanded, const int *tree_nodes, int *out_selected_node,
+               int *out_path_eids, int *out_path_len, int trees, int nodes, int edges, int warps, int path_depth) {
+    select_all(cpuct, c_pw, alpha_pw, soft_winner, edge_child_id, edge_prior, edge_W, edge_N, edge_inflight,
+               node_expand_inflight, node_expanded, tree_nodes, out_selected_node, out_path_eids, out_path_len, trees,
+               nodes, edges, warps, path_depth, NULL);
 }
 
 /* node_level != 0: src/puct/puct_gpu_v2.py:847-927 as written.  node_level == 0: the same conversion applied to
@@ -229,3 +242,174 @@ void po_backup(int node_level, int virtual_loss, const int *edge_child_id, float
         }
     }
 }
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ * Gomoku PUCT loop (selection -> expansion / evaluation -> backup per step).  The reference has no such loop; this
+ * restates the library's own definition (include/puct_gomoku.h) sequentially, so it is a second implementation of
+ * the same specification rather than a restatement of reference code: PARITY UNPINNED against the reference.  The
+ * synthetic evaluator (hash, value, Gamma weights) is shared with the library through its header, because it is
+ * the definition of the workload's inputs; what is restated here is the tree logic.  Pins: tests/test_puct_oracle.py
+ * checks the rules (five in a row exactly) against the brute-force outcome routine of the MCTS-NC oracle, the priors
+ * against the Dirichlet moments, and structural invariants of the trees.
+ * ------------------------------------------------------------------------------------------------------------------ */
+#include "../mcts_numba_cuda_amd/csrc/puct_synthetic.h"
+
+#define G_EDGES 256
+#define G_WORDS 16
+
+typedef struct {
+    int *edge_child; float *edge_prior; float *edge_w; int *edge_n; int *edge_inflight; uint8_t *edge_action;
+    int *node_expanded; int *node_expand_inflight; int *node_count; uint32_t *node_board; int8_t *node_turn;
+    float *node_value; int *out_selected; int *out_path; int *out_len; float *path_values; int *node_legal;
+} po_gomoku_arrays;
+
+static int g_stone(const uint32_t *colour, int cell) { return (colour[cell >> 5] >> (cell & 31)) & 1u; }
+
+static int g_popcount(const uint32_t *w) {
+    int c = 0;
+    for (int i = 0; i < G_WORDS; ++i) c += __builtin_popcount(w[i]);
+    return c;
+}
+
+/* exactly five through `cell` for the colour `mine` */
+static int g_makes_five(const uint32_t *mine, int cell, int m, int n) {
+    static const int dirs[4][2] = {{0, 1}, {1, 0}, {1, 1}, {1, -1}};
+    const int r0 = cell / n, c0 = cell % n;
+    for (int d = 0; d < 4; ++d) {
+        int run = 1;
+        for (int s = -1; s <= 1; s += 2)
+            for (int k = 1;; ++k) {
+                const int r = r0 + s * k * dirs[d][0], c = c0 + s * k * dirs[d][1];
+                if (r < 0 || r >= m || c < 0 || c >= n || !g_stone(mine, r * n + c)) break;
+                ++run;
+            }
+        if (run == 5) return 1;
+    }
+    return 0;
+}
+
+static void g_write_priors(const po_gomoku_arrays *A, size_t node_row, const uint32_t *board, uint64_t bh, int cells,
+                           double alpha) {
+    uint64_t weight[G_EDGES], sum = 0;
+    int legal[G_EDGES], n_legal = 0;
+    for (int c = 0; c < cells; ++c) {
+        legal[c] = !g_stone(board, c) && !g_stone(board + 8, c);
+        if (legal[c]) {
+            weight[c] = psyn_cell_weight(alpha, bh, c);
+            sum += weight[c];
+            ++n_legal;
+        }
+    }
+    for (int c = 0; c < cells; ++c) {
+        if (!legal[c]) continue;
+        int rank = 0;
+        for (int o = 0; o < cells; ++o)
+            if (legal[o] && (weight[o] > weight[c] || (weight[o] == weight[c] && o < c))) ++rank;
+        const size_t e = node_row * G_EDGES + rank;
+        A->edge_prior[e] = psyn_prior(weight[c], sum, n_legal);
+        A->edge_action[e] = (uint8_t)c;
+        A->edge_child[e] = -1;
+        A->edge_n[e] = 0;
+        A->edge_w[e] = 0.0f;
+        A->edge_inflight[e] = 0;
+    }
+}
+
+void po_gomoku_search(const po_gomoku_arrays *A, const int8_t *root, int root_turn, int m, int n, int trees, int nodes,
+                      int warps, int path_depth, int steps, float cpuct, float c_pw, float alpha_pw, int soft_winner,
+                      float dirichlet_alpha, uint64_t seed, int64_t *tally /* [trees][8] */) {
+    const int cells = m * n;
+    const double alpha = (double)dirichlet_alpha;
+    uint32_t words[G_WORDS] = {0};
+    for (int i = 0; i < cells; ++i) {
+        if (root[i] == 1) words[i >> 5] |= 1u << (i & 31);
+        if (root[i] == -1) words[8 + (i >> 5)] |= 1u << (i & 31);
+    }
+    for (int t = 0; t < trees; ++t) {
+        const size_t trow = (size_t)t * nodes;
+        for (int i = 0; i < G_WORDS; ++i) A->node_board[trow * G_WORDS + i] = words[i];
+        const int n_legal = cells - g_popcount(words);
+        A->node_turn[trow] = (int8_t)root_turn;
+        A->node_value[trow] = 0.0f;
+        A->node_expanded[trow] = n_legal == 0 ? TERMINAL : 0;
+        A->node_expand_inflight[trow] = 0;
+        A->node_legal[trow] = n_legal;
+        A->node_count[t] = 1;
+        for (int k = 0; k < 8; ++k) tally[t * 8 + k] = 0;
+        if (n_legal > 0) g_write_priors(A, trow, words, psyn_board_hash(psyn_tree_seed(seed, t), words), cells, alpha);
+    }
+    for (int step = 0; step < steps; ++step) {
+        select_all(cpuct, c_pw, alpha_pw, soft_winner, A->edge_child, A->edge_prior, A->edge_w, A->edge_n, A->edge_inflight,
+                   A->node_expand_inflight, A->node_expanded, A->node_count, A->out_selected, A->out_path, A->out_len, trees,
+                   nodes, G_EDGES, warps, path_depth, A->node_legal);
+        for (int t = 0; t < trees; ++t) {
+            const size_t trow = (size_t)t * nodes;
+            const uint64_t tree_seed = psyn_tree_seed(seed, t);
+            /* which traversals want a child, and does the tree have room for all of them? */
+            int total = 0;
+            for (int w = 0; w < warps; ++w) {
+                const int raw = A->out_selected[(size_t)t * warps + w];
+                const int kind = (raw >> KIND_SHIFT) & KIND_MASK, node = raw & NODE_MASK, slot = (raw >> SLOT_SHIFT) & EDGE_MASK;
+                tally[t * 8 + kind] += 1;
+                if (kind == K_EXPAND && slot < cells - g_popcount(A->node_board + (trow + node) * G_WORDS)) ++total;
+            }
+            const int base = A->node_count[t];
+            const int fits = base + total <= nodes;
+            int next = base;
+            if (fits) {
+                A->node_count[t] = base + total;
+                tally[t * 8 + 5] += total;
+            }
+            for (int w = 0; w < warps; ++w) {
+                const size_t out = (size_t)t * warps + w;
+                const int raw = A->out_selected[out];
+                const int kind = (raw >> KIND_SHIFT) & KIND_MASK, node = raw & NODE_MASK, slot = (raw >> SLOT_SHIFT) & EDGE_MASK;
+                if (kind != K_EXPAND && kind != K_TERMINAL && kind != K_DEPTH_LIMIT) continue;
+                uint32_t board[G_WORDS];
+                for (int i = 0; i < G_WORDS; ++i) board[i] = A->node_board[(trow + node) * G_WORDS + i];
+                const int n_legal = cells - g_popcount(board);
+                const int turn = A->node_turn[trow + node];
+                float u;
+                if (kind == K_EXPAND && slot < n_legal && fits) {
+                    const int child = next++;
+                    const size_t e = (trow + node) * G_EDGES + slot;
+                    const int action = A->edge_action[e];
+                    uint32_t *mine = board + (turn > 0 ? 0 : 8);
+                    mine[action >> 5] |= 1u << (action & 31);
+                    const int win = g_makes_five(mine, action, m, n);
+                    const int terminal = win || n_legal - 1 == 0;
+                    const uint64_t bh = psyn_board_hash(tree_seed, board);
+                    const float v_child = win ? -1.0f : (terminal ? 0.0f : psyn_value(bh));
+                    for (int i = 0; i < G_WORDS; ++i) A->node_board[(trow + child) * G_WORDS + i] = board[i];
+                    A->node_turn[trow + child] = (int8_t)-turn;
+                    A->node_value[trow + child] = v_child;
+                    A->node_expanded[trow + child] = terminal ? TERMINAL : 0;
+                    A->node_expand_inflight[trow + child] = 0;
+                    A->node_legal[trow + child] = n_legal - 1;
+                    A->edge_child[e] = child;
+                    A->edge_n[e] = 1;
+                    A->edge_w[e] = -v_child;
+                    A->node_expanded[trow + node] += 1;
+                    if (!terminal) g_write_priors(A, trow + child, board, bh, cells, alpha);
+                    u = -v_child;
+                } else if (kind == K_TERMINAL) {
+                    u = A->node_value[trow + node];
+                } else {
+                    u = psyn_value(psyn_board_hash(tree_seed, board));
+                }
+                const int L = A->out_len[out] - 1;
+                for (int d = 0; d < L; ++d) A->path_values[out * path_depth + d] = ((L - d) & 1) ? -u : u;
+            }
+        }
+        po_backup(0, 1, NULL, A->edge_w, A->edge_n, A->edge_inflight, NULL, A->node_expand_inflight, A->node_count,
+                  A->out_selected, A->out_path, A->out_len, A->path_values, trees, nodes, G_EDGES, warps, path_depth);
+    }
+}
+
+/* helpers the tests use to pin the evaluator and the rule check */
+double po_det_exp(double x) { return detm_exp(x); }
+double po_gamma(double alpha, uint64_t key) { return psyn_gamma(alpha, key); }
+uint64_t po_cell_weight(double alpha, uint64_t board_hash, int cell) { return psyn_cell_weight(alpha, board_hash, cell); }
+float po_value(uint64_t board_hash) { return psyn_value(board_hash); }
+uint64_t po_board_hash(uint64_t seed, int tree, const uint32_t *words) { return psyn_board_hash(psyn_tree_seed(seed, tree), words); }
+int po_makes_five(const uint32_t *mine, int cell, int m, int n) { return g_makes_five(mine, cell, m, n); }

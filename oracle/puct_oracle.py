@@ -58,3 +58,57 @@ def backup(h, values=None, virtual_loss=1, node_level=False):
                     _ptr(h["node_count"]), _ptr(h["out_selected"]), _ptr(h["out_path"]), _ptr(h["out_len"]),
                     _ptr(values), trees, nodes, edges, warps, depth)
     return h
+
+
+class _GomokuArrays(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in
+                ("edge_child", "edge_prior", "edge_w", "edge_n", "edge_inflight", "edge_action", "node_expanded",
+                 "node_expand_inflight", "node_count", "node_board", "node_turn", "node_value", "out_selected",
+                 "out_path", "out_len", "path_values", "node_legal")]
+
+
+def gomoku_search(board, turn, steps, trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0,
+                  alpha_pw=0.5, soft_winner=0, dirichlet_alpha=0.3, seed=0):
+    """Sequential Gomoku PUCT search (oracle/puct_oracle.c: po_gomoku_search); returns every array plus the tallies."""
+    board = np.ascontiguousarray(board, dtype=np.int8)
+    m, n = board.shape
+    T, N, E, W, D = trees, max_nodes, 256, traversals, path_depth
+    h = {
+        "edge_child": np.full((T, N, E), -1, np.int32), "edge_prior": np.zeros((T, N, E), np.float32),
+        "edge_w": np.zeros((T, N, E), np.float32), "edge_n": np.zeros((T, N, E), np.int32),
+        "edge_inflight": np.zeros((T, N, E), np.int32), "edge_action": np.zeros((T, N, E), np.uint8),
+        "node_expanded": np.zeros((T, N), np.int32), "node_expand_inflight": np.zeros((T, N), np.int32),
+        "node_count": np.zeros((T,), np.int32), "node_board": np.zeros((T, N, 16), np.uint32),
+        "node_turn": np.zeros((T, N), np.int8), "node_value": np.zeros((T, N), np.float32),
+        "out_selected": np.zeros((T, W), np.int32), "out_path": np.full((T, W, D), -1, np.int32),
+        "out_len": np.zeros((T, W), np.int32), "path_values": np.zeros((T, W, D), np.float32),
+        "node_legal": np.zeros((T, N), np.int32),
+    }
+    arrays = _GomokuArrays(*[h[name].ctypes.data for name, _ in _GomokuArrays._fields_])
+    tally = np.zeros((T, 8), np.int64)
+    L = lib()
+    L.po_gomoku_search.restype = None
+    L.po_gomoku_search.argtypes = [ctypes.POINTER(_GomokuArrays), ctypes.c_void_p] + [ctypes.c_int] * 8 + \
+        [ctypes.c_float] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_uint64, ctypes.c_void_p]
+    L.po_gomoku_search(ctypes.byref(arrays), board.ctypes.data, int(turn), m, n, T, N, W, D, int(steps), cpuct, c_pw,
+                       alpha_pw, int(soft_winner), dirichlet_alpha, int(seed), tally.ctypes.data)
+    h["tally"] = tally
+    return h
+
+
+def evaluator():
+    """The synthetic evaluator's primitives, for the tests that pin them."""
+    L = lib()
+    L.po_det_exp.restype = ctypes.c_double
+    L.po_det_exp.argtypes = [ctypes.c_double]
+    L.po_gamma.restype = ctypes.c_double
+    L.po_gamma.argtypes = [ctypes.c_double, ctypes.c_uint64]
+    L.po_cell_weight.restype = ctypes.c_uint64
+    L.po_cell_weight.argtypes = [ctypes.c_double, ctypes.c_uint64, ctypes.c_int]
+    L.po_value.restype = ctypes.c_float
+    L.po_value.argtypes = [ctypes.c_uint64]
+    L.po_board_hash.restype = ctypes.c_uint64
+    L.po_board_hash.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.c_void_p]
+    L.po_makes_five.restype = ctypes.c_int
+    L.po_makes_five.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    return L

@@ -61,3 +61,91 @@ def test_node_level_backup_matches_v2_known_answer():
     po.backup(h, values, node_level=True)
     assert int(h["node_inflight"].sum()) == 0 and int(h["node_expand_inflight"].sum()) == 0
     assert h["edge_n"][0, 0, 1] == 2 and h["edge_w"][0, 0, 1] == np.float32(0.7)
+
+
+# ---- Gomoku PUCT loop: the evaluator and the sequential search -------------------------------------------------------
+import math
+
+import puct_gomoku_checks as gc
+
+
+def test_det_exp_within_one_ulp_of_libm():
+    ev = po.evaluator()
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([rng.uniform(-700, 700, 20000), rng.uniform(-2, 2, 20000), [0.0, -0.0, 1e-10, -1e-10, 0.3465735, 1.0397]])
+    for x in xs:
+        got, want = ev.po_det_exp(float(x)), math.exp(float(x))
+        assert abs(got - want) <= math.ulp(want), x
+    assert ev.po_det_exp(-800.0) == 0.0 and ev.po_det_exp(800.0) == math.inf
+
+
+def test_gamma_variates_have_gamma_moments():
+    ev = po.evaluator()
+    for alpha in (0.3, 0.7):
+        g = np.array([ev.po_gamma(alpha, k * 0x9E3779B97F4A7C15 % 2**64) for k in range(200000)])
+        assert np.all(g >= 0)
+        assert abs(g.mean() - alpha) < 0.01 and abs(g.var() - alpha) < 0.03      # Gamma(alpha, 1): mean = var = alpha
+        # third central moment of Gamma(alpha, 1) is 2 alpha
+        assert abs(((g - g.mean()) ** 3).mean() - 2 * alpha) < 0.15
+
+
+def test_root_priors_have_dirichlet_moments():
+    """Priors of the empty 15x15 board over 64 trees (64 different evaluators): a permutation of the cells in
+    descending order, summing to one, with the marginal variance of Dirichlet(0.3, ..., 0.3)."""
+    board = np.zeros((15, 15), np.int8)
+    h = po.gomoku_search(board, 1, 0, trees=64, traversals=1, max_nodes=2)
+    pri = h["edge_prior"][:, 0, :225].astype(np.float64)
+    acts = h["edge_action"][:, 0, :225]
+    assert np.all(np.sort(acts, axis=1) == np.arange(225))
+    assert np.all(np.diff(pri, axis=1) <= 0) and np.allclose(pri.sum(axis=1), 1.0, atol=1e-5)
+    n, alpha = 225, 0.3
+    want_var = (1 / n) * (1 - 1 / n) / (n * alpha + 1)
+    assert abs(pri.var() / want_var - 1.0) < 0.15          # 14400 samples of a heavy-tailed marginal
+    by_cell = np.zeros((64, 225))
+    np.put_along_axis(by_cell, acts.astype(int), pri, axis=1)
+    assert abs(by_cell.mean(axis=0).mean() - 1 / n) < 1e-9 and by_cell.mean(axis=0).max() < 5 / n   # no favoured cell
+
+
+def test_exactly_five_rule_against_brute_force():
+    ev = po.evaluator()
+    rng = np.random.default_rng(2)
+    hits = 0
+    for _ in range(3000):
+        m, n = int(rng.integers(5, 16)), int(rng.integers(5, 17))
+        if m * n > 256:
+            continue
+        stones = rng.random(m * n) < 0.55
+        cell = int(rng.integers(0, m * n))
+        stones[cell] = True
+        words = np.zeros(8, np.uint32)
+        for c in np.flatnonzero(stones):
+            words[c >> 5] |= np.uint32(1 << (c & 31))
+        want = 5 in gc.run_through(stones, m, n, cell)
+        hits += want
+        assert bool(ev.po_makes_five(words.ctypes.data, cell, m, n)) == want
+    assert hits > 100
+
+
+@pytest.mark.parametrize("shape,stones,traversals,steps,max_nodes,depth", [
+    ((15, 15), 0, 1, 300, 4096, 64), ((15, 15), 12, 4, 150, 4096, 64), ((6, 6), 4, 2, 400, 4096, 64),
+    ((5, 5), 18, 3, 200, 2048, 64), ((9, 9), 0, 8, 120, 300, 64), ((7, 7), 0, 2, 300, 4096, 3)])
+def test_sequential_search_builds_consistent_trees(shape, stones, traversals, steps, max_nodes, depth):
+    from helpers import random_gomoku_root
+    rng = np.random.default_rng(shape[0] * 100 + stones)
+    board, turn = random_gomoku_root(rng, shape[0], shape[1], stones)
+    h = po.gomoku_search(board, turn, steps, trees=3, traversals=traversals, max_nodes=max_nodes, path_depth=depth, seed=5)
+    gc.check_trees(h, board, turn, shape[0], shape[1], max_nodes, depth)
+    tally = h["tally"]
+    assert np.all(tally[:, :5].sum(axis=1) == steps * traversals) and np.all(tally[:, 0] == 0)
+    assert np.array_equal(tally[:, 5], h["node_count"] - 1)
+    # every selection that is not busy adds exactly one visit to one root edge, except an expansion of the root itself
+    # that a full tree could not take
+    for t in range(3):
+        if max_nodes >= 2048:
+            assert gc.visits_below(h, t, 0) == int(tally[t, 1:4].sum())
+        else:
+            assert gc.visits_below(h, t, 0) <= int(tally[t, 1:4].sum())
+    if max_nodes >= 2048 and depth >= 64:
+        gc.check_visit_flow(h, depth)
+    else:
+        assert (tally[:, 3].sum() > 0) or np.any(h["node_count"] + traversals > max_nodes)   # the limit was exercised
