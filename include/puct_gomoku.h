@@ -38,6 +38,7 @@ typedef struct {
     int32_t path_depth;        /* longest path a selection may take, 1..1024 */
     float cpuct, c_pw, alpha_pw;
     int32_t soft_winner;
+    int32_t recalc_attempts;   /* attempts of the winner-recalc claim per level, 1..64; 0 = 2 as in the reference's kernel */
     float dirichlet_alpha;     /* in (0, 1) */
     uint64_t seed;
     int32_t device;

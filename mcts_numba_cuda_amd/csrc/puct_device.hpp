@@ -20,6 +20,7 @@ namespace puct {
 constexpr int kWave = 64;
 constexpr int kMaxWavesPerBlock = 16;
 constexpr int kRecalcAttempts = 2;  // MAX_RECALC_RETRY, src/puct/puct_gpu_v3_cpp.cu:36
+constexpr int kPasses = (PUCT_PACKED_EDGE_MASK + 1) / kWave;  // 64-edge slices of the widest node
 constexpr int kNoEdge = 0x7fffffff;
 
 struct SelectArgs {
@@ -41,6 +42,8 @@ struct SelectArgs {
     // the reference's behaviour.  A caller whose nodes have fewer possible children than `edges` (legal moves) passes
     // it so that progressive widening stops asking for slots a node cannot have.
     const int *node_capacity = nullptr;
+    // Attempts of the winner-recalc claim per level; the reference has 2 compiled in.
+    int recalc_attempts = kRecalcAttempts;
 };
 
 // ---- cross-lane reductions -------------------------------------------------------------------------------------
@@ -159,15 +162,17 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
             const size_t nrow = (size_t)tree * nodes + node;
             const size_t erow = nrow * edges;
 
-            // Everything a level can need from the first 64 edges, requested in one go.
-            int n0 = 0, f0 = 0, c0 = -1;
-            float p0 = 0.0f, w0 = 0.0f;
+            // Everything a level can need from the first 64 edges, requested in one go; the edges of wider nodes follow
+            // once the node's width is known and stay in registers for the rest of the level.
+            int n[kPasses], f[kPasses], c[kPasses];
+            float p[kPasses], w[kPasses];
+            n[0] = 0, f[0] = 0, c[0] = -1, p[0] = 0.0f, w[0] = 0.0f;
             if (lane < edges) {
-                n0 = a.edge_N[erow + lane];
-                f0 = load_relaxed(a.edge_inflight + erow + lane);
-                p0 = a.edge_prior[erow + lane];
-                w0 = a.edge_W[erow + lane];
-                c0 = a.edge_child_id[erow + lane];
+                n[0] = a.edge_N[erow + lane];
+                f[0] = load_relaxed(a.edge_inflight + erow + lane);
+                p[0] = a.edge_prior[erow + lane];
+                w[0] = a.edge_W[erow + lane];
+                c[0] = a.edge_child_id[erow + lane];
             }
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
@@ -191,11 +196,23 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
             }
 
             const int cur_expanded = node_info;
+#pragma unroll
+            for (int i = 1; i < kPasses; ++i) {
+                n[i] = 0, f[i] = 0, c[i] = -1, p[i] = 0.0f, w[i] = 0.0f;
+                const int eid = lane + i * kWave;
+                if (i * kWave < cur_expanded && eid < cur_expanded) {
+                    n[i] = a.edge_N[erow + eid];
+                    f[i] = load_relaxed(a.edge_inflight + erow + eid);
+                    p[i] = a.edge_prior[erow + eid];
+                    w[i] = a.edge_W[erow + eid];
+                    c[i] = a.edge_child_id[erow + eid];
+                }
+            }
             int parent_eff = 1, allowed = 1;
             if (cur_expanded != 1 || a.c_pw != 0.0f) {
-                int total = lane < cur_expanded ? n0 + f0 : 0;
-                for (int eid = lane + kWave; eid < cur_expanded; eid += kWave)
-                    total += a.edge_N[erow + eid] + load_relaxed(a.edge_inflight + erow + eid);
+                int total = 0;
+#pragma unroll
+                for (int i = 0; i < kPasses; ++i) total += lane + i * kWave < cur_expanded ? n[i] + f[i] : 0;
                 total = wave_sum(total);
                 parent_eff = total > 1 ? total : 1;
                 allowed = allowed_children(a.c_pw, a.alpha_pw, parent_eff, capacity);
@@ -239,23 +256,20 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                 // another traversal got there first.
                 const float sqrt_parent = sqrtf((float)parent_eff);
                 best_eid = kNoEdge;
-                for (int attempt = 0; attempt < kRecalcAttempts; ++attempt) {
+                for (int attempt = 0; attempt < a.recalc_attempts; ++attempt) {
                     uint64_t key = 0;
                     int my_inflight = 0;
-                    if (lane < cur_expanded) {
-                        my_inflight = attempt == 0 ? f0 : load_relaxed(a.edge_inflight + erow + lane);
-                        key = candidate_key(puct_score(a.cpuct, p0, w0, n0, my_inflight, sqrt_parent), lane,
-                                            tie_offset, cur_expanded);
-                    }
-                    for (int eid = lane + kWave; eid < cur_expanded; eid += kWave) {
-                        const int f = load_relaxed(a.edge_inflight + erow + eid);
-                        const uint64_t k = candidate_key(
-                            puct_score(a.cpuct, a.edge_prior[erow + eid], a.edge_W[erow + eid], a.edge_N[erow + eid], f,
-                                       sqrt_parent),
-                            eid, tie_offset, cur_expanded);
-                        if (k > key) {
-                            key = k;
-                            my_inflight = f;
+#pragma unroll
+                    for (int i = 0; i < kPasses; ++i) {
+                        const int eid = lane + i * kWave;
+                        if (i * kWave < cur_expanded && eid < cur_expanded) {
+                            const int fi = attempt == 0 ? f[i] : load_relaxed(a.edge_inflight + erow + eid);
+                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], fi, sqrt_parent), eid,
+                                                             tie_offset, cur_expanded);
+                            if (k > key) {
+                                key = k;
+                                my_inflight = fi;
+                            }
                         }
                     }
                     const uint64_t best = wave_max(key);
@@ -288,8 +302,11 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                 break;
             }
 
-            const int best_child =
-                best_eid < kWave ? __builtin_amdgcn_readlane(c0, best_eid) : a.edge_child_id[erow + best_eid];
+            const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
+            int best_child = __builtin_amdgcn_readlane(c[0], best_lane);
+#pragma unroll
+            for (int i = 1; i < kPasses; ++i)
+                if (best_pass == i) best_child = __builtin_amdgcn_readlane(c[i], best_lane);
             if (best_child < 0 || best_child >= node_cnt) {
                 if (lane == 0) atomicSub(&a.edge_inflight[erow + best_eid], 1);
                 rollback_path(a, path, tree, depth, lane, node_cnt);

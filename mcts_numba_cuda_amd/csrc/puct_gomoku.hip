@@ -17,7 +17,6 @@ using namespace puct;
 
 constexpr int kEdges = 256;       // edge slots per node (MAX_ACTION of src/puct/puct_gpu_v2.py:72)
 constexpr int kBoardWords = 16;   // 8 words per colour
-constexpr uint64_t kIllegal = ~0ull;
 
 struct GomokuArgs {
     SelectArgs sel;
@@ -42,7 +41,7 @@ struct GomokuArgs {
 struct Lds {
     int want[kMaxWavesPerBlock];
     uint32_t board[kMaxWavesPerBlock][kBoardWords];
-    uint64_t weight[kMaxWavesPerBlock][kEdges];
+    alignas(16) uint32_t keys[kMaxWavesPerBlock][kEdges];
 };
 
 __device__ __forceinline__ uint64_t wave_sum64(uint64_t v) {
@@ -83,34 +82,66 @@ __device__ __forceinline__ bool makes_five(const uint32_t *mine, int cell, int m
     return __ballot(hit) != 0;
 }
 
-// Priors of a new node: one Gamma weight per legal cell, prior = weight / sum, edge slots in descending prior order
+// Priors of a new node: one Gamma weight per legal cell, prior = weight / sum, edge slots in descending weight order
 // (ties: smaller cell first), so that progressive widening opens the most promising moves first.  Initialises every
-// edge field of the node's legal slots.
-__device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint32_t *board, uint64_t *weight, int lane,
+// edge field of the node's legal slots.  `keys` is this wavefront's LDS scratch.
+__device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint32_t *board, uint32_t *keys, int lane,
                              uint64_t board_hash, int n_legal) {
-    uint64_t mine[4];
+    constexpr int kPer = kEdges / kWave;
+    uint32_t mine[kPer];
+    // Rejection sampling diverges between lanes; every lane walks through its own cells and rounds independently, so
+    // the wavefront runs for the largest per-lane total instead of the sum of per-cell maxima.
+    int i = 0, round = 0;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) mine[k] = 0u;
+    auto legal_cell = [&](int k) {
+        const int c = lane + k * kWave;
+        return c < g.cells && !stone_at(board, c) && !stone_at(board + 8, c);
+    };
+    while (i < kPer && !legal_cell(i)) ++i;
+    while (__ballot(i < kPer) != 0) {
+        if (i < kPer) {
+            const int c = lane + i * kWave;
+            double x;
+            const int ok = psyn_gamma_round(g.dirichlet_alpha, psyn_cell_key(board_hash, c), round, &x);
+            if (ok || round == PSYN_GAMMA_ROUNDS - 1) {
+                const uint32_t key = psyn_weight_key(x, c);
+#pragma unroll
+                for (int k = 0; k < kPer; ++k)
+                    if (k == i) mine[k] = key;
+                ++i;
+                round = 0;
+                while (i < kPer && !legal_cell(i)) ++i;
+            } else {
+                ++round;
+            }
+        }
+    }
     uint64_t sum = 0;
-    for (int i = 0; i < 4; ++i) {
-        const int c = lane + i * kWave;
-        const bool legal = c < g.cells && !stone_at(board, c) && !stone_at(board + 8, c);
-        mine[i] = legal ? psyn_cell_weight(g.dirichlet_alpha, board_hash, c) : kIllegal;
-        weight[c] = mine[i];
-        sum += legal ? mine[i] : 0;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        keys[lane + k * kWave] = mine[k];
+        sum += mine[k] ? psyn_key_weight(mine[k]) : 0;
     }
     sum = wave_sum64(sum);
     wave_lds_fence();
+    int rank[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) rank[k] = 0;
+    const uint4 *keys4 = reinterpret_cast<const uint4 *>(keys);
+    for (int o = 0; o < kEdges / 4; ++o) {
+        const uint4 q = keys4[o];
+#pragma unroll
+        for (int k = 0; k < kPer; ++k)
+            rank[k] += (q.x > mine[k] ? 1 : 0) + (q.y > mine[k] ? 1 : 0) + (q.z > mine[k] ? 1 : 0) + (q.w > mine[k] ? 1 : 0);
+    }
     const size_t erow = ((size_t)tree * g.sel.nodes + node) * kEdges;
-    for (int i = 0; i < 4; ++i) {
-        const int c = lane + i * kWave;
-        if (mine[i] == kIllegal) continue;
-        int rank = 0;
-        for (int o = 0; o < g.cells; ++o) {
-            const uint64_t w = weight[o];
-            rank += (w != kIllegal && (w > mine[i] || (w == mine[i] && o < c))) ? 1 : 0;
-        }
-        const size_t e = erow + rank;
-        g.edge_prior[e] = psyn_prior(mine[i], sum, n_legal);
-        g.edge_action[e] = (uint8_t)c;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+        if (mine[k] == 0u) continue;
+        const size_t e = erow + rank[k];
+        g.edge_prior[e] = psyn_prior(psyn_key_weight(mine[k]), sum, n_legal);
+        g.edge_action[e] = (uint8_t)(lane + k * kWave);
         g.edge_child[e] = -1;
         g.edge_N[e] = 0;
         g.edge_W[e] = 0.0f;
@@ -184,7 +215,7 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
             g.edge_W[erow + slot] = -v_child;
             atomicAdd(&g.node_expanded[trow + node], 1);
         }
-        if (!terminal) write_priors(g, tree, child, board, lds.weight[wave], lane, bh, child_legal);
+        if (!terminal) write_priors(g, tree, child, board, lds.keys[wave], lane, bh, child_legal);
         u = -v_child;
     } else if (kind == PUCT_SELECT_TERMINAL) {
         u = g.node_value[trow + node];
@@ -201,7 +232,7 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
 // Root of every tree: node 0 with the root position and its priors.
 __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const uint32_t *root_board, int root_turn) {
     __shared__ uint32_t board[kBoardWords];
-    __shared__ uint64_t weight[kEdges];
+    __shared__ alignas(16) uint32_t weight[kEdges];
     const int tree = blockIdx.x, lane = threadIdx.x;
     const size_t trow = (size_t)tree * g.sel.nodes;
     const uint32_t w = lane < kBoardWords ? root_board[lane] : 0u;
@@ -327,6 +358,7 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     if (c->path_depth < 1 || c->path_depth > 1024) return fail(PUCT_GOMOKU_E_INVALID, "path_depth = %d, need 1..1024", c->path_depth);
     if (!(c->dirichlet_alpha > 0.0f && c->dirichlet_alpha < 1.0f))
         return fail(PUCT_GOMOKU_E_INVALID, "dirichlet_alpha = %g, need 0 < alpha < 1", (double)c->dirichlet_alpha);
+    if (c->recalc_attempts < 0 || c->recalc_attempts > 64) return fail(PUCT_GOMOKU_E_INVALID, "recalc_attempts = %d, need 0..64", c->recalc_attempts);
     if (!(c->cpuct >= 0.0f) || !(c->c_pw >= 0.0f)) return fail(PUCT_GOMOKU_E_INVALID, "cpuct and c_pw must not be negative");
     HIP_TRY(hipSetDevice(c->device));
     auto *e = new puct_gomoku_engine();
@@ -352,7 +384,8 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     }
     g.sel = SelectArgs{c->cpuct, c->c_pw, c->alpha_pw, c->soft_winner, g.edge_child, g.edge_prior, g.edge_W, g.edge_N, g.edge_inflight,
                        g.node_expand_inflight, g.node_expanded, g.node_count, out_selected, out_path, out_len,
-                       c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth, g.node_legal};
+                       c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth, g.node_legal,
+                       c->recalc_attempts > 0 ? c->recalc_attempts : kRecalcAttempts};
     g.bk = BackupArgs{1, nullptr, g.edge_W, g.edge_N, g.edge_inflight, nullptr, g.node_expand_inflight, g.node_count,
                       out_selected, out_path, out_len, g.path_values, c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth};
     g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes; g.steps = 0;

@@ -51,34 +51,53 @@ PSYN_FN float psyn_value(uint64_t board_hash) {
 /* Uniform double in (0, 1), never 0 or 1. */
 PSYN_FN double psyn_unit(uint64_t h) { return ((double)(h >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
 
-/* Gamma(alpha, 1) variate for 0 < alpha < 1 (Ahrens-Dieter rejection "GS") driven by a counter-based stream of
- * uniforms derived from `key`; at most 16 rounds (the chance of needing more is below 1e-9), after which the last
- * candidate is returned. */
-PSYN_FN double psyn_gamma(double alpha, uint64_t key) {
+/* One round of the Ahrens-Dieter rejection sampler "GS" for Gamma(alpha, 1), 0 < alpha < 1, driven by the uniforms
+ * number 2 * round and 2 * round + 1 of the counter-based stream of `key`.  Writes the candidate to *x and returns
+ * whether it is accepted.  The acceptance tests are taken in the log domain (log u2 <= -x, resp.
+ * log u2 <= (alpha - 1) log x), which lets both branches share two of their three logarithms. */
+PSYN_FN int psyn_gamma_round(double alpha, uint64_t key, int round, double *x) {
     const double b = 1.0 + alpha * 0.36787944117144233; /* 1 + alpha / e */
     const double inv_alpha = 1.0 / alpha;
-    double x = 0.0;
-    for (int round = 0; round < 16; ++round) {
-        const double u1 = psyn_unit(psyn_mix64(key + 2u * (uint64_t)round));
-        const double u2 = psyn_unit(psyn_mix64(key + 2u * (uint64_t)round + 1u));
-        const double p = b * u1;
-        if (p <= 1.0) {
-            x = detm_exp(detm_log(p) * inv_alpha);
-            if (u2 <= detm_exp(-x)) return x;
-        } else {
-            x = -detm_log((b - p) * inv_alpha);
-            if (u2 <= detm_exp((alpha - 1.0) * detm_log(x))) return x;
-        }
+    const double u1 = psyn_unit(psyn_mix64(key + 2u * (uint64_t)round));
+    const double log_u2 = detm_log(psyn_unit(psyn_mix64(key + 2u * (uint64_t)round + 1u)));
+    const double p = b * u1;
+    const int small = p <= 1.0;
+    const double log_t = detm_log(small ? p : (b - p) * inv_alpha);
+    if (small) {
+        *x = detm_exp(log_t * inv_alpha);
+        return log_u2 <= -*x;
     }
+    *x = -log_t;
+    return log_u2 <= (alpha - 1.0) * detm_log(*x);
+}
+
+#define PSYN_GAMMA_ROUNDS 16 /* the chance of needing more is below 1e-9; the last candidate is taken then */
+
+PSYN_FN double psyn_gamma(double alpha, uint64_t key) {
+    double x = 0.0;
+    for (int round = 0; round < PSYN_GAMMA_ROUNDS; ++round)
+        if (psyn_gamma_round(alpha, key, round, &x)) break;
     return x;
 }
 
-/* Gamma variate of `cell` in the position with hash `board_hash`, in 2^-32 fixed point, saturating at 2^40 (a variate
- * of 256, far above anything the generator produces) so that a sum over 256 cells stays below 2^48. */
-PSYN_FN uint64_t psyn_cell_weight(double alpha, uint64_t board_hash, int cell) {
-    const double g = psyn_gamma(alpha, psyn_mix64(board_hash ^ (0x7072696F72ull + ((uint64_t)(uint32_t)cell << 40))));
-    const double scaled = g * 4294967296.0;
-    return scaled >= 1099511627776.0 ? (uint64_t)1099511627776ull : (uint64_t)scaled;
+/* Stream key of `cell` in the position with hash `board_hash`. */
+PSYN_FN uint64_t psyn_cell_key(uint64_t board_hash, int cell) {
+    return psyn_mix64(board_hash ^ (0x7072696F72ull + ((uint64_t)(uint32_t)cell << 40)));
+}
+
+/* The weight of a cell is its Gamma variate, capped at 255 and truncated to a float32 with 15 mantissa bits.  Two
+ * views of the same number: a 32-bit sort key whose unsigned order is "larger weight first, then smaller cell" (0 is
+ * reserved for cells that are not legal), and the weight in 2^-32 fixed point for the exact, order-independent sum
+ * (a sum over 256 cells stays below 2^48). */
+PSYN_FN uint32_t psyn_weight_key(double gamma, int cell) {
+    union { float f; uint32_t u; } v;
+    v.f = (float)(gamma > 255.0 ? 255.0 : gamma);
+    return 0x80000000u | (v.u & 0xFFFFFF00u) | (uint32_t)(255 - cell);
+}
+PSYN_FN uint64_t psyn_key_weight(uint32_t key) {
+    union { float f; uint32_t u; } v;
+    v.u = key & 0x7FFFFF00u;
+    return (uint64_t)((double)v.f * 4294967296.0);
 }
 
 /* Prior of a cell from its weight and the sum of the weights of all legal cells; uniform if every weight is 0. */

@@ -1,7 +1,10 @@
 """Host side of the PUCT select / backup path: a ctypes binding of libpuct_hip.so (C ABI: include/puct_select.h) with
 the calling convention of the reference's binding, src/puct/puct_gpu_v3_cpp.py:118-156 — `launch_select(d, ...)` takes
-a dictionary of device arrays — here torch tensors on the GPU instead of numba device arrays.  There is no CPU
-fallback: without the library, or with tensors that are not on the GPU, every call raises."""
+a dictionary of device arrays — here hipmem.DeviceArray objects or torch tensors on the GPU instead of numba device
+arrays.  There is no CPU fallback: without the library, or with arrays that are not on the GPU, every call raises.
+
+When torch is used in the same process, import torch before this package: torch ships its own copy of the HIP
+runtime, and the copy that is loaded first serves both."""
 import ctypes
 import os
 
@@ -69,16 +72,26 @@ def reason(raw):
 
 
 def _device_ptr(t, dtype, name):
+    """Device address of a contiguous array of `dtype`: a hipmem.DeviceArray or a torch tensor on the GPU."""
+    from .hipmem import DeviceArray
+    if isinstance(t, DeviceArray):
+        if t.dtype != np.dtype(dtype):
+            raise ValueError(f"{name}: expected {np.dtype(dtype)}, got {t.dtype}")
+        return ctypes.c_void_p(t.data_ptr())
     import torch
     want = {np.int32: torch.int32, np.float32: torch.float32}[dtype]
-    if not t.is_cuda or t.dtype != want or not t.is_contiguous():
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != want or not t.is_contiguous():
         raise ValueError(f"{name}: expected a contiguous {want} tensor on the GPU")
     return ctypes.c_void_p(t.data_ptr())
 
 
-def _stream_handle():
-    import torch
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+def _stream_handle(d):
+    """torch's current stream when the arrays are torch tensors, the default stream otherwise."""
+    import sys
+    torch = sys.modules.get("torch")
+    if torch is not None and isinstance(d["edge_child"], torch.Tensor):
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(0)
 
 
 def _check(code, what):
@@ -115,7 +128,7 @@ def launch_select(d, cpuct=1.0, c_pw=1.0, alpha_pw=0.5, soft_winner=0):
         _device_ptr(d["node_expand_inflight"], i32, "node_expand_inflight"),
         _device_ptr(d["node_expanded"], i32, "node_expanded"), _device_ptr(d["node_count"], i32, "node_count"),
         _device_ptr(d["out_selected"], i32, "out_selected"), _device_ptr(d["out_path"], i32, "out_path"),
-        _device_ptr(d["out_len"], i32, "out_len"), trees, nodes, edges, warps, path_depth, _stream_handle())
+        _device_ptr(d["out_len"], i32, "out_len"), trees, nodes, edges, warps, path_depth, _stream_handle(d))
     _check(code, "select")
 
 
@@ -135,7 +148,7 @@ def launch_edge_backup(d, path_edge_values=None, virtual_loss=1):
         _device_ptr(d["node_expand_inflight"], i32, "node_expand_inflight"),
         _device_ptr(d["node_count"], i32, "node_count"), _device_ptr(d["out_selected"], i32, "out_selected"),
         _device_ptr(d["out_path"], i32, "out_path"), _device_ptr(d["out_len"], i32, "out_len"), values,
-        trees, nodes, edges, warps, path_depth, _stream_handle())
+        trees, nodes, edges, warps, path_depth, _stream_handle(d))
     _check(code, "edge backup")
 
 
@@ -152,5 +165,5 @@ def launch_node_backup(d, path_edge_values, virtual_loss=1):
         _device_ptr(d["node_count"], i32, "node_count"), _device_ptr(d["out_selected"], i32, "out_selected"),
         _device_ptr(d["out_path"], i32, "out_path"), _device_ptr(d["out_len"], i32, "out_len"),
         _device_ptr(path_edge_values, f32, "path_edge_values"), trees, nodes, edges, warps, path_depth,
-        _stream_handle())
+        _stream_handle(d))
     _check(code, "node backup")

@@ -21,7 +21,7 @@ class Config(ctypes.Structure):
     _fields_ = [("board_m", ctypes.c_int32), ("board_n", ctypes.c_int32), ("trees", ctypes.c_int32),
                 ("traversals", ctypes.c_int32), ("max_nodes", ctypes.c_int32), ("path_depth", ctypes.c_int32),
                 ("cpuct", ctypes.c_float), ("c_pw", ctypes.c_float), ("alpha_pw", ctypes.c_float),
-                ("soft_winner", ctypes.c_int32), ("dirichlet_alpha", ctypes.c_float), ("seed", ctypes.c_uint64),
+                ("soft_winner", ctypes.c_int32), ("recalc_attempts", ctypes.c_int32), ("dirichlet_alpha", ctypes.c_float), ("seed", ctypes.c_uint64),
                 ("device", ctypes.c_int32)]
 
 
@@ -73,10 +73,10 @@ class PUCTGomoku:
     visits; `root_n`, `root_q`, `selections`, `performance_info` describe the last search."""
 
     def __init__(self, board_shape=(15, 15), trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5,
-                 c_pw=1.0, alpha_pw=0.5, soft_winner=False, dirichlet_alpha=0.3, seed=0, device=0):
+                 c_pw=1.0, alpha_pw=0.5, soft_winner=False, recalc_attempts=0, dirichlet_alpha=0.3, seed=0, device=0):
         self.cfg = Config(int(board_shape[0]), int(board_shape[1]), int(trees), int(traversals), int(max_nodes),
                           int(path_depth), float(cpuct), float(c_pw), float(alpha_pw), int(bool(soft_winner)),
-                          float(dirichlet_alpha), int(seed), int(device))
+                          int(recalc_attempts), float(dirichlet_alpha), int(seed), int(device))
         self._engine = ctypes.c_void_p()
         _check(_lib().puct_gomoku_create(ctypes.byref(self.cfg), ctypes.byref(self._engine)))
         self.result = None

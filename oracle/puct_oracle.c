@@ -290,23 +290,23 @@ static int g_makes_five(const uint32_t *mine, int cell, int m, int n) {
 
 static void g_write_priors(const po_gomoku_arrays *A, size_t node_row, const uint32_t *board, uint64_t bh, int cells,
                            double alpha) {
-    uint64_t weight[G_EDGES], sum = 0;
-    int legal[G_EDGES], n_legal = 0;
+    uint32_t key[G_EDGES];
+    uint64_t sum = 0;
+    int n_legal = 0;
     for (int c = 0; c < cells; ++c) {
-        legal[c] = !g_stone(board, c) && !g_stone(board + 8, c);
-        if (legal[c]) {
-            weight[c] = psyn_cell_weight(alpha, bh, c);
-            sum += weight[c];
+        key[c] = 0;
+        if (!g_stone(board, c) && !g_stone(board + 8, c)) {
+            key[c] = psyn_weight_key(psyn_gamma(alpha, psyn_cell_key(bh, c)), c);
+            sum += psyn_key_weight(key[c]);
             ++n_legal;
         }
     }
     for (int c = 0; c < cells; ++c) {
-        if (!legal[c]) continue;
+        if (!key[c]) continue;
         int rank = 0;
-        for (int o = 0; o < cells; ++o)
-            if (legal[o] && (weight[o] > weight[c] || (weight[o] == weight[c] && o < c))) ++rank;
+        for (int o = 0; o < cells; ++o) rank += key[o] > key[c];
         const size_t e = node_row * G_EDGES + rank;
-        A->edge_prior[e] = psyn_prior(weight[c], sum, n_legal);
+        A->edge_prior[e] = psyn_prior(psyn_key_weight(key[c]), sum, n_legal);
         A->edge_action[e] = (uint8_t)c;
         A->edge_child[e] = -1;
         A->edge_n[e] = 0;
@@ -409,7 +409,7 @@ void po_gomoku_search(const po_gomoku_arrays *A, const int8_t *root, int root_tu
 /* helpers the tests use to pin the evaluator and the rule check */
 double po_det_exp(double x) { return detm_exp(x); }
 double po_gamma(double alpha, uint64_t key) { return psyn_gamma(alpha, key); }
-uint64_t po_cell_weight(double alpha, uint64_t board_hash, int cell) { return psyn_cell_weight(alpha, board_hash, cell); }
+uint32_t po_cell_key(double alpha, uint64_t board_hash, int cell) { return psyn_weight_key(psyn_gamma(alpha, psyn_cell_key(board_hash, cell)), cell); }
 float po_value(uint64_t board_hash) { return psyn_value(board_hash); }
 uint64_t po_board_hash(uint64_t seed, int tree, const uint32_t *words) { return psyn_board_hash(psyn_tree_seed(seed, tree), words); }
 int po_makes_five(const uint32_t *mine, int cell, int m, int n) { return g_makes_five(mine, cell, m, n); }

@@ -103,8 +103,8 @@ def evaluator():
     L.po_det_exp.argtypes = [ctypes.c_double]
     L.po_gamma.restype = ctypes.c_double
     L.po_gamma.argtypes = [ctypes.c_double, ctypes.c_uint64]
-    L.po_cell_weight.restype = ctypes.c_uint64
-    L.po_cell_weight.argtypes = [ctypes.c_double, ctypes.c_uint64, ctypes.c_int]
+    L.po_cell_key.restype = ctypes.c_uint32
+    L.po_cell_key.argtypes = [ctypes.c_double, ctypes.c_uint64, ctypes.c_int]
     L.po_value.restype = ctypes.c_float
     L.po_value.argtypes = [ctypes.c_uint64]
     L.po_board_hash.restype = ctypes.c_uint64

@@ -13,31 +13,35 @@ pytestmark = pytest.mark.gpu
 
 
 def to_device(case):
-    import torch
-    return {k: torch.from_numpy(v).cuda() for k, v in case.items()}
+    from mcts_numba_cuda_amd.hipmem import DeviceArray
+    return {k: DeviceArray(v) for k, v in case.items()}
 
 
 def to_host(d):
-    return {k: v.cpu().numpy() for k, v in d.items()}
+    return {k: v.numpy() for k, v in d.items()}
+
+
+def synchronize():
+    from mcts_numba_cuda_amd.hipmem import synchronize as sync
+    sync()
 
 
 class HipRunner(pc.Runner):
     def select(self, case, **params):
-        import torch
         from mcts_numba_cuda_amd import puct
         self.d = to_device(case)
         puct.launch_select(self.d, **params)
-        torch.cuda.synchronize()
+        synchronize()
         return to_host(self.d)
 
     def release(self):
         return self.backup(None)
 
     def backup(self, values):
-        import torch
         from mcts_numba_cuda_amd import puct
-        puct.launch_edge_backup(self.d, None if values is None else torch.from_numpy(values).cuda())
-        torch.cuda.synchronize()
+        from mcts_numba_cuda_amd.hipmem import DeviceArray
+        puct.launch_edge_backup(self.d, None if values is None else DeviceArray(values))
+        synchronize()
         return to_host(self.d)
 
 
@@ -70,7 +74,6 @@ def test_single_traversal_matches_oracle_exactly(actions, nodes, depth, cpuct, c
 
 @pytest.mark.parametrize("trees,warps,soft", [(16, 8, 0), (16, 16, 0), (4, 40, 0), (16, 16, 1), (128, 4, 0)])
 def test_concurrent_traversals_keep_invariants(trees, warps, soft):
-    import torch
     rng = np.random.default_rng(trees * 100 + warps)
     case = pc.random_forest(rng, trees=trees, nodes=400, actions=16, warps=warps, path_depth=12)
     n_before, w_before = case["edge_n"].copy(), case["edge_w"].copy()
@@ -111,13 +114,12 @@ def test_concurrent_traversals_keep_invariants(trees, warps, soft):
     added = h2["edge_n"] - n_before
     assert int(added.sum()) == int((h["out_len"][holding] - 1).sum())
     assert np.allclose(h2["edge_w"] - w_before, 0.5 * added, atol=1e-3)
-    torch.cuda.synchronize()
 
 
 def test_node_level_backup_known_answer():
     """src/puct/test_puct_gpu_v2.py:1085-1119 through puct_node_backup_launch."""
-    import torch
     from mcts_numba_cuda_amd import puct
+    from mcts_numba_cuda_amd.hipmem import DeviceArray
     h = pc.make_case(nodes=3, actions=4, path_depth=4)
     h["edge_child"][0, 0, :2] = (1, 2)
     h["edge_n"][0, 0, :2] = 1
@@ -130,8 +132,8 @@ def test_node_level_backup_known_answer():
     values = np.zeros((1, 1, 4), np.float32)
     values[0, 0, 0] = 0.7
     d = to_device(h)
-    puct.launch_node_backup(d, torch.from_numpy(values).cuda())
-    torch.cuda.synchronize()
+    puct.launch_node_backup(d, DeviceArray(values))
+    synchronize()
     g = to_host(d)
     assert int(g["node_inflight"].sum()) == 0 and int(g["node_expand_inflight"].sum()) == 0
     assert g["edge_n"][0, 0, 1] == 2 and g["edge_w"][0, 0, 1] == np.float32(0.7)
@@ -143,16 +145,16 @@ def test_node_level_backup_known_answer():
 
 def test_launch_errors_are_reported():
     from mcts_numba_cuda_amd import puct
-    import torch
+    from mcts_numba_cuda_amd.hipmem import DeviceArray
     case = pc.make_case(nodes=2, actions=4, warps=1, path_depth=2)
     d = to_device(case)
-    d["edge_prior"] = d["edge_prior"].double()
+    d["edge_prior"] = DeviceArray(case["edge_prior"].astype(np.float64))
     with pytest.raises(ValueError):
         puct.launch_select(d)
     d = to_device(case)
-    d["out_selected"] = torch.zeros((1, 0), dtype=torch.int32, device="cuda")
-    d["out_len"] = torch.zeros((1, 0), dtype=torch.int32, device="cuda")
-    d["out_path"] = torch.zeros((1, 0, 2), dtype=torch.int32, device="cuda")
+    d["out_selected"] = DeviceArray(np.zeros((1, 0), np.int32))
+    d["out_len"] = DeviceArray(np.zeros((1, 0), np.int32))
+    d["out_path"] = DeviceArray(np.zeros((1, 0, 2), np.int32))
     with pytest.raises(RuntimeError, match="launch failed"):
         puct.launch_select(d)           # zero traversals: the runtime rejects the empty launch, as CUDA does
     assert isinstance(puct._lib().puct_cpp_cuda_error_string(0), bytes)
