@@ -92,6 +92,150 @@ def algorithmic_bytes(res, tree_steps, acp=True):
     return dict(select=select, expand=expand, playout=playout, backup=backup, total=select + expand + playout + backup)
 
 
+# The reference's large-scale selection benchmark (src/puct/test_puct_gpu_v3.py:2069-2160): name -> (trees, edges per
+# node, path depth); 8 traversals per tree, "wide" recurrent trees (every node has all its edges expanded, edge a leads
+# to node a + 1, equal priors, N = 1, W = 0), no progressive widening, so every selection walks `depth` levels and ends
+# at the depth limit.  Published: 1.63 M / 0.64 M / 0.38 M selections/s (winner_recalc, device unstated).
+PUCT_SHAPES = {"eq64_d512": (16384, 64, 512), "eq128_d1024": (8192, 128, 1024), "eq256_d1024": (4096, 256, 1024)}
+PUCT_TRAVERSALS = 8
+# HBM bytes per selection launch from rocprofv3 --pmc FETCH_SIZE (x2) and WRITE_SIZE (x1), strict claim
+PUCT_TRAFFIC = {"eq256_d1024": int((45596114.7 * 2 + 2509333.3) * 1024)}
+
+
+def puct_wide_case(trees, actions, depth, warps):
+    nodes = actions + 1
+    one = {
+        "edge_child": np.broadcast_to(np.arange(1, actions + 1, dtype=np.int32), (nodes, actions)),
+        "edge_prior": np.ones((nodes, actions), np.float32), "edge_w": np.zeros((nodes, actions), np.float32),
+        "edge_n": np.ones((nodes, actions), np.int32), "edge_inflight": np.zeros((nodes, actions), np.int32),
+    }
+    case = {k: np.ascontiguousarray(np.broadcast_to(v, (trees,) + v.shape)) for k, v in one.items()}
+    case.update({
+        "node_expand_inflight": np.zeros((trees, nodes), np.int32), "node_expanded": np.full((trees, nodes), actions, np.int32),
+        "node_count": np.full((trees,), nodes, np.int32), "out_selected": np.zeros((trees, warps), np.int32),
+        "out_path": np.full((trees, warps, depth), -1, np.int32), "out_len": np.zeros((trees, warps), np.int32)})
+    return case
+
+
+def bench_puct_select(args):
+    """One bench step = one selection launch over all trees (timed with HIP events on the launch stream), followed by
+    an untimed release of the claims, as the reference times it (src/puct/test_puct_gpu_v3.py:632-650)."""
+    from mcts_numba_cuda_amd import puct
+    from mcts_numba_cuda_amd.hipmem import DeviceArray, Event, synchronize
+    trees, actions, depth = PUCT_SHAPES[args.puct_shape]
+    warps = PUCT_TRAVERSALS
+    steps = args.steps if args.steps != N_ROOTS else 10
+    case = puct_wide_case(trees, actions, depth, warps)
+    d = {k: DeviceArray(v) for k, v in case.items()}
+    def timed(soft):
+        for _ in range(max(args.warmup, 1)):
+            puct.launch_select(d, cpuct=1.0, c_pw=0.0, soft_winner=soft)
+            puct.launch_edge_backup(d)
+        synchronize()
+        pairs = []
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            a, b = Event(), Event()
+            a.record()
+            puct.launch_select(d, cpuct=1.0, c_pw=0.0, soft_winner=soft)
+            b.record()
+            sel, lens = d["out_selected"], d["out_len"]
+            puct.launch_edge_backup(d)
+            pairs.append((a, b))
+        synchronize()
+        wall = time.perf_counter() - t0
+        ms = sum(a.elapsed_ms(b) for a, b in pairs)
+        kinds = (sel.numpy() >> 22) & 7
+        lens = lens.numpy()
+        # a traversal either reaches the depth limit or gives up busy (the reference's criterion: some valid
+        # selections, full-length paths, nothing left in flight after the release;
+        # src/puct/test_puct_gpu_v3.py:2141-2150)
+        ok = bool(np.all((kinds == 3) | (kinds == 4)) and lens.max() == depth + 1 and np.all(lens[kinds == 3] == depth + 1)
+                  and not d["edge_inflight"].numpy().any())
+        return ms, wall, ok, float((kinds == 4).mean())
+
+    ms, wall, ok, busy_share = timed(0)
+    ms_soft, _, ok_soft, busy_soft = timed(1)
+    selections = steps * trees * warps
+    # per level: node word, ticket counter, and N / W / prior / child / in-flight of every edge; one path entry.  Exact
+    # for the soft-winner run, in which every traversal walks all `depth` levels; with the strict claim a busy traversal
+    # stops early, so only the completed ones are counted.
+    level_bytes = 8 + 20 * actions + 4
+    alg_bytes = int(trees * warps * (1.0 - busy_share)) * depth * level_bytes
+    alg_bytes_soft = trees * warps * depth * level_bytes
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import puct_oracle as po
+        sample = 64
+        h = {k: np.ascontiguousarray(v[:sample]) for k, v in case.items()}
+        t1 = time.perf_counter()
+        po.select(h, cpuct=1.0, c_pw=0.0)
+        dt = time.perf_counter() - t1
+        cpu = {"value": sample * warps / dt, "unit": "selections/s", "cores": 1, "kind": "port",
+               "sample": f"first {sample} trees of the same workload, one launch ({sample * warps} selections of {depth} levels), "
+                         "sequential CPU oracle"}
+    out = {"metric": "PUCT selections/s, deep-wide select benchmark of the reference (winner_recalc, 8 traversals per tree)",
+           "value": selections / (ms * 1e-3), "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+           "ms_per_step": ms / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 scores + int32 atomics",
+           "data": "synthetic",
+           "config": {"workload": f"{args.puct_shape}: {trees} trees x {warps} traversals, {actions} edges per node, depth {depth}, "
+                                  "equal priors, c_pw=0, terminal by depth limit; one puct_select_winner_recalc_launch per step"},
+           "valid": ok and ok_soft, "busy_share_last_launch": busy_share, "wall_s_incl_release": wall,
+           "soft_winner": {"value": selections / (ms_soft * 1e-3), "unit": "selections/s", "ms_per_step": ms_soft / steps,
+                           "busy_share_last_launch": busy_soft, "levels_per_s": selections * depth / (ms_soft * 1e-3),
+                           "algorithmic_GB_per_s": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9,
+                           "hbm_frac": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9 / HBM_PEAK_GBS},
+           "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms / steps * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": alg_bytes / (ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": PUCT_TRAFFIC.get(args.puct_shape),
+                        "kernel": "select_kernel", "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": ms / steps},
+           "cpu_baseline": cpu}
+    print(json.dumps(out))
+
+
+def bench_puct_gomoku(args):
+    """BASELINE configs[4]: PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step,
+    Dirichlet(0.3) priors and hashed values, c_puct = 1.5, 4000 steps; one bench step = one whole search."""
+    from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
+    steps = args.steps if args.steps != N_ROOTS else 5
+    search_steps = 4000
+    board = np.zeros((15, 15), np.int8)
+    e = PUCTGomoku(trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0, alpha_pw=0.5,
+                   recalc_attempts=16, dirichlet_alpha=0.3, seed=0)
+    for _ in range(max(args.warmup, 1)):
+        e.run(board, 1, 200)
+    sel = useful = nodes = 0
+    dev = 0.0
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        e.run(board, 1, search_steps)
+        sel += e.performance_info["selections"]
+        useful += e.performance_info["selections"] - e.selections["busy"]
+        nodes += e.performance_info["nodes_total"]
+        dev += e.result.time_device
+    wall = time.perf_counter() - t0
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import puct_oracle as po
+        t1 = time.perf_counter()
+        h = po.gomoku_search(board, 1, 250, trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0,
+                             dirichlet_alpha=0.3, seed=0)
+        dt = time.perf_counter() - t1
+        cpu = {"value": 250 * 256 / dt, "unit": "selections/s", "cores": 1, "kind": "port",
+               "sample": "the same search for 250 steps (64000 selections), sequential CPU oracle",
+               "selections_not_busy_per_s": int(h["tally"][:, 1:4].sum()) / dt}
+    out = {"metric": "PUCT selections/s, Gomoku 15x15 search loop with virtual loss (16 trees x 16 traversals)",
+           "value": sel / wall, "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+           "ms_per_step": wall / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32 scores + int32 atomics", "data": "synthetic",
+           "config": {"workload": "Gomoku 15x15 empty board, 16 trees x 16 traversals per step, Dirichlet(0.3) priors and hashed "
+                                  "values, c_puct=1.5, c_pw=1.0, alpha_pw=0.5, 16 claim attempts, 4000 steps per search, "
+                                  "node limit 16384 per tree"},
+           "search_steps_per_s": steps * search_steps / wall, "selections_not_busy_per_s": useful / wall,
+           "nodes_created_per_search": nodes / steps, "device_share": dev / wall, "roofline": None, "cpu_baseline": cpu}
+    e.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,6 +246,10 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by) and exit")
+    ap.add_argument("--workload", default="c4", choices=("c4", "puct_select", "puct_gomoku"),
+                    help="c4: the headline MCTS-NC search (default); puct_select: the reference's deep-wide PUCT selection "
+                         "benchmark through puct_select_winner_recalc_launch; puct_gomoku: the Gomoku PUCT search loop")
+    ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (trees are independent and would shard over GPUs with one "
@@ -116,6 +264,11 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "copies": 4}))
         return
+
+    if args.workload == "puct_select":
+        return bench_puct_select(args)
+    if args.workload == "puct_gomoku":
+        return bench_puct_gomoku(args)
 
     import contextlib
     import io

@@ -20,6 +20,10 @@ def hip():
         _hip.hipFree.argtypes = [vp]
         _hip.hipMemcpy.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int]
         _hip.hipMemset.argtypes = [vp, ctypes.c_int, ctypes.c_size_t]
+        _hip.hipEventCreate.argtypes = [ctypes.POINTER(vp)]
+        _hip.hipEventRecord.argtypes = [vp, vp]
+        _hip.hipEventDestroy.argtypes = [vp]
+        _hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), vp, vp]
         _hip.hipGetErrorString.restype = ctypes.c_char_p
         _hip.hipGetErrorString.argtypes = [ctypes.c_int]
     return _hip
@@ -72,5 +76,29 @@ class DeviceArray:
     def __del__(self):
         try:
             self.free()
+        except Exception:
+            pass
+
+
+class Event:
+    """A HIP event on the default stream (timing of the launches made through the C ABIs with a NULL stream)."""
+
+    def __init__(self):
+        self._ev = ctypes.c_void_p()
+        check(hip().hipEventCreate(ctypes.byref(self._ev)), "hipEventCreate")
+
+    def record(self):
+        check(hip().hipEventRecord(self._ev, ctypes.c_void_p(0)), "hipEventRecord")
+
+    def elapsed_ms(self, later):
+        """Milliseconds from this event to `later` (both must have completed)."""
+        ms = ctypes.c_float()
+        check(hip().hipEventElapsedTime(ctypes.byref(ms), self._ev, later._ev), "hipEventElapsedTime")
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self._ev:
+                hip().hipEventDestroy(self._ev)
         except Exception:
             pass
