@@ -366,6 +366,23 @@ def main():
                         "sample": f"first {n_sample_roots} roots of the workload, {sample_steps} MCTS steps each ({cpu_playouts} playouts), "
                                   "CPU oracle (scalar restatement of the reference's kernels) with OpenMP over playouts"}
 
+    cpu_mcts = None
+    if not args.no_cpu_baseline:
+        # the reference's own CPU player (src/mcts.py, mirrored in mcts_numba_cuda_amd/mcts.py): one playout per step,
+        # single-threaded, on the first root of the workload for two seconds
+        from mcts_numba_cuda_amd.c4 import C4
+        from mcts_numba_cuda_amd.mcts import MCTS
+        state = C4()
+        b0, f0, t0_ = roots[0]
+        state.board[:], state.column_fills[:], state.turn = b0, f0, t0_
+        with contextlib.redirect_stdout(quiet):
+            cpu_ai = MCTS(search_time_limit=2.0, search_steps_limit=np.inf, vanilla=True, ucb_c=2.0, seed=0)
+            cpu_ai.run(state)
+        cpu_mcts = {"playouts_per_s": cpu_ai.performance_info["playouts_per_second"],
+                    "steps_per_s": cpu_ai.performance_info["steps_per_second"], "cores": 1,
+                    "kind": "host mirror of the reference's CPU MCTS (pure Python, no numba)",
+                    "sample": "first root of the workload, 2 s time limit"}
+
     out = {"metric": "playouts/s + steps/s, C4 6x7 ACP-prodigal 4x256 on 1 MI355X; % of roofline",
            "value": value, "unit": "playouts/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -377,7 +394,7 @@ def main():
            "device_loop_share": dev_time / elapsed,
            "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
            "batched": batched,
-           "roofline": roofline, "cpu_baseline": cpu_baseline}
+           "roofline": roofline, "cpu_baseline": cpu_baseline, "cpu_mcts": cpu_mcts}
     print(json.dumps(out))
 
 
