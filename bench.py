@@ -192,6 +192,63 @@ def bench_puct_select(args):
     print(json.dumps(out))
 
 
+def bench_gomoku(args):
+    """BASELINE configs[3]: Gomoku 15x15, 32 seeded roots with 0..20 stones placed alternately on random cells,
+    ocp_thrifty, n_trees=4, n_playouts=128, 2000 steps, device_memory=16 GiB; one bench step = one search."""
+    import contextlib
+    import io
+    from mcts_numba_cuda_amd import MCTSNC
+    rng = np.random.Generator(np.random.PCG64(0))
+    roots = []
+    for _ in range(32):
+        board = np.zeros((15, 15), np.int8)
+        turn = 1
+        for c in rng.permutation(225)[:int(rng.integers(0, 21))]:
+            board[c // 15, c % 15] = turn
+            turn = -turn
+        roots.append((board, turn))
+    steps = min(args.steps, len(roots)) if args.steps != N_ROOTS else 8
+    quiet = io.StringIO()
+    with contextlib.redirect_stdout(quiet):
+        e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=2000, n_trees=4, n_playouts=128,
+                   variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
+        e.init_device_side_arrays()
+        for w in range(max(args.warmup, 1)):
+            e.reseed()
+            e.run(roots[w][0], None, roots[w][1])
+        playouts = mcts_steps = plies = 0
+        dev = 0.0
+        t0 = time.perf_counter()
+        for k in range(steps):
+            e.reseed()
+            e.run(roots[k][0], None, roots[k][1])
+            playouts += e.performance_info["playouts"]
+            mcts_steps += e.steps
+            plies += e.performance_info["playout_plies"]
+            dev += e.time_device_loop
+        wall = time.perf_counter() - t0
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle.oracle import Oracle
+        cores = min(16, os.cpu_count() or 1)
+        o = Oracle("gomoku", (15, 15), 0, 225, 4, 128, "ocp_thrifty", ucb_c=2.0, seed=0, device_memory=16.0, threads=cores)
+        t1 = time.perf_counter()
+        o.run(roots[0][0], None, roots[0][1], 300)
+        dt = time.perf_counter() - t1
+        cpu = {"value": int(o.result("root_ns").max()) / dt, "unit": "playouts/s", "cores": cores, "kind": "port",
+               "mcts_steps_per_s": 300 / dt, "sample": "first root, 300 MCTS steps, CPU oracle with OpenMP over playouts"}
+    out = {"metric": "playouts/s + steps/s, Gomoku 15x15 OCP-thrifty 4x128 on 1 MI355X", "value": playouts / wall,
+           "unit": "playouts/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1), "ms_per_step": wall / steps * 1e3,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bit boards + int32 counters (UCB in f64 rounded to f32)",
+           "data": "synthetic",
+           "config": {"workload": "Gomoku 15x15, seeded roots with 0-20 random stones, ocp_thrifty n_trees=4 n_playouts=128 ucb_c=2.0 "
+                                  "search_steps_limit=2000 device_memory=16GiB seed=0; one MCTSNC.run() per root, sequential"},
+           "mcts_steps_per_s": mcts_steps / wall, "playout_plies_per_s": plies / dev, "device_loop_share": dev / wall,
+           "roofline": None, "cpu_baseline": cpu}
+    e._release()
+    print(json.dumps(out))
+
+
 def bench_puct_gomoku(args):
     """BASELINE configs[4]: PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step,
     Dirichlet(0.3) priors and hashed values, c_puct = 1.5, 4000 steps; one bench step = one whole search."""
@@ -246,7 +303,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by) and exit")
-    ap.add_argument("--workload", default="c4", choices=("c4", "puct_select", "puct_gomoku"),
+    ap.add_argument("--workload", default="c4", choices=("c4", "gomoku", "puct_select", "puct_gomoku"),
                     help="c4: the headline MCTS-NC search (default); puct_select: the reference's deep-wide PUCT selection "
                          "benchmark through puct_select_winner_recalc_launch; puct_gomoku: the Gomoku PUCT search loop")
     ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
@@ -265,6 +322,8 @@ def main():
         print(json.dumps({"copy_calibration_bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "copies": 4}))
         return
 
+    if args.workload == "gomoku":
+        return bench_gomoku(args)
     if args.workload == "puct_select":
         return bench_puct_select(args)
     if args.workload == "puct_gomoku":

@@ -206,9 +206,11 @@ __global__ void reset_kernel(const TreeRef *refs, int n_refs, const uint32_t *ro
     h->arrive = 0; h->gen = 0;
 }
 
-// Dynamic LDS layout of the search kernel (bytes): per-thread legal lists and line words.
+// Dynamic LDS layout of the search kernel (bytes): per thread a legal list (one byte per cell, four cells per
+// dword) and one dword per board line (low half: stones of +1, high half: stones of -1); dword k of thread t sits at
+// index k * threads + t, so the lanes of a wavefront never share a bank whatever cells they touch.
 __host__ __device__ inline size_t playout_lds_bytes(int cells, int lines, int threads) {
-    return (size_t)cells * threads + (size_t)2 * lines * threads * sizeof(uint16_t);
+    return ((size_t)((cells + 3) / 4) + (size_t)lines) * sizeof(uint32_t) * threads;
 }
 
 template <bool ACP>
@@ -227,23 +229,23 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
     const int n_lines = 3 * (m + n) - 2;
 
     extern __shared__ unsigned char s_dyn[];
-    uint8_t *const s_list = s_dyn;                                                       // [cells][nthreads]
-    uint16_t *const s_lines = reinterpret_cast<uint16_t *>(s_dyn + (size_t)cells * nthreads);  // [2][n_lines][nthreads]
+    const int list_dwords = (cells + 3) >> 2;
+    uint32_t *const s_list = reinterpret_cast<uint32_t *>(s_dyn);      // [list_dwords][nthreads]
+    uint32_t *const s_lines = s_list + (size_t)list_dwords * nthreads;  // [n_lines][nthreads]
+    const uint32_t div_n = 65536u / (uint32_t)n + 1u;                   // (a * div_n) >> 16 == a / n for a < 1024, n <= 32
 
     __shared__ int32_t s_path[kMaxPath];
     __shared__ LeafInfo s_leaf;
     __shared__ uint32_t s_bb[16];             // board of the selected node: [0..7] +1 stones, [8..15] -1 stones
     __shared__ uint32_t s_cbb[16];            // board of the child being played out
     __shared__ int16_t s_actions[kMaxCells];  // ordinal -> action of the selected node's expandable children
-    __shared__ uint8_t s_tmpl[kMaxCells];     // legal list template of the child being played out
-    __shared__ uint16_t s_ltmpl[2][kMaxLines];
-    __shared__ uint16_t s_cell[kMaxCells];    // cell -> row | column << 8
+    __shared__ uint32_t s_tmpl[kMaxCells / 4];  // legal list template of the child being played out (bytes)
+    __shared__ uint32_t s_ltmpl[kMaxLines];     // line words of both players (low / high half)
     __shared__ int32_t s_red[4][2];
     __shared__ unsigned long long s_key[4];
     __shared__ int32_t s_flag, s_chosen, s_abort, s_redo, s_tot[2], s_count;
     __shared__ ExactScratch s_exact;
 
-    for (int c = tid; c < cells; c += nthreads) s_cell[c] = (uint16_t)((c / n) | ((c % n) << 8));
     if (tid == 0) s_abort = 0;
     uint64_t e0 = 0, e1 = 0;
     if (!ACP && tid == 0) { e0 = ref.rng_expand[0]; e1 = ref.rng_expand[1]; }
@@ -368,26 +370,35 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                 // templates: board, legal list in row-major order, line words of both players
                 if (tid < 16) s_cbb[tid] = (tid < 8) ? pn->bb_pos[tid] : pn->bb_neg[tid - 8];
                 __syncthreads();
-                if (tid == 0) {
+                if (wave == 0) {  // empty cells in row-major order, compacted with ballots
+                    uint8_t *tm = reinterpret_cast<uint8_t *>(s_tmpl);
                     int cnt = 0;
-                    for (int c = 0; c < cells; c++)
-                        if (!bb_test(s_cbb, c) && !bb_test(s_cbb + 8, c)) s_tmpl[cnt++] = (uint8_t)c;
-                    s_count = cnt;
-                }
-                for (int idx = tid; idx < 2 * n_lines; idx += nthreads) {
-                    const int p = idx / n_lines, ln = idx - p * n_lines;
-                    const uint32_t *bb = s_cbb + 8 * p;
-                    uint32_t v = 0;
-                    if (ln < m) { for (int jj = 0; jj < n; jj++) v |= (uint32_t)bb_test(bb, ln * n + jj) << jj; }
-                    else if (ln < m + n) { const int jj = ln - m; for (int ii = 0; ii < m; ii++) v |= (uint32_t)bb_test(bb, ii * n + jj) << ii; }
-                    else if (ln < m + n + (m + n - 1)) {
-                        const int d = ln - (m + n);  // d = i - j + (n - 1)
-                        for (int jj = 0; jj < n; jj++) { const int ii = d + jj - (n - 1); if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
-                    } else {
-                        const int e = ln - (m + n) - (m + n - 1);  // e = i + j
-                        for (int jj = 0; jj < n; jj++) { const int ii = e - jj; if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
+                    for (int base = 0; base < cells; base += 64) {
+                        const int c = base + lane;
+                        const bool empty = c < cells && !bb_test(s_cbb, c) && !bb_test(s_cbb + 8, c);
+                        const unsigned long long mask = __ballot(empty);
+                        if (empty) tm[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (uint8_t)c;
+                        cnt += __popcll(mask);
                     }
-                    s_ltmpl[p][ln] = (uint16_t)v;
+                    if (lane == 0) s_count = cnt;
+                }
+                for (int ln = tid; ln < n_lines; ln += nthreads) {
+                    uint32_t word = 0;
+                    for (int p = 0; p < 2; p++) {
+                        const uint32_t *bb = s_cbb + 8 * p;
+                        uint32_t v = 0;
+                        if (ln < m) { for (int jj = 0; jj < n; jj++) v |= (uint32_t)bb_test(bb, ln * n + jj) << jj; }
+                        else if (ln < m + n) { const int jj = ln - m; for (int ii = 0; ii < m; ii++) v |= (uint32_t)bb_test(bb, ii * n + jj) << ii; }
+                        else if (ln < m + n + (m + n - 1)) {
+                            const int d = ln - (m + n);  // d = i - j + (n - 1)
+                            for (int jj = 0; jj < n; jj++) { const int ii = d + jj - (n - 1); if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
+                        } else {
+                            const int e = ln - (m + n) - (m + n - 1);  // e = i + j
+                            for (int jj = 0; jj < n; jj++) { const int ii = e - jj; if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
+                        }
+                        word |= v << (16 * p);
+                    }
+                    s_ltmpl[ln] = word;
                 }
                 __syncthreads();
                 const int count0 = s_count;
@@ -400,28 +411,38 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                     if (t < P) {
                         s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1];
                         s0_start = s0; s1_start = s1;
-                        for (int i = 0; i < count0; i++) s_list[i * nthreads + tid] = s_tmpl[i];
-                        for (int i = 0; i < n_lines; i++) { s_lines[i * nthreads + tid] = s_ltmpl[0][i]; s_lines[(n_lines + i) * nthreads + tid] = s_ltmpl[1][i]; }
+                        {
+                            const int used = (count0 + 3) >> 2;
+#pragma unroll 8
+                            for (int k = 0; k < used; k++) s_list[k * nthreads + tid] = s_tmpl[k];
+#pragma unroll 8
+                            for (int k = 0; k < n_lines; k++) s_lines[k * nthreads + tid] = s_ltmpl[k];
+                        }
+                        uint8_t *const lb = reinterpret_cast<uint8_t *>(s_list + tid);   // byte i: lb[(i >> 2) * stride4 + (i & 3)]
+                        uint32_t *const lp = s_lines + tid;
+                        const int stride4 = nthreads << 2;
                         int count = count0, turn = pturn, status = count0 == 0 ? 2 : 0;
                         while (status == 0) {
                             const uint64_t x = rng_next(s0, s1);
                             const float u = uniform_from_bits((uint32_t)x, (uint32_t)(x >> 32));
                             const int ord = (int)(u * (float)count);  // single-precision product (src/mctsnc.py:1882)
                             if (ord >= count) { status = 3; break; }
-                            const int a = s_list[ord * nthreads + tid];
-                            s_list[ord * nthreads + tid] = s_list[(count - 1) * nthreads + tid];  // swap-remove (:209-217)
                             count--;
+                            uint8_t *const slot = lb + (ord >> 2) * stride4 + (ord & 3);
+                            const int a = *slot;
+                            *slot = lb[(count >> 2) * stride4 + (count & 3)];  // swap-remove (:209-217)
                             plies++;
-                            const uint32_t ij = s_cell[a];
-                            const int i = (int)(ij & 0xffu), jj = (int)(ij >> 8);
-                            uint16_t *ln = s_lines + (size_t)(turn == 1 ? 0 : n_lines) * nthreads + tid;
-                            const int l_row = i, l_col = m + jj, l_dia = m + n + (i - jj + n - 1), l_ant = m + n + (m + n - 1) + (i + jj);
-                            uint32_t v;
-                            bool win = false;
-                            v = ln[l_row * nthreads] | (1u << jj); ln[l_row * nthreads] = (uint16_t)v; win |= line_neighbours(v, jj) == 4;
-                            v = ln[l_col * nthreads] | (1u << i);  ln[l_col * nthreads] = (uint16_t)v; win |= line_neighbours(v, i) == 4;
-                            v = ln[l_dia * nthreads] | (1u << jj); ln[l_dia * nthreads] = (uint16_t)v; win |= line_neighbours(v, jj) == 4;
-                            v = ln[l_ant * nthreads] | (1u << jj); ln[l_ant * nthreads] = (uint16_t)v; win |= line_neighbours(v, jj) == 4;
+                            const int i = (int)(((uint32_t)a * div_n) >> 16), jj = a - i * n;
+                            const int sh = turn == 1 ? 0 : 16;
+                            uint32_t *const p_row = lp + i * nthreads, *const p_col = lp + (m + jj) * nthreads;
+                            uint32_t *const p_dia = lp + (m + n + (i - jj + n - 1)) * nthreads;
+                            uint32_t *const p_ant = lp + (m + n + (m + n - 1) + (i + jj)) * nthreads;
+                            // the four lines through a cell are four different words: read all, then write all
+                            uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
+                            w_row |= (1u << jj) << sh; w_col |= (1u << i) << sh; w_dia |= (1u << jj) << sh; w_ant |= (1u << jj) << sh;
+                            *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
+                            const bool win = (line_neighbours((w_row >> sh) & 0xffffu, jj) == 4) | (line_neighbours((w_col >> sh) & 0xffffu, i) == 4) |
+                                             (line_neighbours((w_dia >> sh) & 0xffffu, jj) == 4) | (line_neighbours((w_ant >> sh) & 0xffffu, jj) == 4);
                             if (win) { status = 1; outcome = turn; }
                             else if (count == 0) { status = 2; outcome = 0; }
                             turn = -turn;
