@@ -367,6 +367,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
     __shared__ int32_t s_poc[kMaxCols][2];
     __shared__ int16_t s_ae[16], s_root_ae[16];
     __shared__ int32_t s_chosen, s_abort, s_redo;
+    __shared__ double s_explore[kMaxPath][8];   // c * sqrt(log(N) / n) of every child of every path node after this step
     __shared__ uint8_t s_nth[256 * 8];
     __shared__ ExactScratch s_exact;
 
@@ -554,6 +555,27 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_playout += t2 - tk; tk = t2; }
         st_levels += L; st_expanded += k_exp; st_played += do_playouts ? 1 : 0;
 
+        // ---- exploration terms of the path nodes' children after this step ----
+        // The visit counts after the backup are known before the playout results of the other workgroups arrive (the
+        // wins are not), so the expensive part of every UCB that has to be re-evaluated is computed here, by the
+        // wavefronts that do not take part in the exchange.
+        const int n_tot_known = (ACP && mode == kModeExpand) ? P * k_exp : P;
+        const int n_levels = (mode == kModeExpand) ? L + 1 : L;
+        {
+            const int first = (nwaves > 1) ? kWave : 0, workers = blockDim.x - first;
+            if (tid >= first) {
+                for (int i = tid - first; i < n_levels * 8; i += workers) {
+                    const int lvl = i >> 3, a = i & 7;
+                    int n;
+                    if (lvl == L) n = ACP ? (((expmask >> a) & 1u) ? P : 0) : ((a == chosen) ? P : 0);
+                    else n = (int)s_rec[lvl][kDwNs + a] + ((a == (int)s_pslot[lvl + 1]) ? n_tot_known : 0);
+                    const int N = ((lvl == 0) ? s_t.root_ns : (int)s_rec[lvl - 1][kDwNs + s_pslot[lvl]]) + n_tot_known;
+                    s_explore[lvl][a] = (n > 0) ? (double)args.ucb_c * __dsqrt_rn(det_log((double)N) / (double)n) : 0.0;
+                }
+            }
+            if (!ACP) __syncthreads();   // all-children-playouts workgroups meet at the barrier that ends the exchange
+        }
+
         // ================= exchange of the playout results between the workgroups of the tree =================
         // Every workgroup publishes (step tag, -1 wins, +1 wins) in its own slot of a double-buffered line and then
         // reads all slots of the step: one hand-off per step.  Because every workgroup publishes every step, none can
@@ -663,22 +685,18 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
                     s_ae[A] = tag;
                 }
             }
-        }
-        __syncthreads();
-        if (ACP && tid == 0 && mode != kModeExpand) s_ae[0] = 0;
-        // ---- best-child slots of the path nodes, all levels in parallel (8 lanes per level) ----
-        {
-            const int n_levels = (mode == kModeExpand) ? L + 1 : L;
-            for (int base_i = 0; base_i < n_levels * 8; base_i += blockDim.x) {
-                const int i = base_i + tid;
-                const int lvl = i >> 3, a = i & 7;
+            if (ACP && lane == 0 && mode != kModeExpand) s_ae[0] = 0;
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");   // the backed-up counters, for the other lanes
+            // ---- best-child slots of the path nodes, eight levels at a time (8 lanes per level): the win ratio of the
+            // backed-up counters plus the exploration term prepared before the exchange, narrowed as in ucb_value() ----
+            for (int base = 0; base < n_levels; base += 8) {
+                const int lvl = base + (lane >> 3), a = lane & 7;
                 unsigned long long key = 0;
                 if (lvl < n_levels) {
                     const uint32_t mask = s_rec[lvl][kDwMask] & 0xffu;
                     if ((mask >> a) & 1u) {
                         const int n = (int)s_rec[lvl][kDwNs + a], wins = (int)s_rec[lvl][kDwWins + a];
-                        const int N = (lvl == 0) ? s_t.root_ns : (int)s_rec[lvl - 1][kDwNs + s_pslot[lvl]];
-                        const float ucb = (n == 0) ? __builtin_inff() : ucb_value(wins, n, det_log((double)N), args.ucb_c);
+                        const float ucb = (n == 0) ? __builtin_inff() : (float)((double)wins / (double)(float)n + s_explore[lvl][a]);
                         key = (((unsigned long long)__float_as_uint(ucb) + 1ull) << 8) | (unsigned long long)(7u - bitrev3((uint32_t)a));
                     }
                 }
@@ -691,11 +709,9 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
                     s_rec[lvl][kDwMask] = (s_rec[lvl][kDwMask] & 0x00ffffffu) | (best << 24);
                 }
             }
-        }
-        __syncthreads();
-        if (gen == 0 && tid < 16) s_root_ae[tid] = s_ae[tid];  // _memorize_root_actions_expanded (:1683-1688)
-        // ---- write the path records back: level l by workgroup l % G, one 128-byte store per record ----
-        if (wave == 0) {
+            if (gen == 0 && lane < 16) s_root_ae[lane] = s_ae[lane];  // _memorize_root_actions_expanded (:1683-1688)
+            __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+            // ---- write the path records back: level l by workgroup l % G, one 128-byte store per record ----
             for (int l0 = ACP ? g : 0; l0 <= L; l0 += 2 * (ACP ? G : 1)) {
                 const int lvl = l0 + ((lane >= 32) ? (ACP ? G : 1) : 0);
                 if (lvl <= L) reinterpret_cast<uint32_t *>(nodes + s_pnode[lvl])[lane & 31] = s_rec[lvl][lane & 31];
