@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MCTS-NC search hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): Connect 4 6x7, 64 seeded roots each reached by 10..20 uniform-random legal
+Workload (the headline configuration): Connect 4 6x7, 64 seeded roots each reached by 10..20 uniform-random legal
 plies (non-terminal), acp_prodigal, n_trees=4, n_playouts=256, ucb_c=2.0, search_steps_limit=5000,
 device_memory=2 GiB, seed 0, random streams restarted for every root.
 
@@ -193,7 +193,7 @@ def bench_puct_select(args):
 
 
 def bench_gomoku(args):
-    """BASELINE configs[3]: Gomoku 15x15, 32 seeded roots with 0..20 stones placed alternately on random cells,
+    """Gomoku 15x15, 32 seeded roots with 0..20 stones placed alternately on random cells,
     ocp_thrifty, n_trees=4, n_playouts=128, 2000 steps, device_memory=16 GiB; one bench step = one search."""
     import contextlib
     import io
@@ -250,7 +250,7 @@ def bench_gomoku(args):
 
 
 def bench_puct_gomoku(args):
-    """BASELINE configs[4]: PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step,
+    """PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step,
     Dirichlet(0.3) priors and hashed values, c_puct = 1.5, 4000 steps; one bench step = one whole search."""
     from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
     steps = args.steps if args.steps != N_ROOTS else 5

@@ -64,84 +64,8 @@ def condense_dump(path, out):
     np.savez_compressed(out, **arrays)
 
 
-_INSTANCE_RE = re.compile(r"MCTSNC\(search_time_limit=([^,]+), search_steps_limit=([^,]+), n_trees=(\d+), n_playouts=(\d+), "
-                          r"variant='(\w+)', device_memory=([^,]+), ucb_c=([^,]+), seed: (\d+)\)")
-
-
-def parse_instance(s):
-    m = _INSTANCE_RE.search(s)
-    if not m:
-        return None
-    return dict(n_trees=int(m.group(3)), n_playouts=int(m.group(4)), variant=m.group(5), device_memory=float(m.group(6)),
-                ucb_c=float(m.group(7)), seed=int(m.group(8)))
-
-
-def parse_block(lines, i):
-    """Parses a '{' ... '}]' block printed by utils.dict_to_str starting at lines[i] == '{'; returns (dict, next_i)."""
-    assert lines[i].strip() == "{", lines[i]
-    out = {}
-    i += 1
-    while not lines[i].startswith("}"):
-        line = lines[i].strip().rstrip(",")
-        key, _, val = line.partition(": ")
-        val = re.sub(r"np\.(?:float|int)\d+\(([^()]*)\)", r"\1", val)  # newer numpy reprs in some logs
-        val = re.sub(r"\b(nan|inf)\b", r"None", val)
-        try:
-            out[key] = ast.literal_eval(val)
-        except (ValueError, SyntaxError):
-            out[key] = val
-        i += 1
-    return out, i + 1
-
-
-def parse_log(log, n_games):
-    lines = log.split("\n")
-    games = []
-    i = 0
-    cur = None
-    while i < len(lines):
-        ln = lines[i]
-        if ln.startswith("MCTS-NC EXPERIMENT..."):  # an interrupted experiment restarted in the same log
-            games, cur = [], None
-        m = re.match(r"GAME (\d+)/(\d+):", ln)
-        if m:
-            if int(m.group(1)) > n_games:
-                break
-            cur = {"black": lines[i + 1][len("BLACK: "):], "white": lines[i + 2][len("WHITE: "):], "events": []}
-            games.append(cur)
-            ply = 0
-            i += 3
-            continue
-        if cur is not None and (ln.startswith("MCTSNC RUN...") or ln.startswith("MCTS RUN...")):
-            kind = "mctsnc" if ln.startswith("MCTSNC") else "mcts"
-            if not lines[i + 1].startswith("[actions info:"):  # search cut off by an interruption
-                i += 1
-                continue
-            actions, j = parse_block(lines, i + 2)
-            assert lines[j].startswith("[performance info:"), lines[j]
-            perf, j = parse_block(lines, j + 1)
-            ev = {"type": kind, "side": "black" if ply % 2 == 0 else "white", "steps": perf["steps"], "playouts": perf["playouts"]}
-            best = actions.pop("best")
-            ev["best"] = best["index"]
-            ev["actions"] = {str(k): [v["n"], v["n_wins"], int(v["win_flag"])] for k, v in actions.items()}
-            ev["n_root"] = best["n_root"]
-            tr = perf.get("trees") or perf.get("tree")
-            if kind == "mctsnc":
-                ev["trees"] = {k: tr[k] for k in ["mean_depth", "max_depth", "mean_size", "max_size"]}
-            else:
-                ev["tree"] = {k: tr[k] for k in ["n_root", "mean_depth", "max_depth", "size"]}
-            cur["events"].append(ev)
-            i = j
-            continue
-        m = re.match(r"MOVE PLAYED: (\d+)", ln)
-        if m and cur is not None:
-            cur["events"].append({"type": "move", "action": int(m.group(1))})
-            ply += 1
-        m = re.match(r"GAME OUTCOME: (.*)", ln)
-        if m and cur is not None:
-            cur["outcome"] = m.group(1)
-        i += 1
-    return games
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+from mcts_numba_cuda_amd.archive import parse_instance, parse_log  # noqa: E402  (the log parser lives with the replay tool)
 
 
 def condense_archives(ref_root, out):

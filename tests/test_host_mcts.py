@@ -99,3 +99,37 @@ def test_host_states_drive_the_gpu_engine():
             if state.compute_outcome() is not None:
                 break
     assert int(np.abs(state.board).sum()) >= 6 or state.compute_outcome() is not None
+
+
+def test_archive_log_parser_reads_the_runner_format():
+    """A log fragment in the format the reference's runner prints (src/game_runner.py, src/mctsnc.py:1255-1257,
+    src/utils.py:23-30), with a numpy-2 style scalar repr as some archives have."""
+    from mcts_numba_cuda_amd.archive import parse_instance, parse_log
+    inst = "MCTSNC(search_time_limit=5.0, search_steps_limit=inf, n_trees=4, n_playouts=256, variant='acp_prodigal', device_memory=2.0, ucb_c=2.0, seed: 0)"
+    assert parse_instance(inst) == dict(n_trees=4, n_playouts=256, variant="acp_prodigal", device_memory=2.0, ucb_c=2.0, seed=0)
+    log = "\n".join([
+        "GAME 1/100:", "BLACK: " + inst, "WHITE: MCTS(search_time_limit=5.0, search_steps_limit=inf, vanilla=True, ucb_c=2.0, seed: 0)",
+        "MCTSNC RUN... [" + inst + "]", "[actions info:", "{",
+        "  0: {'name': '0', 'n_root': 512, 'win_flag': False, 'n': 256, 'n_wins': 100, 'q': np.float64(0.39), 'ucb': 1.5},",
+        "  3: {'name': '3', 'n_root': 512, 'win_flag': True, 'n': 256, 'n_wins': 256, 'q': 1.0, 'ucb': inf},",
+        "  best: {'index': 3, 'name': '3', 'n_root': 512, 'win_flag': True, 'n': 256, 'n_wins': 256, 'q': 1.0, 'ucb': inf}",
+        "}]", "[performance info:", "{", "  steps: 1,", "  steps_per_second: 10.0,", "  playouts: 512,", "  playouts_per_second: 5120.0,",
+        "  times_[ms]: {'total': 1.0},", "  trees: {'count': 4, 'mean_depth': 0.75, 'max_depth': 1, 'mean_size': 3.0, 'max_size': 3}", "}]",
+        "MCTSNC RUN DONE. [time: 0.1 s; best action: 3]", "MOVE PLAYED: 3", "GAME OUTCOME: BLACK WINS"])
+    games = parse_log(log, 5)
+    assert len(games) == 1 and games[0]["outcome"] == "BLACK WINS"
+    search, move = games[0]["events"]
+    assert search == {"type": "mctsnc", "side": "black", "steps": 1, "playouts": 512, "best": 3, "n_root": 512,
+                      "actions": {"0": [256, 100, 0], "3": [256, 256, 1]},
+                      "trees": {"mean_depth": 0.75, "max_depth": 1, "mean_size": 3.0, "max_size": 3}}
+    assert move == {"type": "move", "action": 3}
+
+
+@pytest.mark.gpu
+def test_archive_replay_tool_reproduces_a_recorded_game(archives):
+    """The replay tool on the fixture of the north-star archive: every MCTSNC search of the first game reproduces the
+    logged root table, best action and tree statistics."""
+    from mcts_numba_cuda_amd import archive
+    entry = archives[find_archive(archives, "mcts_5_inf_vanilla", "mctsnc_5_inf_4_256_acp_prodigal")]
+    checked, failures = archive.replay(entry, max_games=1)
+    assert checked >= 10 and failures == []
