@@ -340,6 +340,19 @@ __device__ __forceinline__ uint32_t child_record_dword(int lane, uint64_t cpos, 
     return v;
 }
 
+// Dynamic LDS of the search kernel: the exploration terms (8 doubles per tree level; the exact replay of a playout
+// uses the same bytes earlier in the step) and the cached path records (the 24 meaningful dwords of a node record per
+// level).  A path has at most m * n + 1 nodes.
+constexpr int kRecDwords = 24;
+__host__ __device__ inline int path_levels(int m, int n) { return m * n + 2; }
+__host__ __device__ inline size_t explore_bytes(int m, int n) {
+    const size_t need = (size_t)path_levels(m, n) * 8 * sizeof(double), exact = (sizeof(ExactScratch) + 7) & ~(size_t)7;
+    return need > exact ? need : exact;
+}
+__host__ __device__ inline size_t search_lds_bytes(int m, int n) {
+    return explore_bytes(m, n) + (size_t)path_levels(m, n) * kRecDwords * sizeof(uint32_t);
+}
+
 template <bool ACP>
 __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
     // XCD-aware decode: consecutive blockIdx values go to different XCDs, so the workgroups of one tree
@@ -357,7 +370,10 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
     const Geometry geo(args.m, args.n);
 
     // the records of the nodes on the last selected path, kept current locally (index = tree level)
-    __shared__ uint32_t s_rec[kMaxPath][32];
+    extern __shared__ double s_dyn[];
+    double (*const s_explore)[8] = reinterpret_cast<double (*)[8]>(s_dyn);
+    ExactScratch &s_exact = *reinterpret_cast<ExactScratch *>(s_dyn);
+    uint32_t (*const s_rec)[kRecDwords] = reinterpret_cast<uint32_t (*)[kRecDwords]>(reinterpret_cast<char *>(s_dyn) + explore_bytes(args.m, args.n));
     __shared__ int32_t s_pnode[kMaxPath];
     __shared__ uint8_t s_pslot[kMaxPath];   // action that leads from level l-1 to level l
     __shared__ TreeLocal s_t;
@@ -367,17 +383,8 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
     __shared__ int32_t s_poc[kMaxCols][2];
     __shared__ int16_t s_ae[16], s_root_ae[16];
     __shared__ int32_t s_chosen, s_abort, s_redo;
-    __shared__ double s_explore[kMaxPath][8];   // c * sqrt(log(N) / n) of every child of every path node after this step
-    __shared__ uint8_t s_nth[256 * 8];
-    __shared__ ExactScratch s_exact;
 
-    // nth_table[mask * 8 + k] = index of the k-th set bit of mask
-    for (int i = tid; i < 256 * 8; i += blockDim.x) {
-        uint32_t mask = (uint32_t)i >> 3; const int k = i & 7;
-        for (int j = 0; j < k; j++) mask &= mask - 1;
-        s_nth[i] = (uint8_t)(mask ? __ffs(mask) - 1 : 0);
-    }
-    if (tid < 32) s_rec[0][tid] = reinterpret_cast<const uint32_t *>(nodes)[tid];
+    if (tid < kRecDwords) s_rec[0][tid] = reinterpret_cast<const uint32_t *>(nodes)[tid];
     if (tid < 16) { s_ae[tid] = hdr->ae[tid]; s_root_ae[tid] = hdr->root_ae[tid]; }
     if (tid < kMaxCols) { s_poc[tid][0] = hdr->poc[tid][0]; s_poc[tid][1] = hdr->poc[tid][1]; }
     if (tid == 0) {
@@ -416,7 +423,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
             if (lane < Lp) follow = (s_rec[lane][kDwMask] >> 24) == (uint32_t)s_pslot[lane + 1];
             const unsigned long long div = __ballot(!follow);
             int d = div ? (int)__ffsll((long long)div) - 1 : Lp;
-            uint32_t w = s_rec[d][lane & 31];
+            uint32_t w = (lane & 31) < kRecDwords ? s_rec[d][lane & 31] : 0u;
             int node = s_pnode[d];
             for (;;) {
                 const uint32_t meta = (uint32_t)__builtin_amdgcn_readlane(w, kDwMask);
@@ -425,7 +432,7 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
                 node = __builtin_amdgcn_readlane(w, kDwBase) + __popc(mask & ((1u << a) - 1u));
                 d++;
                 w = reinterpret_cast<const uint32_t *>(nodes + node)[lane & 31];
-                if (lane < 32) s_rec[d][lane] = w;
+                if (lane < kRecDwords) s_rec[d][lane] = w;
                 if (lane == 0) { s_pnode[d] = node; s_pslot[d] = (uint8_t)a; }
             }
             if (lane == 0) {
@@ -492,7 +499,9 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
                     const float u = rng_uniform(e0, e1);
                     int ord = (int)(int16_t)((double)u * (double)k_exp);
                     if (ord > k_exp - 1) ord = k_exp - 1;
-                    s_chosen = s_nth[expmask * 8 + ord];
+                    uint32_t rest = expmask;   // the ord-th set bit of the mask
+                    for (int j = 0; j < ord; j++) rest &= rest - 1u;
+                    s_chosen = __ffs(rest) - 1;
                 }
                 __syncthreads();
                 chosen = s_chosen;
@@ -714,7 +723,8 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
             // ---- write the path records back: level l by workgroup l % G, one 128-byte store per record ----
             for (int l0 = ACP ? g : 0; l0 <= L; l0 += 2 * (ACP ? G : 1)) {
                 const int lvl = l0 + ((lane >= 32) ? (ACP ? G : 1) : 0);
-                if (lvl <= L) reinterpret_cast<uint32_t *>(nodes + s_pnode[lvl])[lane & 31] = s_rec[lvl][lane & 31];
+                if (lvl <= L)   // the last eight dwords of a record are unused and stay zero
+                    reinterpret_cast<uint32_t *>(nodes + s_pnode[lvl])[lane & 31] = (lane & 31) < kRecDwords ? s_rec[lvl][lane & 31] : 0u;
             }
         }
         gen++;

@@ -412,14 +412,15 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    const size_t lds = c4::search_lds_bytes(c.board_m, c.board_n);
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
         args.nsteps = nsteps;
         if (e0->acp) {
             void *kargs[] = {&args};
-            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, 0, stream));
+            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
         } else {
-            hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, 0, stream, args);
+            hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, lds, stream, args);
             HIP_TRY(hipGetLastError());
         }
         return MCTSNC_OK;
@@ -559,10 +560,12 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
             HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
                                                                  gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
         else
-            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, 0));
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, c4::search_lds_bytes(c.board_m, c.board_n)));
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
         const int64_t max_refs = (int64_t)per_cu * cus / (8 * e0->G) * 8;   // the grid is 8 * G * ceil(refs / 8) workgroups
         group = (int)std::max<int64_t>(1, std::min<int64_t>(n, max_refs / c.n_trees));
+        const int n_groups = (n + group - 1) / group;
+        group = (n + n_groups - 1) / n_groups;   // groups of equal size
     }
     const size_t cells = (size_t)c.board_m * c.board_n;
     for (int start = 0; start < n; start += group) {
