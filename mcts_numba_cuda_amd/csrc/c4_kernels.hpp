@@ -226,20 +226,6 @@ __device__ __forceinline__ bool bb_has_four(BB p, int H) {
     return (r.lo | q.lo | r.hi | q.hi) != 0;
 }
 
-// xoroshiro128+ step on 32-bit halves (the 64-bit shifts of the generic form are slow vector instructions)
-struct Rng32 { uint32_t s0l, s0h, s1l, s1h; };
-
-__device__ __forceinline__ void rng_next32(Rng32 &r, uint32_t &out_lo, uint32_t &out_hi) {
-    const uint64_t sum = (((uint64_t)r.s0h << 32) | r.s0l) + (((uint64_t)r.s1h << 32) | r.s1l);
-    out_lo = (uint32_t)sum; out_hi = (uint32_t)(sum >> 32);
-    const uint32_t tl = r.s1l ^ r.s0l, th = r.s1h ^ r.s0h;
-    // rotl(s0, 55) = rotr(s0, 9); t << 14; rotl(t, 36) = halves swapped, then rotl 4
-    const uint32_t r0l = __builtin_amdgcn_alignbit(r.s0h, r.s0l, 9), r0h = __builtin_amdgcn_alignbit(r.s0l, r.s0h, 9);
-    const uint32_t shl = tl << 14, shh = __builtin_amdgcn_alignbit(th, tl, 18);
-    r.s0l = r0l ^ tl ^ shl; r.s0h = r0h ^ th ^ shh;
-    r.s1l = __builtin_amdgcn_alignbit(th, tl, 28); r.s1h = __builtin_amdgcn_alignbit(tl, th, 28);
-}
-
 // cur: stones of the side to move, opp: the other side's.  Returns -1 / 0 / +1, or 2 when a draw of the
 // uniform rounded up to 1.0f (the caller then replays the playout with exact_playout).  The ply body is free of
 // branches: lanes leave through the loop condition only.

@@ -422,9 +422,12 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                         uint32_t *const lp = s_lines + tid;
                         const int stride4 = nthreads << 2;
                         int count = count0, turn = pturn, status = count0 == 0 ? 2 : 0;
+                        Rng32 rg;
+                        rg.s0l = (uint32_t)s0; rg.s0h = (uint32_t)(s0 >> 32); rg.s1l = (uint32_t)s1; rg.s1h = (uint32_t)(s1 >> 32);
                         while (status == 0) {
-                            const uint64_t x = rng_next(s0, s1);
-                            const float u = uniform_from_bits((uint32_t)x, (uint32_t)(x >> 32));
+                            uint32_t xl, xh;
+                            rng_next32(rg, xl, xh);
+                            const float u = uniform_from_bits(xl, xh);
                             const int ord = (int)(u * (float)count);  // single-precision product (src/mctsnc.py:1882)
                             if (ord >= count) { status = 3; break; }
                             count--;
@@ -447,6 +450,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                             else if (count == 0) { status = 2; outcome = 0; }
                             turn = -turn;
                         }
+                        s0 = ((uint64_t)rg.s0h << 32) | rg.s0l; s1 = ((uint64_t)rg.s1h << 32) | rg.s1l;
                         redo = status == 3;
                     }
                     if (tid == 0) s_redo = 0;
