@@ -340,7 +340,7 @@ __host__ __device__ inline size_t search_lds_bytes(int m, int n) {
 }
 
 template <bool ACP>
-__global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
+__device__ __forceinline__ void search_body(const SearchArgs &args) {
     // XCD-aware decode: consecutive blockIdx values go to different XCDs, so the workgroups of one tree
     // are spaced 8 apart and meet in one L2.
     const int b = blockIdx.x;
@@ -748,6 +748,10 @@ __global__ void __launch_bounds__(512) search_kernel(SearchArgs args) {
         }
     }
 }
+
+template <bool ACP>
+__global__ void __launch_bounds__(512) search_kernel(SearchArgs args) { search_body<ACP>(args); }
+
 
 // Per-tree digest for the final reductions (_reduce_over_trees_*, src/mctsnc.py:2222-2296).
 struct TreeDigest {

@@ -556,16 +556,23 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     int group = n;
     if (e0->acp && n > 1) {
         int per_cu = 0, cus = 0;
-        if (e0->is_gomoku())
+        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
+        auto searches_resident = [&](int blocks_per_cu) {   // the grid is 8 * G * ceil(refs / 8) workgroups
+            return (int)std::max<int64_t>(1, ((int64_t)blocks_per_cu * cus / (8 * e0->G) * 8) / c.n_trees);
+        };
+        if (e0->is_gomoku()) {
             HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
                                                                  gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
-        else
-            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, c4::search_lds_bytes(c.board_m, c.board_n)));
-        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        const int64_t max_refs = (int64_t)per_cu * cus / (8 * e0->G) * 8;   // the grid is 8 * G * ceil(refs / 8) workgroups
-        group = (int)std::max<int64_t>(1, std::min<int64_t>(n, max_refs / c.n_trees));
+            group = searches_resident(per_cu);
+        } else {
+            const size_t lds = c4::search_lds_bytes(c.board_m, c.board_n);
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
+            group = searches_resident(per_cu);
+        }
+        group = std::min(group, n);
         const int n_groups = (n + group - 1) / group;
         group = (n + n_groups - 1) / n_groups;   // groups of equal size
+        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] batch of %d: %d resident workgroups per CU, groups of %d\n", n, per_cu, group);
     }
     const size_t cells = (size_t)c.board_m * c.board_n;
     for (int start = 0; start < n; start += group) {
