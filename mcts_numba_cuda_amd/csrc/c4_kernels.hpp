@@ -63,7 +63,9 @@ struct __attribute__((aligned(128))) TreeHdr {
     // line 1: result exchange between the workgroups of the tree: [step parity][column] = step tag << 32 | -1 wins << 16 | +1 wins
     unsigned long long mail[2][kMaxCols];
     // line 2: steps completed since the last reset
-    uint32_t gen;    uint32_t pad2[31];
+    uint32_t gen;
+    uint32_t xcc[kMaxCols];        // XCC (L2 domain) each workgroup of the tree runs on, reported at the start of a launch
+    uint32_t pad2[31 - kMaxCols];
     // line 3: per-action playout results (trees_playout_outcomes_children[ti]), one writer per slot
     int32_t poc[kMaxCols][2]; int32_t pad3[16];
     // line 4: trees_actions_expanded[ti] and the row memorised at the first step of a run
@@ -368,7 +370,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
     __shared__ int32_t s_gather[kMaxCols][2];
     __shared__ int32_t s_poc[kMaxCols][2];
     __shared__ int16_t s_ae[16], s_root_ae[16];
-    __shared__ int32_t s_chosen, s_abort, s_redo;
+    __shared__ int32_t s_chosen, s_abort, s_redo, s_xcd_local;
 
     if (tid < kRecDwords) s_rec[0][tid] = reinterpret_cast<const uint32_t *>(nodes)[tid];
     if (tid < 16) { s_ae[tid] = hdr->ae[tid]; s_root_ae[tid] = hdr->root_ae[tid]; }
@@ -394,6 +396,14 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
     const bool timing = args.stage_timing != 0 && g == 0;
     const int root_turn = hdr->root_turn;
     uint32_t gen = hdr->gen;  // steps completed since reset
+    // Workgroups that share an XCC share its L2, and their stores are visible to each other as soon as they have left the
+    // write-through L1: publishing a result then needs no L2 write-back.  Whether the tree's workgroups do share one is
+    // established from their hardware XCC ids after the first, fully fenced, exchange of the launch.
+    bool xcd_local = false;
+    if (ACP && tid == 0) {
+        hdr->xcc[g] = (uint32_t)__builtin_amdgcn_s_getreg(6164) & 0xfu;   // HW_REG_XCC_ID, bits 3:0
+        s_xcd_local = 0;
+    }
     __syncthreads();
 
     for (int step = 0; step < args.nsteps; step++) {
@@ -580,7 +590,12 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
                 unsigned long long *mail = hdr->mail[gen & 1];
                 if (lane == 0) {
                     const unsigned long long v = ((unsigned long long)(gen + 1u) << 32) | ((unsigned long long)(uint32_t)res_neg << 16) | (unsigned long long)(uint32_t)res_pos;
-                    __hip_atomic_store(&mail[g], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                    if (xcd_local) {
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // earlier stores have reached the shared L2
+                        __hip_atomic_store(&mail[g], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    } else {
+                        __hip_atomic_store(&mail[g], v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
                 unsigned long long v = 0;
                 bool bad = false;
@@ -596,11 +611,17 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
                     }
                 }
                 fence_acquire_agent();
+                if (step == 0) {
+                    const uint32_t mine = (uint32_t)__builtin_amdgcn_s_getreg(6164) & 0xfu;
+                    const uint32_t theirs = (lane < G) ? __hip_atomic_load(&hdr->xcc[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : mine;
+                    if (__ballot(theirs != mine) == 0 && lane == 0) s_xcd_local = 1;
+                }
                 if (lane < G) { s_gather[lane][0] = (int32_t)((v >> 16) & 0xffffu); s_gather[lane][1] = (int32_t)(v & 0xffffu); }
                 if (__ballot(bad) != 0 && lane == 0) s_abort = 1;
             }
             __syncthreads();
             if (s_abort) break;
+            xcd_local = s_xcd_local != 0;
             if (timing) tk_exchange += wall_clock64() - tk;
         }
 
