@@ -254,10 +254,12 @@ __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const u
     if (n_legal > 0) write_priors(g, tree, 0, board, weight, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
 }
 
-// Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one: the vector L1 is
-// written through but keeps lines that device-scope atomics of other wavefronts have changed underneath it.
+// Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one.  All wavefronts of a
+// tree run on one CU: stores leave its write-through L1 towards the L2 they all share (the workgroup-scope release waits
+// for that), but the L1 keeps lines that device-scope atomics of other wavefronts have changed underneath it, so the
+// acquire side drops the L1.  No L2 write-back is needed.
 __device__ __forceinline__ void phase_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
