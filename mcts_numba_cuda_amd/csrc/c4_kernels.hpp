@@ -370,7 +370,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
     __shared__ int32_t s_gather[kMaxCols][2];
     __shared__ int32_t s_poc[kMaxCols][2];
     __shared__ int16_t s_ae[16], s_root_ae[16];
-    __shared__ int32_t s_chosen, s_abort, s_redo, s_xcd_local;
+    __shared__ int32_t s_abort, s_redo, s_xcd_local;
 
     if (tid < kRecDwords) s_rec[0][tid] = reinterpret_cast<const uint32_t *>(nodes)[tid];
     if (tid < 16) { s_ae[tid] = hdr->ae[tid]; s_root_ae[tid] = hdr->root_ae[tid]; }
@@ -389,7 +389,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
         const uint64_t *p = ref.rng_playout + 2 * ((size_t)(ACP ? g * P : 0) + tid);
         s0 = p[0]; s1 = p[1];
     }
-    if (!ACP && tid == 0) { e0 = ref.rng_expand[0]; e1 = ref.rng_expand[1]; }
+    if (!ACP) { e0 = ref.rng_expand[0]; e1 = ref.rng_expand[1]; }
     uint32_t plies = 0, u1 = 0;
     uint32_t st_levels = 0, st_children = 0, st_expanded = 0, st_played = 0;
     unsigned long long tk_select = 0, tk_expand = 0, tk_playout = 0, tk_backup = 0, tk_exchange = 0, tk = 0;
@@ -495,29 +495,35 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
             }
         } else {
             if (mode == kModeExpand) {
-                // all children are created (src/mctsnc.py:1756-1821), one is drawn for the playouts (:1435,:1511)
-                if (tid == 0) {
+                // all children are created (src/mctsnc.py:1756-1821), one is drawn for the playouts (:1435,:1511); every
+                // thread carries the expansion generator and draws the same number
+                {
                     const float u = rng_uniform(e0, e1);
                     int ord = (int)(int16_t)((double)u * (double)k_exp);
                     if (ord > k_exp - 1) ord = k_exp - 1;
                     uint32_t rest = expmask;   // the ord-th set bit of the mask
                     for (int j = 0; j < ord; j++) rest &= rest - 1u;
-                    s_chosen = __ffs(rest) - 1;
+                    chosen = __ffs(rest) - 1;
                 }
-                __syncthreads();
-                chosen = s_chosen;
-                uint64_t chosen_pos = 0, chosen_neg = 0; int chosen_outcome = 2;
-                for (int a = 0; a < ncols; a++) {
-                    if (!((expmask >> a) & 1u)) continue;
-                    const int child = size + __popc(expmask & ((1u << a) - 1u));
-                    const uint64_t newbit = (all + geo.bottom(a)) & geo.col_mask(a);
-                    const uint64_t cpos = leaf.bb_pos | (mover == 1 ? newbit : 0ull);
-                    const uint64_t cneg = leaf.bb_neg | (mover == 1 ? 0ull : newbit);
-                    const bool win = geo.has_four(mover == 1 ? cpos : cneg);
-                    const int outcome = win ? mover : (((all | newbit) == geo.full) ? 0 : 2);
-                    if (a == chosen) { chosen_pos = cpos; chosen_neg = cneg; chosen_outcome = outcome; }
-                    if (wave == 0 && lane < 32)
-                        reinterpret_cast<uint32_t *>(nodes + child)[lane] = child_record_dword(lane, cpos, cneg, leaf.node, L + 1, -mover, outcome, a);
+                // lane a (mod 8) of every wavefront evaluates child a; wave 0 then stores two records per instruction
+                const int a_l = min(lane & 7, ncols - 1);
+                const uint64_t newbit_l = (all + geo.bottom(a_l)) & geo.col_mask(a_l);
+                const uint64_t cpos_l = leaf.bb_pos | (mover == 1 ? newbit_l : 0ull);
+                const uint64_t cneg_l = leaf.bb_neg | (mover == 1 ? 0ull : newbit_l);
+                const bool win_l = geo.has_four(mover == 1 ? cpos_l : cneg_l);
+                const int outcome_l = win_l ? mover : (((all | newbit_l) == geo.full) ? 0 : 2);
+                const uint64_t chosen_pos = (uint64_t)__shfl((unsigned long long)cpos_l, chosen), chosen_neg = (uint64_t)__shfl((unsigned long long)cneg_l, chosen);
+                const int chosen_outcome = __shfl(outcome_l, chosen);
+                if (wave == 0) {
+                    for (int a0 = 0; a0 < ncols; a0 += 2) {
+                        const int a = a0 + (lane >> 5);
+                        const uint64_t cpos = (uint64_t)__shfl((unsigned long long)cpos_l, a & 7), cneg = (uint64_t)__shfl((unsigned long long)cneg_l, a & 7);
+                        const int outcome = __shfl(outcome_l, a & 7);
+                        if (a < ncols && ((expmask >> a) & 1u)) {
+                            const int child = size + __popc(expmask & ((1u << a) - 1u));
+                            reinterpret_cast<uint32_t *>(nodes + child)[lane & 31] = child_record_dword(lane & 31, cpos, cneg, leaf.node, L + 1, -mover, outcome, a);
+                        }
+                    }
                 }
                 if (chosen_outcome != 2) { res_neg = chosen_outcome == -1 ? P : 0; res_pos = chosen_outcome == 1 ? P : 0; }
                 else { do_playouts = true; pl_turn = -mover; pl_cur = (pl_turn == 1) ? chosen_pos : chosen_neg; pl_opp = (pl_turn == 1) ? chosen_neg : chosen_pos; }
