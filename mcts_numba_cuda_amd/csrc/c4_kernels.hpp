@@ -505,7 +505,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
                     for (int j = 0; j < ord; j++) rest &= rest - 1u;
                     chosen = __ffs(rest) - 1;
                 }
-                // lane a (mod 8) of every wavefront evaluates child a; wave 0 then stores two records per instruction
+                // lane a (mod 8) of every wavefront evaluates child a; a store instruction writes two records
                 const int a_l = min(lane & 7, ncols - 1);
                 const uint64_t newbit_l = (all + geo.bottom(a_l)) & geo.col_mask(a_l);
                 const uint64_t cpos_l = leaf.bb_pos | (mover == 1 ? newbit_l : 0ull);
@@ -514,8 +514,8 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
                 const int outcome_l = win_l ? mover : (((all | newbit_l) == geo.full) ? 0 : 2);
                 const uint64_t chosen_pos = (uint64_t)__shfl((unsigned long long)cpos_l, chosen), chosen_neg = (uint64_t)__shfl((unsigned long long)cneg_l, chosen);
                 const int chosen_outcome = __shfl(outcome_l, chosen);
-                if (wave == 0) {
-                    for (int a0 = 0; a0 < ncols; a0 += 2) {
+                {   // every wavefront stores two of the records
+                    for (int a0 = 2 * wave; a0 < ncols; a0 += 2 * nwaves) {
                         const int a = a0 + (lane >> 5);
                         const uint64_t cpos = (uint64_t)__shfl((unsigned long long)cpos_l, a & 7), cneg = (uint64_t)__shfl((unsigned long long)cneg_l, a & 7);
                         const int outcome = __shfl(outcome_l, a & 7);
