@@ -761,6 +761,16 @@ int mctsnc_init_device(mctsnc_engine *e) {
         const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->block);
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (e->acp) {
+            // as many workgroups per tree as stay resident together (each takes every G-th child of the expanded node)
+            int per_cu = 0, cus = 0;
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e->block, lds));
+            HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
+            const int64_t resident = (int64_t)per_cu * cus;
+            int64_t g_fit = resident / (8 * ((T + 7) / 8));   // the grid is 8 * G * ceil(T / 8) workgroups
+            if (g_fit > A) g_fit = A;
+            if (g_fit > e->G) e->G = (int)g_fit;
+        }
     }
     int rc = upload_rng(e);
     if (rc) return rc;
