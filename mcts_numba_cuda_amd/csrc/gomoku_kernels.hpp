@@ -173,13 +173,17 @@ __device__ inline int exact_playout(ExactScratch &s, int m, int n, const uint32_
     }
 }
 
-// run of set bits next to `bit` on both sides of a line word, each side capped at five
-__device__ __forceinline__ int line_neighbours(uint32_t v, int bit) {
-    const uint32_t right = ~(v >> (bit + 1));
-    const int run_r = min(5, (int)__builtin_ctz(right | 0x20u));
-    const uint32_t left = ~((v << (31 - bit)) << 1);  // bits below `bit`, aligned to the top
-    const int run_l = min(5, (int)__builtin_clz(left | 0x04000000u));
-    return run_r + run_l;
+// Two 16-bit line words side by side: bit s of a half is set where a run of exactly five stones starts at s (the
+// cells before and after the run are empty, the opponent's or off the board).  "Exactly four neighbours" of
+// compute_outcome_gomoku (src/mctsnc_game_mechanics.py:220-281) = the stone lies in such a run.
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t exact_five_starts(uint32_t packed) {
+    const u16x2 v = __builtin_bit_cast(u16x2, packed);
+    const u16x2 two = v & (v >> 1);
+    const u16x2 four = two & (two >> 2);
+    const u16x2 five = four & (v >> 4);
+    const u16x2 exact = five & ~(v << 1) & ~(v >> 5);
+    return __builtin_bit_cast(uint32_t, exact);
 }
 
 struct LeafInfo {
@@ -370,14 +374,14 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                 // templates: board, legal list in row-major order, line words of both players
                 if (tid < 16) s_cbb[tid] = (tid < 8) ? pn->bb_pos[tid] : pn->bb_neg[tid - 8];
                 __syncthreads();
-                if (wave == 0) {  // empty cells in row-major order, compacted with ballots
+                if (wave == 0) {  // empty cells in row-major order as (row << 4 | column), compacted with ballots
                     uint8_t *tm = reinterpret_cast<uint8_t *>(s_tmpl);
                     int cnt = 0;
                     for (int base = 0; base < cells; base += 64) {
                         const int c = base + lane;
                         const bool empty = c < cells && !bb_test(s_cbb, c) && !bb_test(s_cbb + 8, c);
                         const unsigned long long mask = __ballot(empty);
-                        if (empty) tm[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (uint8_t)c;
+                        if (empty) { const uint32_t ci = ((uint32_t)c * div_n) >> 16; tm[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (uint8_t)((ci << 4) | ((uint32_t)c - ci * (uint32_t)n)); }
                         cnt += __popcll(mask);
                     }
                     if (lane == 0) s_count = cnt;
@@ -420,8 +424,10 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                         }
                         uint8_t *const lb = reinterpret_cast<uint8_t *>(s_list + tid);   // byte i: lb[(i >> 2) * stride4 + (i & 3)]
                         uint32_t *const lp = s_lines + tid;
-                        const int stride4 = nthreads << 2;
-                        int count = count0, turn = pturn, status = count0 == 0 ? 2 : 0;
+                        const uint32_t nt = (uint32_t)nthreads, stride4 = nt << 2;
+                        int count = count0, outcome_if_win = pturn, status = count0 == 0 ? 2 : 0;
+                        // byte selector that packs the mover's halves of two line words into one dword; flips with the side to move
+                        uint32_t sel = pturn == 1 ? 0x05040100u : 0x07060302u;
                         Rng32 rg;
                         rg.s0l = (uint32_t)s0; rg.s0h = (uint32_t)(s0 >> 32); rg.s1l = (uint32_t)s1; rg.s1h = (uint32_t)(s1 >> 32);
                         while (status == 0) {
@@ -431,24 +437,27 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                             const int ord = (int)(u * (float)count);  // single-precision product (src/mctsnc.py:1882)
                             if (ord >= count) { status = 3; break; }
                             count--;
-                            uint8_t *const slot = lb + (ord >> 2) * stride4 + (ord & 3);
-                            const int a = *slot;
-                            *slot = lb[(count >> 2) * stride4 + (count & 3)];  // swap-remove (:209-217)
+                            uint8_t *const slot = lb + __umul24((uint32_t)ord >> 2, stride4) + (ord & 3);
+                            const uint32_t a = *slot;
+                            *slot = lb[__umul24((uint32_t)count >> 2, stride4) + (count & 3)];  // swap-remove (:209-217)
                             plies++;
-                            const int i = (int)(((uint32_t)a * div_n) >> 16), jj = a - i * n;
-                            const int sh = turn == 1 ? 0 : 16;
-                            uint32_t *const p_row = lp + i * nthreads, *const p_col = lp + (m + jj) * nthreads;
-                            uint32_t *const p_dia = lp + (m + n + (i - jj + n - 1)) * nthreads;
-                            uint32_t *const p_ant = lp + (m + n + (m + n - 1) + (i + jj)) * nthreads;
+                            const uint32_t i = a >> 4, jj = a & 15u;
+                            const uint32_t sh = (sel & 2u) << 3;  // 0 for the +1 side, 16 for the -1 side
+                            uint32_t *const p_row = lp + __umul24(i, nt), *const p_col = lp + __umul24((uint32_t)m + jj, nt);
+                            uint32_t *const p_dia = lp + __umul24((uint32_t)(m + n + n - 1) + i - jj, nt);
+                            uint32_t *const p_ant = lp + __umul24((uint32_t)(m + n + m + n - 1) + i + jj, nt);
                             // the four lines through a cell are four different words: read all, then write all
                             uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
-                            w_row |= (1u << jj) << sh; w_col |= (1u << i) << sh; w_dia |= (1u << jj) << sh; w_ant |= (1u << jj) << sh;
+                            const uint32_t bit_j = (1u << jj) << sh;
+                            w_row |= bit_j; w_col |= (1u << i) << sh; w_dia |= bit_j; w_ant |= bit_j;
                             *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
-                            const bool win = (line_neighbours((w_row >> sh) & 0xffffu, jj) == 4) | (line_neighbours((w_col >> sh) & 0xffffu, i) == 4) |
-                                             (line_neighbours((w_dia >> sh) & 0xffffu, jj) == 4) | (line_neighbours((w_ant >> sh) & 0xffffu, jj) == 4);
-                            if (win) { status = 1; outcome = turn; }
+                            const uint32_t win_j = (0x1fu << jj) >> 4, win_i = (0x1fu << i) >> 4;  // starts of a run of five through the stone
+                            const uint32_t hit = exact_five_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
+                            const uint32_t hit2 = exact_five_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
+                            if ((hit | hit2) != 0) { status = 1; outcome = outcome_if_win; }
                             else if (count == 0) { status = 2; outcome = 0; }
-                            turn = -turn;
+                            outcome_if_win = -outcome_if_win;
+                            sel ^= 0x02020202u;
                         }
                         s0 = ((uint64_t)rg.s0h << 32) | rg.s0l; s1 = ((uint64_t)rg.s1h << 32) | rg.s1l;
                         redo = status == 3;
