@@ -38,19 +38,13 @@ __host__ __device__ __forceinline__ float rng_uniform(uint64_t &s0, uint64_t &s1
 __host__ __device__ inline double det_log(double x) { return detm_log(x); }
 
 #ifdef __HIPCC__
-// float32((x >> 11) * 2^-53) for x = hi * 2^32 + lo, without double arithmetic.  The 11 discarded bits are
-// cleared, the value is shifted left until hi has its top bit at position 25 or above (an exact rescaling), and the
-// bits left in lo are folded into bit 0 of hi as a sticky bit: float32 conversion then drops at least two bits of hi,
-// so round-to-nearest-even sees the same round and sticky information as the exact value.  (If hi was 0, the shift
-// moves all of lo into hi and nothing is left to fold.)
+// float32((x >> 11) * 2^-53) for x = hi * 2^32 + lo (xoroshiro128p_uniform_float32 of numba.cuda.random as the
+// reference calls it, src/mctsnc.py:1882): the 11 discarded bits are cleared, the remaining 53 significant bits are
+// exact in float64 (two conversions and one fused multiply-add, all exact), the narrowing rounds once to nearest even
+// as the reference's float32 cast does, and the scaling by 2^-64 is exact.  Five instructions per draw.
 __device__ __forceinline__ float uniform_from_bits(uint32_t lo, uint32_t hi) {
-    lo &= 0xfffff800u;
-    int sh = (int)__clz((int)hi) - 6;  // __clz(0) = 32
-    sh = sh < 0 ? 0 : sh;
-    const uint32_t hi2 = sh ? __builtin_amdgcn_alignbit(hi, lo, 32 - sh) : hi;
-    const uint32_t lo2 = lo << sh;
-    const uint32_t t = hi2 | (lo2 != 0 ? 1u : 0u);
-    return ldexpf((float)t, -32 - sh);
+    const double d = __builtin_fma((double)hi, 4294967296.0, (double)(lo & 0xfffff800u));
+    return (float)d * 0x1p-64f;
 }
 
 // xoroshiro128+ step on 32-bit halves (the 64-bit shifts of the generic form are slow vector instructions)
