@@ -57,3 +57,14 @@ def test_gomoku_large_playout_count_runs_in_rounds():
     e, o = engines("ocp_thrifty", 1, 512, 15, 15)
     board, turn = random_gomoku_root(np.random.default_rng(2), 15, 15, 8)
     compare_with_oracle(e, o, board, None, turn, 12)
+
+
+@pytest.mark.parametrize("variant", ["ocp_prodigal", "acp_thrifty"])
+def test_gomoku_sixteen_wide_boards(variant):
+    """16 is the widest line the engine holds (one 16-bit half per side and line): fives and longer runs that touch
+    the last cell of a row, column or diagonal must be judged as on any other board."""
+    rng = np.random.default_rng(16)
+    for (m, n), steps in (((16, 16), 30), ((5, 16), 120), ((16, 5), 120), ((16, 6), 60)):
+        e, o = engines(variant, 2, 64, m, n)
+        board, turn = random_gomoku_root(rng, m, n, 6)
+        compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else max(3, steps // 10))
