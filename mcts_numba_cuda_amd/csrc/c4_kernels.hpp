@@ -65,7 +65,11 @@ struct __attribute__((aligned(128))) TreeHdr {
     // line 2: steps completed since the last reset
     uint32_t gen;
     uint32_t xcc[kMaxCols];        // XCC (L2 domain) each workgroup of the tree runs on, reported at the start of a launch
-    uint32_t pad2[31 - kMaxCols];
+    uint32_t pad2a;
+    // launch number << 32 | 1 + index of the tree that the workgroups which have just finished this one take next
+    // (written by workgroup 0 when a launch has more trees than resident workgroup sets)
+    unsigned long long next_job;
+    uint32_t pad2[31 - kMaxCols - 3];
     // line 3: per-action playout results (trees_playout_outcomes_children[ti]), one writer per slot
     int32_t poc[kMaxCols][2]; int32_t pad3[16];
     // line 4: trees_actions_expanded[ti] and the row memorised at the first step of a run
@@ -99,6 +103,8 @@ struct SearchArgs {
     float ucb_c;
     int32_t stage_timing;   // accumulate per-stage device time in the tree headers
     int32_t *abort_flag;
+    int32_t *queue;         // next tree not yet handed out, or null when every tree has its own workgroups
+    uint32_t launch_seq;    // distinguishes the launches that use the queue
 };
 
 struct Geometry {
@@ -298,7 +304,7 @@ __global__ void reset_kernel(const TreeRef *refs, int n_refs, const uint64_t *ro
     h->size = 1; h->root_ns = 0; h->root_wins = 0; h->max_depth = 0; h->depth_sum = 0;
     h->selected = 0; h->path_len = 0; h->mode = 0; h->error = 0; h->root_turn = root_turns[r];
     for (int i = 0; i < kMaxCols; i++) { h->mail[0][i] = 0; h->mail[1][i] = 0; }
-    h->gen = 0; h->plies = 0; h->u1_events = 0;
+    h->gen = 0; h->next_job = 0; h->plies = 0; h->u1_events = 0;
     h->stat_levels = 0; h->stat_children = 0; h->stat_expanded = 0; h->stat_played = 0;
     h->t_select = 0; h->t_expand = 0; h->t_playout = 0; h->t_backup = 0; h->t_exchange = 0;
 }
@@ -341,15 +347,10 @@ __host__ __device__ inline size_t search_lds_bytes(int m, int n) {
     return explore_bytes(m, n) + (size_t)path_levels(m, n) * kRecDwords * sizeof(uint32_t);
 }
 
+// The whole search of tree `r` by its G workgroups; this one is number g of them.
 template <bool ACP>
-__device__ __forceinline__ void search_body(const SearchArgs &args) {
-    // XCD-aware decode: consecutive blockIdx values go to different XCDs, so the workgroups of one tree
-    // are spaced 8 apart and meet in one L2.
-    const int b = blockIdx.x;
+__device__ __forceinline__ void search_body(const SearchArgs &args, const int r, const int g) {
     const int G = args.G;
-    const int r = (b & 7) + 8 * ((b >> 3) / G);
-    const int g = (b >> 3) % G;
-    if (r >= args.n_refs) return;
     const TreeRef ref = args.refs[r];
     Node *const nodes = ref.nodes;
     TreeHdr *const hdr = ref.hdr;
@@ -785,8 +786,44 @@ __device__ __forceinline__ void search_body(const SearchArgs &args) {
     }
 }
 
+// XCD-aware decode: consecutive blockIdx values go to different XCDs, so the G workgroups of one set are spaced 8
+// apart and meet in one L2.  Set u starts on tree u; when a launch has more trees than sets (a large batch of
+// searches), a set that has finished its tree takes the next one from the queue: workgroup 0 draws the index and
+// leaves it in the finished tree's header for the others.  Five wavefronts per SIMD (at most 96 vector registers, two
+// dwords spilled) let five workgroups share a CU in such batches; a single search is no slower for it.
 template <bool ACP>
-__global__ void __launch_bounds__(512) search_kernel(SearchArgs args) { search_body<ACP>(args); }
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(5, 5))) search_kernel(SearchArgs args) {
+    const int b = blockIdx.x;
+    const int G = args.G;
+    const int g = (b >> 3) % G;
+    int r = (b & 7) + 8 * ((b >> 3) / G);
+    __shared__ int32_t s_next;
+    while (r < args.n_refs) {
+        search_body<ACP>(args, r, g);
+        if (args.queue == nullptr) break;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            TreeHdr *const hdr = args.refs[r].hdr;
+            int32_t next = args.n_refs;  // nothing more unless told otherwise
+            if (__hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+                if (g == 0) {
+                    next = atomicAdd(args.queue, 1);
+                    __hip_atomic_store(&hdr->next_job, ((unsigned long long)args.launch_seq << 32) | (uint32_t)(next + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+                } else {
+                    for (uint32_t spins = 0; spins <= (kSpinLimit >> 4); spins++) {  // the others of the set finish within microseconds of each other
+                        const unsigned long long v = __hip_atomic_load(&hdr->next_job, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                        if ((uint32_t)(v >> 32) == args.launch_seq) { next = (int32_t)(uint32_t)v - 1; break; }
+                        if ((spins & 1023u) == 1023u && __hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                        __builtin_amdgcn_s_sleep(8);
+                    }
+                }
+            }
+            s_next = next;
+        }
+        __syncthreads();
+        r = s_next;
+    }
+}
 
 
 // Per-tree digest for the final reductions (_reduce_over_trees_*, src/mctsnc.py:2222-2296).

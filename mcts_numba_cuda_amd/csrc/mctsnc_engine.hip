@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstdarg>
@@ -411,12 +412,33 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
-    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    const dim3 block(e0->block);
     const size_t lds = c4::search_lds_bytes(c.board_m, c.board_n);
+    // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
+    // all its workgroups must be resident together: a batch with more trees than resident sets starts one tree per
+    // set and hands the remaining trees out through a queue as sets finish.
+    int sets = 8 * ((n_refs + 7) / 8);
+    args.queue = nullptr; args.launch_seq = 0;
+    if (e0->acp) {
+        int per_cu = 0, cus = 0;
+        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
+        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
+        const int resident_sets = (int)((int64_t)per_cu * cus / (8 * e0->G)) * 8;
+        if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * e0->G);
+        if (sets > resident_sets) { sets = resident_sets; args.queue = e0->d_abort + 1; }
+        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets (%d workgroups per CU resident)%s\n", n_refs, sets, per_cu, args.queue ? ", queue" : "");
+    }
+    const dim3 grid(e0->G * sets);
+    static std::atomic<uint32_t> launch_counter{0};
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
         args.nsteps = nsteps;
         if (e0->acp) {
+            if (args.queue) {
+                args.launch_seq = ++launch_counter;
+                if (args.launch_seq == 0) args.launch_seq = ++launch_counter;   // 0 is what a reset header holds
+                HIP_TRY(hipMemcpyAsync(args.queue, &sets, sizeof(int32_t), hipMemcpyHostToDevice, stream));
+            }
             void *kargs[] = {&args};
             HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
         } else {
@@ -554,21 +576,13 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     // resident: a batch whose grid exceeds what the device holds at once runs as consecutive groups of searches, each
     // with the whole budget.
     int group = n;
-    if (e0->acp && n > 1) {
+    if (e0->acp && n > 1 && e0->is_gomoku()) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        auto searches_resident = [&](int blocks_per_cu) {   // the grid is 8 * G * ceil(refs / 8) workgroups
-            return (int)std::max<int64_t>(1, ((int64_t)blocks_per_cu * cus / (8 * e0->G) * 8) / c.n_trees);
-        };
-        if (e0->is_gomoku()) {
-            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
-                                                                 gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
-            group = searches_resident(per_cu);
-        } else {
-            const size_t lds = c4::search_lds_bytes(c.board_m, c.board_n);
-            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
-            group = searches_resident(per_cu);
-        }
+        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
+                                                             gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
+        // the grid is 8 * G * ceil(refs / 8) workgroups
+        group = (int)std::max<int64_t>(1, ((int64_t)per_cu * cus / (8 * e0->G) * 8) / c.n_trees);
         group = std::min(group, n);
         const int n_groups = (n + group - 1) / group;
         group = (n + n_groups - 1) / n_groups;   // groups of equal size
@@ -709,7 +723,7 @@ int mctsnc_init_device(mctsnc_engine *e) {
     HIP_TRY(hipMalloc(&e->d_rng_playout, sizeof(uint64_t) * 2 * e->n_rng_playout));
     if (!e->acp) HIP_TRY(hipMalloc(&e->d_rng_expand, sizeof(uint64_t) * 2 * T));
     HIP_TRY(hipMalloc(&e->d_root_turns, sizeof(int32_t) * T));
-    HIP_TRY(hipMalloc(&e->d_abort, sizeof(int32_t)));
+    HIP_TRY(hipMalloc(&e->d_abort, 2 * sizeof(int32_t)));   // [0] abort flag, [1] head of the tree queue of a batch launch
     const size_t rng_per_tree = (size_t)(e->acp ? c.max_actions * c.n_playouts : c.n_playouts);
     if (!e->is_gomoku()) {
         HIP_TRY(hipMalloc(&e->d_nodes, sizeof(c4::Node) * S * T));
