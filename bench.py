@@ -376,8 +376,8 @@ def main():
 
         batched = None
         if not args.no_batched:
-            # the same 64 searches, all handed to the device at once (the engine runs them in as few fully resident
-            # groups as the device allows); results are identical to the sequential runs
+            # the same 64 searches, all handed to the device at once (one launch: the resident sets of workgroups take
+            # further trees from a queue as they finish theirs); results are identical to the sequential runs
             nb = min(len(roots), max(args.steps, 1))
             engines = [eng] + [new_engine() for _ in range(nb - 1)]
             chunk = roots[:nb]

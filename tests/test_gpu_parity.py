@@ -105,17 +105,18 @@ def test_run_batch_equals_single_runs():
             np.testing.assert_array_equal(eb.read_array("rng_playout"), es.read_array("rng_playout"))
 
 
-def test_run_batch_larger_than_the_device_runs_in_groups():
-    """A batch whose workgroups cannot all be resident at once (48 searches x 4 trees x 7 columns = 1344 workgroups of
-    256 threads) is split into consecutive groups; every search still ends exactly where a separate run ends."""
+def test_run_batch_larger_than_the_device_takes_trees_from_the_queue():
+    """A batch whose workgroups cannot all be resident at once (80 searches x 4 trees x 7 columns = 2240 workgroups of
+    256 threads): the resident sets of workgroups start on one tree each and take the others from a queue as they
+    finish; every search still ends exactly where a separate run ends."""
     from mcts_numba_cuda_amd import run_batch
     rng = np.random.default_rng(17)
     params = dict(n_trees=4, n_playouts=256, variant="acp_thrifty", device_memory=0.02, ucb_c=2.0, seed=3)
-    roots = [random_c4_root(rng, int(rng.integers(0, 24))) for _ in range(48)]
+    roots = [random_c4_root(rng, int(rng.integers(0, 24))) for _ in range(80)]
     batch = [make_engine(params) for _ in roots]
     run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=120)
     single = make_engine(params)
-    for k in (0, 7, 31, 32, 33, 47):
+    for k in (0, 7, 31, 43, 44, 45, 62, 79):
         single.reseed()
         single.run(*roots[k], forced_search_steps_limit=120)
         assert batch[k].actions_info == single.actions_info
@@ -161,3 +162,27 @@ def test_tree_full_and_terminal_paths_match_oracle():
             board, fills, turn = random_c4_root(rng, plies)
             compare_with_oracle(e, o, board, fills, turn, steps=200)
         assert max(e.read_array("depths", t).shape[0] for t in range(2)) <= e.max_tree_size
+
+
+def test_gomoku_run_batch_in_groups():
+    """Three Gomoku all-child-playouts searches in one call.  One such search already fills the device (8 trees x 64
+    workgroups of 74 KB of LDS, two per CU), so the host runs them in consecutive groups; results equal separate runs."""
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    rng = np.random.default_rng(23)
+
+    def mk():
+        e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, n_trees=8, n_playouts=128, variant="acp_prodigal", device_memory=0.5,
+                   seed=4, verbose_info=False, game="gomoku")
+        e.init_device_side_arrays()
+        return e
+    from helpers import random_gomoku_root
+    roots = [random_gomoku_root(rng, 15, 15, int(rng.integers(0, 12))) for _ in range(3)]
+    batch = [mk() for _ in roots]
+    run_batch(batch, [r[0] for r in roots], None, [r[1] for r in roots], forced_search_steps_limit=4)
+    single = mk()
+    for k in range(3):
+        single.reseed()
+        single.run(roots[k][0], None, roots[k][1], forced_search_steps_limit=4)
+        assert batch[k].actions_info == single.actions_info
+        for name in ("trees", "ns", "ns_wins"):
+            np.testing.assert_array_equal(batch[k].read_array(name, 7), single.read_array(name, 7))
