@@ -190,7 +190,7 @@ __device__ __forceinline__ uint32_t exact_five_starts(uint32_t packed) {
 }
 
 struct LeafInfo {
-    int32_t node, depth, turn, flags, outcome;
+    int32_t node, depth, turn, flags, outcome, size;
 };
 
 // ---- kernels ----------------------------------------------------------------------------------------------------
@@ -276,27 +276,31 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
         if (timing) tk = wall_clock64();
         // ================= selection: follow the memoised best children =================
         if (wave == 0) {
+            // one coalesced load of the 128-byte record per level (lane i: dword i), fields handed round with readlane
+            const int size_now = hdr->size;   // in flight during the walk
             int node = 0, depth = 0;
+            uint32_t w, meta;
             for (;;) {
-                const Node *nd = nodes + node;
-                const uint32_t flags = nd->flags;
+                w = reinterpret_cast<const uint32_t *>(nodes + node)[lane & 31];
+                meta = (uint32_t)__builtin_amdgcn_readlane((int)w, 5);   // flags | pad << 8 | action << 16
                 if (lane == 0) s_path[depth] = node;
-                if (flags & kLeaf) break;
-                st_children += (uint32_t)nd->n_children;
-                node = nd->best_child;
+                if (meta & kLeaf) break;
+                st_children += (uint32_t)__builtin_amdgcn_readlane((int)w, 2);
+                node = __builtin_amdgcn_readlane((int)w, 3);
                 depth++;
             }
-            const Node *nd = nodes + node;
-            if (lane < 8) { s_bb[lane] = nd->bb_pos[lane]; s_bb[8 + lane] = nd->bb_neg[lane]; }
+            if (lane >= 8 && lane < 24) s_bb[lane - 8] = w;   // dwords 8..15: stones of +1, 16..23: stones of -1
+            const uint32_t dto = (uint32_t)__builtin_amdgcn_readlane((int)w, 4);   // depth | turn << 16 | outcome << 24
             if (lane == 0) {
-                LeafInfo li; li.node = node; li.depth = depth; li.turn = nd->turn; li.flags = nd->flags; li.outcome = nd->outcome;
+                LeafInfo li; li.node = node; li.depth = depth; li.turn = (int8_t)(dto >> 16); li.flags = (int32_t)(meta & 0xffu); li.outcome = (int8_t)(dto >> 24);
+                li.size = size_now;
                 s_leaf = li;
             }
         }
         __syncthreads();
         const LeafInfo leaf = s_leaf;
         const int L = leaf.depth;
-        const int size = hdr->size;
+        const int size = leaf.size;
         const int mover = leaf.turn;
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_select += t2 - tk; tk = t2; }
 
