@@ -433,7 +433,8 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 const uint32_t mask = meta & 0xffu, a = meta >> 24;
                 node = __builtin_amdgcn_readlane(w, kDwBase) + __popc(mask & ((1u << a) - 1u));
                 d++;
-                w = reinterpret_cast<const uint32_t *>(nodes + node)[lane & 31];
+                // read past the L1: the record may have been rewritten by another workgroup of the tree since this CU last saw it
+                w = __hip_atomic_load(reinterpret_cast<const uint32_t *>(nodes + node) + (lane & 31), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (lane < kRecDwords) s_rec[d][lane] = w;
                 if (lane == 0) { s_pnode[d] = node; s_pslot[d] = (uint8_t)a; }
             }
@@ -622,7 +623,9 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                         if ((spins & 1023u) == 0 && __hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { bad = true; break; }
                     }
                 }
-                fence_acquire_agent();
+                // the only device memory read later in a step are tree records, which the walk reads past the L1; so
+                // workgroups on one XCC (one L2) need no cache invalidation here
+                if (xcd_local) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); else fence_acquire_agent();
                 if (step == 0) {
                     const uint32_t mine = (uint32_t)__builtin_amdgcn_s_getreg(6164) & 0xfu;
                     const uint32_t theirs = (lane < G) ? __hip_atomic_load(&hdr->xcc[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : mine;
