@@ -371,7 +371,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
     __shared__ int32_t s_gather[kMaxCols][2];
     __shared__ int32_t s_poc[kMaxCols][2];
     __shared__ int16_t s_ae[16], s_root_ae[16];
-    __shared__ int32_t s_abort, s_redo, s_xcd_local;
+    __shared__ int32_t s_abort, s_xcd_local;
 
     if (tid < kRecDwords) s_rec[0][tid] = reinterpret_cast<const uint32_t *>(nodes)[tid];
     if (tid < 16) { s_ae[tid] = hdr->ae[tid]; s_root_ae[tid] = hdr->root_ae[tid]; }
@@ -469,7 +469,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
             const uint32_t legal = geo.legal_cols(all);
             int room = S - size; if (room < 0) room = 0;
             expmask = legal;
-            while (__popc(expmask) > room) expmask &= ~(1u << (31 - __clz(expmask)));  // children beyond the pool end are dropped
+            while ((int)__popc(expmask) > room) expmask &= ~(1u << (31 - __clz(expmask)));  // children beyond the pool end are dropped
             mode = expmask ? kModeExpand : kModeFull;
         }
         const int k_exp = __popc(expmask);

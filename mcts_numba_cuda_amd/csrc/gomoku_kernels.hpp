@@ -252,7 +252,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
     __shared__ unsigned long long s_lkey[kLevels];   // per level of a chunk of the backup's arg-max: best key,
     __shared__ double s_llog[kLevels];               // log of the node's visit count,
     __shared__ int32_t s_lbase[kLevels], s_lkc[kLevels];   // first child and number of children
-    __shared__ int32_t s_flag, s_chosen, s_abort, s_redo, s_tot[2], s_count;
+    __shared__ int32_t s_flag, s_chosen, s_abort, s_redo, s_count;
     __shared__ ExactScratch s_exact;
 
     if (tid == 0) s_abort = 0;
