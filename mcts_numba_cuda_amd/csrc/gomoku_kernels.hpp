@@ -445,16 +445,27 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                         uint32_t sel = pturn == 1 ? 0x05040100u : 0x07060302u;
                         Rng32 rg;
                         rg.s0l = (uint32_t)s0; rg.s0h = (uint32_t)(s0 >> 32); rg.s1l = (uint32_t)s1; rg.s1h = (uint32_t)(s1 >> 32);
-                        while (status == 0) {
+                        // A ply is two chains of dependent work with an LDS round trip each: draw a cell (generator, product,
+                        // list read, swap-remove) and judge it (four line reads, stone, test for five).  They are software
+                        // pipelined: while cell k is judged, cell k + 1 is already drawn.  When ply k ends the game, the
+                        // generator goes back to its state after draw k; what draw k + 1 did to the list no longer matters.
+                        uint32_t a = 0;   // cell of the current ply, already taken off the list
+                        if (status == 0) {
                             uint32_t xl, xh;
                             rng_next32(rg, xl, xh);
-                            const float u = uniform_from_bits(xl, xh);
-                            const int ord = (int)(u * (float)count);  // single-precision product (src/mctsnc.py:1882)
-                            if (ord >= count) { status = 3; break; }
-                            count--;
-                            uint8_t *const slot = lb + __umul24((uint32_t)ord >> 2, stride4) + (ord & 3);
-                            const uint32_t a = *slot;
-                            *slot = lb[__umul24((uint32_t)count >> 2, stride4) + (count & 3)];  // swap-remove (:209-217)
+                            const int ord = (int)(uniform_from_bits(xl, xh) * (float)count);  // single-precision product (src/mctsnc.py:1882)
+                            if (ord >= count) status = 3;
+                            else {
+                                count--;
+                                uint8_t *const slot = lb + __umul24((uint32_t)ord >> 2, stride4) + (ord & 3);
+                                a = *slot;
+                                *slot = lb[__umul24((uint32_t)count >> 2, stride4) + (count & 3)];  // swap-remove (:209-217)
+                            }
+                        }
+                        while (status == 0) {
+                            // LDS operations keep their program order, so the order below is what hides their latency:
+                            // the current ply's line reads go first and return while the next cell is drawn; the list
+                            // reads of that draw return while the lines are tested.
                             plies++;
                             const uint32_t i = a >> 4, jj = a & 15u;
                             const uint32_t sh = (sel & 2u) << 3;  // 0 for the +1 side, 16 for the -1 side
@@ -463,14 +474,28 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                             uint32_t *const p_ant = lp + __umul24((uint32_t)(m + n + m + n - 1) + i + jj, nt);
                             // the four lines through a cell are four different words: read all, then write all
                             uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
+                            // draw of the next ply (count = cells left after the current one)
+                            const Rng32 rg_now = rg;
+                            uint32_t xl, xh;
+                            rng_next32(rg, xl, xh);
+                            const int ord_n = (int)(uniform_from_bits(xl, xh) * (float)count);
+                            const bool stale_n = ord_n >= count;   // u rounded up to 1.0f: the next ply would read one past the list
+                            const int count_n = count > 0 ? count - 1 : 0;
+                            uint8_t *const slot_n = lb + __umul24((uint32_t)ord_n >> 2, stride4) + (ord_n & 3);
+                            const uint32_t a_n = *slot_n;
+                            const uint8_t last_n = lb[__umul24((uint32_t)count_n >> 2, stride4) + (count_n & 3)];
+                            // the current ply's stone and the test for five
                             const uint32_t bit_j = (1u << jj) << sh;
                             w_row |= bit_j; w_col |= (1u << i) << sh; w_dia |= bit_j; w_ant |= bit_j;
                             *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
                             const uint32_t win_j = (0x1fu << jj) >> 4, win_i = (0x1fu << i) >> 4;  // starts of a run of five through the stone
                             const uint32_t hit = exact_five_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
                             const uint32_t hit2 = exact_five_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
-                            if ((hit | hit2) != 0) { status = 1; outcome = outcome_if_win; }
-                            else if (count == 0) { status = 2; outcome = 0; }
+                            *slot_n = last_n;   // swap-remove of the next draw
+                            if ((hit | hit2) != 0) { status = 1; outcome = outcome_if_win; rg = rg_now; }
+                            else if (count == 0) { status = 2; outcome = 0; rg = rg_now; }
+                            else if (stale_n) status = 3;
+                            count = count_n; a = a_n;
                             outcome_if_win = -outcome_if_win;
                             sel ^= 0x02020202u;
                         }
