@@ -102,6 +102,7 @@ struct SearchArgs {
     int32_t thrifty;        // layout of the actions_expanded row
     float ucb_c;
     int32_t stage_timing;   // accumulate per-stage device time in the tree headers
+    int32_t agent_fences;   // never take the same-XCC shortcuts (full device-scope release and acquire every step)
     int32_t *abort_flag;
     int32_t *queue;         // next tree not yet handed out, or null when every tree has its own workgroups
     uint32_t launch_seq;    // distinguishes the launches that use the queue
@@ -629,7 +630,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 if (step == 0) {
                     const uint32_t mine = (uint32_t)__builtin_amdgcn_s_getreg(6164) & 0xfu;
                     const uint32_t theirs = (lane < G) ? __hip_atomic_load(&hdr->xcc[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : mine;
-                    if (__ballot(theirs != mine) == 0 && lane == 0) s_xcd_local = 1;
+                    if (__ballot(theirs != mine) == 0 && lane == 0 && !args.agent_fences) s_xcd_local = 1;
                 }
                 if (lane < G) { s_gather[lane][0] = (int32_t)((v >> 16) & 0xffffu); s_gather[lane][1] = (int32_t)(v & 0xffffu); }
                 if (__ballot(bad) != 0 && lane == 0) s_abort = 1;

@@ -89,6 +89,7 @@ struct SearchArgs {
     int32_t thrifty;
     float ucb_c;
     int32_t stage_timing;
+    int32_t agent_fences;   // never take the same-XCC shortcuts (full device-scope release and acquire every step)
     int32_t *abort_flag;
 };
 
@@ -699,7 +700,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
             if (step == 0) {
                 bool same = true;
                 for (int q = tid; q < G; q += nthreads) same = same && atomic_load_relaxed(&hdr->xcc[q]) == my_xcc;
-                xcd_local = __syncthreads_and(same) != 0;
+                xcd_local = __syncthreads_and(same) != 0 && !args.agent_fences;
             }
         } else {
             __threadfence_block();

@@ -186,3 +186,27 @@ def test_gomoku_run_batch_in_groups():
         assert batch[k].actions_info == single.actions_info
         for name in ("trees", "ns", "ns_wins"):
             np.testing.assert_array_equal(batch[k].read_array(name, 7), single.read_array(name, 7))
+
+
+@pytest.mark.parametrize("game,variant", [("c4", "acp_prodigal"), ("c4", "acp_thrifty"), ("gomoku", "acp_prodigal")])
+def test_device_scope_fences_give_the_same_trees(game, variant, monkeypatch):
+    """The all-child kernels skip L2 write-backs and invalidations once a tree's workgroups are known to share an
+    XCC.  MCTSNC_AGENT_FENCES keeps them on the general path (full device-scope release and acquire every step), which
+    a device that spreads a tree over XCCs would take; results must not depend on it."""
+    monkeypatch.setenv("MCTSNC_AGENT_FENCES", "1")
+    rng = np.random.default_rng(31)
+    if game == "c4":
+        from oracle.oracle import Oracle
+        params = dict(n_trees=3, n_playouts=64, variant=variant, device_memory=0.25, ucb_c=2.0, seed=5)
+        e = make_engine(params)
+        o = Oracle("c4", (6, 7), 7, 7, 3, 64, variant, ucb_c=2.0, seed=5, device_memory=0.25, threads=8)
+        board, fills, turn = random_c4_root(rng, 9)
+        compare_with_oracle(e, o, board, fills, turn, 300)
+    else:
+        from oracle.oracle import Oracle
+        from helpers import random_gomoku_root
+        params = dict(n_trees=2, n_playouts=64, variant=variant, device_memory=0.5, ucb_c=2.0, seed=5)
+        e = make_engine(params, board_shape=(9, 9), extra=0, actions=81, game="gomoku")
+        o = Oracle("gomoku", (9, 9), 0, 81, 2, 64, variant, ucb_c=2.0, seed=5, device_memory=0.5, threads=8)
+        board, turn = random_gomoku_root(rng, 9, 9, 6)
+        compare_with_oracle(e, o, board, None, turn, 12)
