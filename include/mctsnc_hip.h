@@ -128,7 +128,8 @@ int mctsnc_reseed(mctsnc_engine *e);
 
 /* Runs n engines of identical configuration concurrently, one search each, in a single device pass
  * (no counterpart in the reference, which runs one search at a time; results per engine equal those of
- * mctsnc_run).  boards: n * m*n bytes, extras: n * extra_len bytes or NULL, turns: n entries. */
+ * mctsnc_run; searches beyond what the device holds at once start as earlier ones finish).  boards: n * m*n bytes,
+ * extras: n * extra_len bytes or NULL, turns: n entries. */
 int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
                      const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
                      mctsnc_result *out);
