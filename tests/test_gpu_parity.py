@@ -210,3 +210,29 @@ def test_device_scope_fences_give_the_same_trees(game, variant, monkeypatch):
         o = Oracle("gomoku", (9, 9), 0, 81, 2, 64, variant, ucb_c=2.0, seed=5, device_memory=0.5, threads=8)
         board, turn = random_gomoku_root(rng, 9, 9, 6)
         compare_with_oracle(e, o, board, None, turn, 12)
+
+
+def test_time_limited_batch_over_several_launches_through_the_queue():
+    """A time budget splits a batch into several kernel launches, each of which hands the trees beyond the resident
+    workgroup sets out through the queue again: every search must end where a single search of as many steps ends."""
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    rng = np.random.default_rng(41)
+
+    def mk(limit):
+        e = MCTSNC((6, 7), 7, 7, search_time_limit=limit, search_steps_limit=np.inf, n_trees=4, n_playouts=256,
+                   variant="acp_prodigal", device_memory=0.05, ucb_c=2.0, seed=9, verbose_info=False)
+        e.init_device_side_arrays()
+        return e
+    roots = [random_c4_root(rng, int(rng.integers(4, 20))) for _ in range(72)]
+    batch = [mk(0.05) for _ in roots]
+    run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots])
+    steps = batch[0].steps
+    assert steps > 64 and all(e.steps == steps for e in batch)   # more than the first chunk: at least two launches
+    single = mk(np.inf)
+    for k in (0, 43, 44, 71):
+        single.reseed()
+        single.run(*roots[k], forced_search_steps_limit=steps)
+        assert batch[k].actions_info == single.actions_info
+        for ti in range(4):
+            for name in ("trees", "ns", "ns_wins"):
+                np.testing.assert_array_equal(batch[k].read_array(name, ti), single.read_array(name, ti))
