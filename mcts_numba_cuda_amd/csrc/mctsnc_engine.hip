@@ -517,7 +517,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
-    const dim3 grid(8 * e0->G * ((n_refs + 7) / 8)), block(e0->block);
+    // fewer than 8 trees (all-child-playouts): every tree is spread over 8 / next_pow2(trees) XCDs
+    args.span = (e0->acp && n_refs < 8) ? 8 / next_pow2(n_refs) : 1;
+    const dim3 grid(args.span == 1 ? 8 * e0->G * ((n_refs + 7) / 8) : 8 * ((e0->G + args.span - 1) / args.span)), block(e0->block);
     const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->block);
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
@@ -783,7 +785,8 @@ int mctsnc_init_device(mctsnc_engine *e) {
             HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e->block, lds));
             HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
             const int64_t resident = (int64_t)per_cu * cus;
-            int64_t g_fit = resident / (8 * ((T + 7) / 8));   // the grid is 8 * G * ceil(T / 8) workgroups
+            // the grid is 8 * G * ceil(T / 8) workgroups, or next_pow2(T) * G for fewer than 8 trees
+            int64_t g_fit = resident / (T < 8 ? next_pow2(T) : 8 * ((T + 7) / 8));
             if (g_fit > A) g_fit = A;
             if (g_fit > e->G) e->G = (int)g_fit;
         }
