@@ -479,6 +479,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                             uint32_t *const p_ant = lp + __umul24((uint32_t)(m + n + m + n - 1) + i + jj, nt);
                             // the four lines through a cell are four different words: read all, then write all
                             uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
+                            __builtin_amdgcn_sched_barrier(0);   // the line reads are in flight while the next cell is drawn
                             // draw of the next ply (count = cells left after the current one)
                             const Rng32 rg_now = rg;
                             uint32_t xl, xh;
