@@ -18,7 +18,8 @@ def engines(variant, T, P, m, n, seed=3, device_memory=0.5, **okw):
 
 
 @pytest.mark.parametrize("variant,T,P,steps", [("ocp_thrifty", 4, 128, 60), ("ocp_prodigal", 2, 64, 80),
-                                               ("acp_thrifty", 2, 64, 6), ("acp_prodigal", 1, 128, 5)])
+                                               ("acp_thrifty", 2, 64, 6), ("acp_prodigal", 1, 128, 5),
+                                               ("acp_prodigal", 3, 64, 4), ("acp_thrifty", 5, 64, 3)])
 def test_gomoku_15x15_full_state(variant, T, P, steps):
     """Two consecutive searches on 15x15 (random streams carried over): every per-node array, the step scratch,
     the reduced root table and the generator states must equal the oracle's."""
