@@ -732,10 +732,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                         key = (((unsigned long long)__float_as_uint(ucb) + 1ull) << 8) | (unsigned long long)(7u - bitrev3((uint32_t)a));
                     }
                 }
-                for (int off = 1; off < 8; off <<= 1) {
-                    const unsigned long long o = __shfl_xor(key, off);
-                    key = o > key ? o : key;
-                }
+                key = max_over_8_lanes(key);
                 if (lvl < n_levels && a == 0) {
                     const uint32_t best = bitrev3(7u - (uint32_t)(key & 0xffull));
                     s_rec[lvl][kDwMask] = (s_rec[lvl][kDwMask] & 0x00ffffffu) | (best << 24);
