@@ -33,7 +33,7 @@ N_ROOTS = 64
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per search-kernel launch from rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy gives) and WRITE_SIZE
 # (x1), averaged over the first four roots: (5299.5 * 2 + 8909.5) KiB
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 19857203
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 20125389
 
 
 def has_four(board, token):
