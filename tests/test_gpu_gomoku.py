@@ -69,3 +69,11 @@ def test_gomoku_sixteen_wide_boards(variant):
         e, o = engines(variant, 2, 64, m, n)
         board, turn = random_gomoku_root(rng, m, n, 6)
         compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else max(3, steps // 10))
+
+
+def test_gomoku_all_child_playouts_in_rounds():
+    """n_playouts = 512 with all-child-playouts: every child's playouts run in two rounds of 256, one tree spread over
+    all XCDs."""
+    e, o = engines("acp_thrifty", 1, 512, 9, 9)
+    board, turn = random_gomoku_root(np.random.default_rng(5), 9, 9, 5)
+    compare_with_oracle(e, o, board, None, turn, 3)
