@@ -41,7 +41,6 @@ struct GomokuArgs {
 struct Lds {
     int want[kMaxWavesPerBlock];
     uint32_t board[kMaxWavesPerBlock][kBoardWords];
-    alignas(16) uint32_t keys[kMaxWavesPerBlock][kEdges];
 };
 
 __device__ __forceinline__ uint64_t wave_sum64(uint64_t v) {
@@ -82,11 +81,53 @@ __device__ __forceinline__ bool makes_five(const uint32_t *mine, int cell, int m
     return __ballot(hit) != 0;
 }
 
+// Bitonic sort of the wavefront's 256 keys, largest first: element e = 4 * lane + k lives in v[k] of `lane`.  Partners
+// at element distance 1 and 2 are registers of the same lane; lane distances 1, 2 and 8 are DPP moves, 4 and 16 LDS
+// swizzles (no memory), 32 an LDS permute.
+template <int LANE_XOR>
+__device__ __forceinline__ uint32_t from_lane_xor(uint32_t x, int lane) {
+    if (LANE_XOR == 1) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xf, 0xf, true);    // quad_perm [1,0,3,2]
+    if (LANE_XOR == 2) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xf, 0xf, true);    // quad_perm [2,3,0,1]
+    if (LANE_XOR == 8) return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x128, 0xf, 0xf, true);   // row_ror:8
+    if (LANE_XOR == 4) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x101F);                      // bit mode: xor 4
+    if (LANE_XOR == 16) return (uint32_t)__builtin_amdgcn_ds_swizzle((int)x, 0x401F);                     // bit mode: xor 16
+    return (uint32_t)__builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, (int)x);
+}
+template <int SIZE, int DIST>
+__device__ __forceinline__ void bitonic_step(uint32_t (&v)[4], int lane) {
+    uint32_t p[4];
+    if (DIST < 4) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) p[k] = v[k ^ DIST];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) p[k] = from_lane_xor<DIST / 4>(v[k], lane);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int e = 4 * lane + k;
+        const bool descending = (e & SIZE) == 0, first = (e & DIST) == 0;   // SIZE == 256: every block descends
+        const uint32_t hi = v[k] > p[k] ? v[k] : p[k], lo = v[k] > p[k] ? p[k] : v[k];
+        v[k] = (first == descending) ? hi : lo;
+    }
+}
+template <int SIZE, int DIST>
+__device__ __forceinline__ void bitonic_merge(uint32_t (&v)[4], int lane) {
+    bitonic_step<SIZE, DIST>(v, lane);
+    if constexpr (DIST > 1) bitonic_merge<SIZE, DIST / 2>(v, lane);
+}
+template <int SIZE>
+__device__ __forceinline__ void bitonic_sort(uint32_t (&v)[4], int lane) {
+    if constexpr (SIZE > 2) bitonic_sort<SIZE / 2>(v, lane);
+    bitonic_merge<SIZE, SIZE / 2>(v, lane);
+}
+__device__ __forceinline__ void sort_keys_descending(uint32_t (&v)[4], int lane) { bitonic_sort<256>(v, lane); }
+
 // Priors of a new node: one Gamma weight per legal cell, prior = weight / sum, edge slots in descending weight order
 // (ties: smaller cell first), so that progressive widening opens the most promising moves first.  Initialises every
-// edge field of the node's legal slots.  `keys` is this wavefront's LDS scratch.
-__device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint32_t *board, uint32_t *keys, int lane,
-                             uint64_t board_hash, int n_legal) {
+// edge field of the node's legal slots.  All 64 lanes must call it together.
+__device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint32_t *board, int lane, uint64_t board_hash,
+                             int n_legal) {
     constexpr int kPer = kEdges / kWave;
     uint32_t mine[kPer];
     // Rejection sampling diverges between lanes; every lane walks through its own cells and rounds independently, so
@@ -119,35 +160,22 @@ __device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint
     }
     uint64_t sum = 0;
 #pragma unroll
-    for (int k = 0; k < kPer; ++k) {
-        keys[lane + k * kWave] = mine[k];
-        sum += mine[k] ? psyn_key_weight(mine[k]) : 0;
-    }
+    for (int k = 0; k < kPer; ++k) sum += mine[k] ? psyn_key_weight(mine[k]) : 0;
     sum = wave_sum64(sum);
-    wave_lds_fence();
-    int rank[kPer];
-#pragma unroll
-    for (int k = 0; k < kPer; ++k) rank[k] = 0;
-    const uint4 *keys4 = reinterpret_cast<const uint4 *>(keys);
-    for (int o = 0; o < kEdges / 4; ++o) {
-        const uint4 q = keys4[o];
-#pragma unroll
-        for (int k = 0; k < kPer; ++k)
-            rank[k] += (q.x > mine[k] ? 1 : 0) + (q.y > mine[k] ? 1 : 0) + (q.z > mine[k] ? 1 : 0) + (q.w > mine[k] ? 1 : 0);
-    }
-    const size_t erow = ((size_t)tree * g.sel.nodes + node) * kEdges;
+    // slot of a cell = rank of its key among the node's keys, largest first (0 = not a legal cell: last)
+    sort_keys_descending(mine, lane);
+    const size_t erow = ((size_t)tree * g.sel.nodes + node) * kEdges + (size_t)kPer * lane;
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
         if (mine[k] == 0u) continue;
-        const size_t e = erow + rank[k];
+        const size_t e = erow + k;
         g.edge_prior[e] = psyn_prior(psyn_key_weight(mine[k]), sum, n_legal);
-        g.edge_action[e] = (uint8_t)(lane + k * kWave);
+        g.edge_action[e] = (uint8_t)(255u - (mine[k] & 0xFFu));
         g.edge_child[e] = -1;
         g.edge_N[e] = 0;
         g.edge_W[e] = 0.0f;
         g.edge_inflight[e] = 0;
     }
-    wave_lds_fence();
 }
 
 // Expansion / evaluation of one step for the traversals of one tree; all wavefronts of the workgroup call it.
@@ -215,7 +243,7 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
             g.edge_W[erow + slot] = -v_child;
             atomicAdd(&g.node_expanded[trow + node], 1);
         }
-        if (!terminal) write_priors(g, tree, child, board, lds.keys[wave], lane, bh, child_legal);
+        if (!terminal) write_priors(g, tree, child, board, lane, bh, child_legal);
         u = -v_child;
     } else if (kind == PUCT_SELECT_TERMINAL) {
         u = g.node_value[trow + node];
@@ -232,7 +260,6 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
 // Root of every tree: node 0 with the root position and its priors.
 __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const uint32_t *root_board, int root_turn) {
     __shared__ uint32_t board[kBoardWords];
-    __shared__ alignas(16) uint32_t weight[kEdges];
     const int tree = blockIdx.x, lane = threadIdx.x;
     const size_t trow = (size_t)tree * g.sel.nodes;
     const uint32_t w = lane < kBoardWords ? root_board[lane] : 0u;
@@ -251,7 +278,7 @@ __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const u
         g.node_legal[trow] = n_legal;
         g.node_count[tree] = 1;
     }
-    if (n_legal > 0) write_priors(g, tree, 0, board, weight, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
+    if (n_legal > 0) write_priors(g, tree, 0, board, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
 }
 
 // Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one.  All wavefronts of a
