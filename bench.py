@@ -374,7 +374,7 @@ def main():
         device_synchronize()
         elapsed = time.perf_counter() - t0
 
-        batched = None
+        batched = trees_512 = None
         if not args.no_batched:
             # the same 64 searches, all handed to the device at once (one launch: the resident sets of workgroups take
             # further trees from a queue as they finish theirs); results are identical to the sequential runs
@@ -395,6 +395,22 @@ def main():
             for e in engines[1:]:
                 e._release()
             del engines
+            # the widest search the reference's interface allows (n_trees=512, its MAX_N_TREES): the tree traffic of
+            # one search is large enough here for the HBM fraction to mean something
+            wide = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=512, n_playouts=P,
+                          variant="acp_prodigal", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
+            wide.init_device_side_arrays()
+            b, f, t = np.zeros((M, N), np.int8), np.zeros(N, np.int8), 1     # empty board
+            for rep in range(2):
+                wide.reseed()
+                t1 = time.perf_counter()
+                wide.run(b, f, t)
+                wt = time.perf_counter() - t1
+            wbytes = algorithmic_bytes(wide._result, wide.steps * 512)["total"]
+            trees_512 = {"n_trees": 512, "root": "empty board", "playouts_per_s": wide.performance_info["playouts"] / wt, "ms_per_search": wt * 1e3,
+                         "mcts_steps_per_s": wide.steps / wt, "tree_steps_per_s": wide.steps * 512 / wt,
+                         "algorithmic_GB_per_s": wbytes / wt / 1e9, "hbm_frac": wbytes / wt / 1e9 / HBM_PEAK_GBS}
+            wide._release()
         eng._release()      # free the pools now rather than at interpreter exit, after the HIP runtime has shut down
 
     value = playouts / elapsed
@@ -454,7 +470,7 @@ def main():
            "mcts_steps_per_s": mcts_steps / elapsed,
            "device_loop_share": dev_time / elapsed,
            "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
-           "batched": batched,
+           "batched": batched, "trees_512": trees_512,
            "roofline": roofline, "cpu_baseline": cpu_baseline, "cpu_mcts": cpu_mcts}
     print(json.dumps(out))
 

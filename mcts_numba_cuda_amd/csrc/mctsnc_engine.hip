@@ -519,17 +519,36 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
     // fewer than 8 trees (all-child-playouts): every tree is spread over 8 / next_pow2(trees) XCDs
     args.span = (e0->acp && n_refs < 8) ? 8 / next_pow2(n_refs) : 1;
-    const dim3 grid(args.span == 1 ? 8 * e0->G * ((n_refs + 7) / 8) : 8 * ((e0->G + args.span - 1) / args.span)), block(e0->block);
+    const dim3 block(e0->block);
     const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->block);
+    // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
+    // whole: more trees than the device holds rows of 8 * G workgroups for are searched by consecutive launches over
+    // equal groups of trees, every group for the same number of steps before the budget is looked at again.
+    int group = n_refs;
+    if (e0->acp && args.span == 1) {
+        int per_cu = 0, cus = 0;
+        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
+        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block, lds));
+        const int64_t rows = (int64_t)per_cu * cus / (8 * e0->G);
+        if (rows < 1) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * e0->G);
+        const int64_t n_groups = ((n_refs + 7) / 8 + rows - 1) / rows;
+        group = (int)(8 * (((n_refs + 7) / 8 + n_groups - 1) / n_groups));
+        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees, %d workgroups per tree, %d resident workgroups per CU: launches of %d trees\n", n_refs, e0->G, per_cu, group);
+    }
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
         args.nsteps = nsteps;
-        if (e0->acp) {
-            void *kargs[] = {&args};
-            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
-        } else {
-            hipLaunchKernelGGL(gomoku::search_kernel<false>, grid, block, lds, stream, args);
-            HIP_TRY(hipGetLastError());
+        for (int start = 0; start < n_refs; start += group) {
+            args.refs = d_refs + start;
+            args.n_refs = std::min(group, n_refs - start);
+            if (e0->acp) {
+                const dim3 grid(args.span == 1 ? 8 * e0->G * ((args.n_refs + 7) / 8) : 8 * ((e0->G + args.span - 1) / args.span));
+                void *kargs[] = {&args};
+                HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+            } else {
+                hipLaunchKernelGGL(gomoku::search_kernel<false>, dim3(8 * ((args.n_refs + 7) / 8)), block, lds, stream, args);
+                HIP_TRY(hipGetLastError());
+            }
         }
         return MCTSNC_OK;
     }, steps, dev_time, time_loop);
@@ -576,34 +595,8 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     mctsnc_engine *e0 = engines[0];
     const mctsnc_config &c = e0->cfg;
     HIP_TRY(hipSetDevice(c.device));
-    // The all-children-playouts kernels synchronise workgroups of one tree with each other, so a launch must be fully
-    // resident: a batch whose grid exceeds what the device holds at once runs as consecutive groups of searches, each
-    // with the whole budget.
-    int group = n;
-    if (e0->acp && n > 1 && e0->is_gomoku()) {
-        int per_cu = 0, cus = 0;
-        HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block,
-                                                             gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e0->block)));
-        // the grid is 8 * G * ceil(refs / 8) workgroups
-        group = (int)std::max<int64_t>(1, ((int64_t)per_cu * cus / (8 * e0->G) * 8) / c.n_trees);
-        group = std::min(group, n);
-        const int n_groups = (n + group - 1) / group;
-        group = (n + n_groups - 1) / n_groups;   // groups of equal size
-        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] batch of %d: %d resident workgroups per CU, groups of %d\n", n, per_cu, group);
-    }
-    const size_t cells = (size_t)c.board_m * c.board_n;
-    for (int start = 0; start < n; start += group) {
-        const int k = std::min(group, n - start);
-        const int8_t *b = boards + (size_t)start * cells;
-        if (e0->is_gomoku())
-            rc = run_many_gomoku(engines + start, k, b, turns + start, bud, out + start);
-        else
-            rc = run_many_c4(engines + start, k, b, extras ? extras + (size_t)start * extra_len : nullptr, extra_len, turns + start, bud,
-                             out + start);
-        if (rc) return rc;
-    }
-    return MCTSNC_OK;
+    if (e0->is_gomoku()) return run_many_gomoku(engines, n, boards, turns, bud, out);
+    return run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out);
 }
 
 int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t need) {
@@ -786,9 +779,9 @@ int mctsnc_init_device(mctsnc_engine *e) {
             HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
             const int64_t resident = (int64_t)per_cu * cus;
             // the grid is 8 * G * ceil(T / 8) workgroups, or next_pow2(T) * G for fewer than 8 trees
+            // (more trees than the device holds workgroups: one workgroup per tree, several launches per step budget)
             int64_t g_fit = resident / (T < 8 ? next_pow2(T) : 8 * ((T + 7) / 8));
-            if (g_fit > A) g_fit = A;
-            if (g_fit > e->G) e->G = (int)g_fit;
+            e->G = (int)std::min<int64_t>(std::max<int64_t>(g_fit, 1), A);
         }
     }
     int rc = upload_rng(e);

@@ -77,3 +77,15 @@ def test_gomoku_all_child_playouts_in_rounds():
     e, o = engines("acp_thrifty", 1, 512, 9, 9)
     board, turn = random_gomoku_root(np.random.default_rng(5), 9, 9, 5)
     compare_with_oracle(e, o, board, None, turn, 3)
+
+
+@pytest.mark.parametrize("variant,T,steps", [("acp_thrifty", 20, 3), ("acp_prodigal", 40, 3), ("acp_prodigal", 512, 2),
+                                             ("ocp_thrifty", 512, 12)])
+def test_gomoku_many_trees(variant, T, steps):
+    """More trees than the device holds 32 workgroups each for: fewer workgroups per tree, down to one, and past that
+    consecutive launches over groups of trees (n_trees = 512 is the reference's MAX_N_TREES, src/mctsnc.py:195)."""
+    rng = np.random.default_rng(21)
+    e, o = engines(variant, T, 32, 15, 15, seed=5, device_memory=2.0)
+    for stones in (8, 1):
+        board, turn = random_gomoku_root(rng, 15, 15, stones)
+        compare_with_oracle(e, o, board, None, turn, steps)

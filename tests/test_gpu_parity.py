@@ -84,6 +84,20 @@ def test_against_oracle_full_state(variant, T, P):
         compare_with_oracle(e, o, board, fills, turn, steps=150 if P >= 256 else 300)
 
 
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
+def test_widest_search_512_trees(variant):
+    """n_trees = 512 is the reference's MAX_N_TREES (src/mctsnc.py:195): more trees than the device holds sets of
+    workgroups for, so the all-children kernel takes trees from its queue within one search."""
+    rng = np.random.default_rng(77)
+    params = dict(n_trees=512, n_playouts=32, variant=variant, device_memory=1.0, ucb_c=2.0, seed=5)
+    e = make_engine(params)
+    from oracle.oracle import Oracle
+    o = Oracle("c4", (6, 7), 7, 7, 512, 32, variant, ucb_c=2.0, seed=5, device_memory=1.0, threads=8)
+    for plies in (10, 3):
+        board, fills, turn = random_c4_root(rng, plies)
+        compare_with_oracle(e, o, board, fills, turn, steps=40)
+
+
 def test_run_batch_equals_single_runs():
     """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
     from mcts_numba_cuda_amd import run_batch
