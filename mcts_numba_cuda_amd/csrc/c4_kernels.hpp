@@ -215,7 +215,7 @@ __device__ inline int exact_playout(ExactScratch &s, const Geometry &g, uint64_t
 
 struct BB { uint32_t lo, hi; };
 
-__device__ __forceinline__ BB bb_shr(BB x, int s) {  // 0 < s < 32
+__device__ __forceinline__ BB bb_shr(BB x, int s) {  // 0 < s < 32 (the largest is 2 * (rows + 2))
     BB r; r.lo = __builtin_amdgcn_alignbit(x.hi, x.lo, s); r.hi = x.hi >> s; return r;
 }
 __device__ __forceinline__ BB bb_and(BB a, BB b) { BB r; r.lo = a.lo & b.lo; r.hi = a.hi & b.hi; return r; }
@@ -265,7 +265,7 @@ __device__ __forceinline__ int fast_playout(const Geometry &g, uint64_t cur, uin
         const int sh = ord * 4;
         const int c = (int)((list >> sh) & 7u);
         const int c4 = c * 4;
-        const int h = (int)((fills >> c4) & 7u);
+        const int h = (int)((fills >> c4) & 15u);
         const int pos = c * H + h;
         const uint32_t bit = 1u << (pos & 31);
         a.lo |= (pos < 32) ? bit : 0u;

@@ -665,8 +665,9 @@ int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
     const mctsnc_config &c = *cfg;
     if (c.game != MCTSNC_GAME_C4 && c.game != MCTSNC_GAME_GOMOKU) return fail(MCTSNC_E_INVALID, "unknown game %d", c.game);
     if (c.game == MCTSNC_GAME_C4) {
-        if (c.board_m < 1 || c.board_n < 1 || c.board_n > c4::kMaxCols || (c.board_m + 1) * c.board_n > 64)
-            return fail(MCTSNC_E_INVALID, "Connect 4 board %dx%d unsupported: needs columns <= %d and (rows + 1) * columns <= 64", c.board_m, c.board_n, c4::kMaxCols);
+        // 13 rows: the playout keeps column fills in 4-bit fields and shifts 32-bit halves by up to 2 * (rows + 2)
+        if (c.board_m < 1 || c.board_n < 1 || c.board_n > c4::kMaxCols || c.board_m > 13 || (c.board_m + 1) * c.board_n > 64)
+            return fail(MCTSNC_E_INVALID, "Connect 4 board %dx%d unsupported: needs columns <= %d, rows <= 13 and (rows + 1) * columns <= 64", c.board_m, c.board_n, c4::kMaxCols);
         if (c.max_actions != c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 has one action per column (%d), got max_actions = %d", c.board_n, c.max_actions);
         if (c.extra_info_memory < c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 keeps the column fills in extra_info: needs >= %d bytes", c.board_n);
     } else {

@@ -61,7 +61,7 @@ def test_configuration_errors_are_reported(L):
     from mcts_numba_cuda_amd import _lib
     good = dict(game=0, board_m=6, board_n=7, extra_info_memory=7, max_actions=7, n_trees=4, n_playouts=256, variant=3, ucb_c=2.0,
                 seed=0, max_tree_size=1000, device=0)
-    bad_cases = [dict(game=7), dict(board_n=9), dict(board_m=9), dict(max_actions=6), dict(n_playouts=100), dict(n_playouts=1024),
+    bad_cases = [dict(game=7), dict(board_n=9), dict(board_m=9), dict(board_m=14, board_n=4, max_actions=4), dict(max_actions=6), dict(n_playouts=100), dict(n_playouts=1024),
                  dict(n_trees=0), dict(variant=4), dict(ucb_c=-1.0), dict(max_tree_size=0), dict(max_tree_size=2**24 + 1),
                  dict(extra_info_memory=3)]
     for bad in bad_cases:

@@ -98,6 +98,21 @@ def test_widest_search_512_trees(variant):
         compare_with_oracle(e, o, board, fills, turn, steps=40)
 
 
+@pytest.mark.parametrize("m,n", [(4, 5), (5, 6), (8, 7), (7, 8), (6, 8), (12, 4), (13, 4), (10, 5)])
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "acp_prodigal"])
+def test_other_connect4_boards(m, n, variant):
+    """Boards other than 6x7 up to what a 64-bit column-major bitboard with one spare row holds: small ones end in
+    draws and full columns within a few steps, 7x8 and 8x7 use the last bits, 13 rows is the tallest board."""
+    rng = np.random.default_rng(100 * m + n)
+    params = dict(n_trees=3, n_playouts=64, variant=variant, device_memory=0.25, ucb_c=2.0, seed=9)
+    e = make_engine(params, board_shape=(m, n), extra=n, actions=n)
+    from oracle.oracle import Oracle
+    o = Oracle("c4", (m, n), n, n, 3, 64, variant, ucb_c=2.0, seed=9, device_memory=0.25, threads=8)
+    for plies in (2, m * n // 2):
+        board, fills, turn = random_c4_root(rng, plies, m, n)
+        compare_with_oracle(e, o, board, fills, turn, steps=250)
+
+
 def test_run_batch_equals_single_runs():
     """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
     from mcts_numba_cuda_amd import run_batch
