@@ -113,6 +113,29 @@ def test_other_connect4_boards(m, n, variant):
         compare_with_oracle(e, o, board, fills, turn, steps=250)
 
 
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
+def test_small_playout_counts_and_exploration_constants(variant):
+    """n_playouts below a wavefront (down to one playout per node), ucb_c = 0 (pure exploitation: ties everywhere) and
+    other constants, a budget of a single step, on both games."""
+    from helpers import random_gomoku_root
+    from oracle.oracle import Oracle
+    rng = np.random.default_rng(5)
+    for P, c in ((1, 2.0), (2, 0.0), (4, 0.5), (16, 7.25)):
+        params = dict(n_trees=2, n_playouts=P, variant=variant, device_memory=0.25, ucb_c=c, seed=13)
+        e = make_engine(params)
+        o = Oracle("c4", (6, 7), 7, 7, 2, P, variant, ucb_c=c, seed=13, device_memory=0.25, threads=8)
+        for plies, steps in ((6, 1), (14, 300)):
+            board, fills, turn = random_c4_root(rng, plies)
+            compare_with_oracle(e, o, board, fills, turn, steps=steps)
+    for P, c in ((1, 2.0), (8, 0.0), (16, 1.0)):
+        params = dict(n_trees=2, n_playouts=P, variant=variant, device_memory=0.5, ucb_c=c, seed=13)
+        e = make_engine(params, board_shape=(15, 15), extra=0, actions=225, game="gomoku")
+        o = Oracle("gomoku", (15, 15), 0, 225, 2, P, variant, ucb_c=c, seed=13, device_memory=0.5, threads=8)
+        for stones, steps in ((3, 1), (10, 30 if variant.startswith("ocp") else 4)):
+            board, turn = random_gomoku_root(rng, 15, 15, stones)
+            compare_with_oracle(e, o, board, None, turn, steps)
+
+
 def test_run_batch_equals_single_runs():
     """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
     from mcts_numba_cuda_amd import run_batch
