@@ -69,6 +69,18 @@ def test_recorded_games(archives, pair):
     assert n >= 5
 
 
+def test_first_recorded_game_of_every_archive(archives):
+    """The reference's experiments cover every (variant, n_trees, n_playouts) combination it was run with on
+    Connect 4; the first game of each archive (root tables, best actions and tree statistics of every search, in the
+    recorded order and with the recorded step counts) must come out of the HIP engine unchanged."""
+    total = 0
+    for key in sorted(archives):
+        n = replay.replay_archive(archives[key], make_engine, engine_run_search, max_games=1)
+        assert n >= 3, key
+        total += n
+    assert total > 700
+
+
 @pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
 @pytest.mark.parametrize("T,P", [(1, 32), (3, 64), (4, 256), (9, 128)])
 def test_against_oracle_full_state(variant, T, P):
