@@ -12,11 +12,14 @@ Outputs:
                                       ns_wins; plus the last step's scratch arrays.
   * archive_games.json                for every archive: engine parameters and, for the first games,
                                       the ordered list of moves and MCTSNC / MCTS searches.
+  * north_star_experiment.json.gz     all 100 games of the experiment with acp_prodigal 4x256 against the CPU
+                                      player (moves and MCTSNC searches only), in the same format.
 
 Usage: python tests/golden/make_fixtures.py [/root/reference]
 """
 import ast
 import glob
+import gzip
 import json
 import os
 import re
@@ -90,10 +93,31 @@ def condense_archives(ref_root, out):
     json.dump(res, open(out, "w"), separators=(",", ":"))
 
 
+NORTH_STAR = "mcts_5_inf_vanilla;mctsnc_5_inf_4_256_acp_prodigal;C4_6x7"
+
+
+def condense_whole_experiment(ref_root, out):
+    path = [p for p in glob.glob(os.path.join(ref_root, "experiments", "*.zip")) if NORTH_STAR in p][0]
+    name = os.path.basename(path)
+    z = zipfile.ZipFile(path)
+    log = z.read([n for n in z.namelist() if n.endswith(".log")][0]).decode()
+    games = parse_log(log, 10 ** 6)
+    engines = {}
+    for g in games:
+        g["events"] = [e for e in g["events"] if e["type"] in ("move", "mctsnc")]
+        for side in ("black", "white"):
+            inst = parse_instance(g[side])
+            if inst:
+                engines[g[side]] = inst
+    with gzip.GzipFile(out, "wb", mtime=0) as f:
+        f.write(json.dumps({"archive": name, "engines": engines, "games": games}, separators=(",", ":")).encode())
+
+
 if __name__ == "__main__":
     ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
     for variant in ("ocp_thrifty", "acp_thrifty"):
         condense_dump(os.path.join(ref, "extras", f"mctsnc_{variant}_c4_1000steps.json"),
                       os.path.join(HERE, f"dump_{variant}_c4_1000steps.npz"))
     condense_archives(ref, os.path.join(HERE, "archive_games.json"))
+    condense_whole_experiment(ref, os.path.join(HERE, "north_star_experiment.json.gz"))
     print("fixtures written to", HERE)

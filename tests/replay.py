@@ -18,6 +18,14 @@ def load_archives():
         return json.load(f)
 
 
+def load_whole_experiment():
+    """All 100 games of the reference's experiment with acp_prodigal 4x256 against its CPU player (moves and MCTSNC
+    searches), shaped like one entry of load_archives()."""
+    import gzip
+    with gzip.open(os.path.join(GOLDEN, "north_star_experiment.json.gz"), "rt") as f:
+        return json.load(f)
+
+
 def find_archive(archives, a, b=None):
     """Key of the archive whose two AI short names are (a, b) in either order; b=None matches any."""
     for key in archives:

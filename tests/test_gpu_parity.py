@@ -46,6 +46,15 @@ def test_north_star_a100_game(archives):
     assert n >= 10
 
 
+def test_north_star_whole_experiment():
+    """All 100 games of that experiment, 1362 searches with 7.4 million MCTS steps in the recorded order: the engine's
+    random streams run on from search to search and from game to game as the reference's single instance did."""
+    entry = replay.load_whole_experiment()
+    assert len(entry["games"]) == 100
+    n = replay.replay_archive(entry, make_engine, engine_run_search)
+    assert n == 1362
+
+
 ARCHIVE_PAIRS = [
     ("mcts_5_inf_vanilla", "mctsnc_1_inf_1_32_ocp_thrifty"),
     ("mcts_5_inf_vanilla", "mctsnc_1_inf_2_64_ocp_prodigal"),
