@@ -301,8 +301,13 @@ template <typename Launch>
 int budget_loop(mctsnc_engine *e0, const Budget &bud, Launch launch, int64_t &steps, double &dev_time, double &time_loop) {
     hipStream_t stream = e0->stream;
     const bool forced = bud.forced < INFINITY;
-    const double step_budget = forced ? bud.forced : bud.steps_limit;
+    double step_budget = forced ? bud.forced : bud.steps_limit;
     const double time_budget = forced ? INFINITY : bud.time_limit;
+    // The visit counters are int32 as in the reference (src/mctsnc.py:334-335); a root gains at most n_playouts (one
+    // child) or n_playouts * max_actions (all children) visits per step.  The reference would wrap around silently --
+    // at its speed it never gets there; here the search ends before a counter can overflow.
+    const double counter_cap = std::floor(2147483647.0 / ((double)e0->cfg.n_playouts * (e0->acp ? e0->cfg.max_actions : 1)));
+    if (step_budget > counter_cap) step_budget = counter_cap;
     steps = 0;
     dev_time = 0.0;
     const double t_loop = now_s();

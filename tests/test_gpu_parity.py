@@ -157,6 +157,24 @@ def test_small_playout_counts_and_exploration_constants(variant):
             compare_with_oracle(e, o, board, None, turn, steps)
 
 
+def test_search_ends_before_visit_counters_overflow():
+    """512 playouts on each of 7 children add up to 3584 visits of the root per step: its int32 counter (the reference's
+    dtype, src/mctsnc.py:334) would overflow after 599 186 steps, which this engine reaches within seconds.  The search
+    ends there, whatever the limits say, with every count still exact."""
+    from mcts_numba_cuda_amd import MCTSNC
+    e = MCTSNC((6, 7), 7, 7, search_time_limit=60.0, search_steps_limit=np.inf, n_trees=1, n_playouts=512, variant="acp_prodigal",
+               device_memory=1.0, ucb_c=2.0, seed=1, verbose_info=False)
+    e.init_device_side_arrays()
+    e.run(np.zeros((6, 7), np.int8), np.zeros(7, np.int8), 1)
+    cap = (2**31 - 1) // (512 * 7)
+    assert e.steps == cap
+    info = e.actions_info
+    n_root = info["best"]["n_root"]
+    assert 2**30 < n_root <= cap * 512 * 7 < 2**31    # fewer than 7 children deep in the tree
+    assert sum(entry["n"] for a, entry in info.items() if a != "best") == n_root
+    assert e.time_total < 30.0
+
+
 def test_run_batch_equals_single_runs():
     """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
     from mcts_numba_cuda_amd import run_batch
