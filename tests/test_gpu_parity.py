@@ -38,6 +38,33 @@ def test_reference_tree_dump_1000_steps(variant):
             np.testing.assert_array_equal(e.read_array("playout_outcomes_children", ti), d["playout_outcomes_children"][ti])
 
 
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "acp_thrifty"])
+def test_json_dump_equals_reference_dump(variant, tmp_path):
+    """MCTSNC._json_dump (src/mctsnc.py:2377-2462) of the same run, condensed by the routine that condensed the
+    reference's own dump file into the fixture: every array and the recorded parameters come out identical."""
+    import importlib.util
+    from mcts_numba_cuda_amd import MCTSNC
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOLDEN, "make_fixtures.py"))
+    make_fixtures = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(make_fixtures)
+    e = MCTSNC((6, 7), 7, 7, search_time_limit=np.inf, search_steps_limit=1000, n_trees=4, n_playouts=128, variant=variant,
+               device_memory=1.5, ucb_c=2.0, seed=0, verbose_info=False)
+    e.init_device_side_arrays()
+    e.run(np.zeros((6, 7), np.int8), np.zeros(7, np.int8), 1)
+    e._json_dump(str(tmp_path / "dump.json"))
+    make_fixtures.condense_dump(str(tmp_path / "dump.json"), str(tmp_path / "dump.npz"))
+    mine, ref = np.load(tmp_path / "dump.npz"), np.load(os.path.join(GOLDEN, f"dump_{variant}_c4_1000steps.npz"))
+    assert sorted(mine.files) == sorted(ref.files)
+    for key in ref.files:
+        if key == "selected_paths":     # entries past a path's length are whatever earlier steps left there
+            for ti in range(4):
+                length = int(ref[key][ti, -1])
+                assert int(mine[key][ti, -1]) == length
+                np.testing.assert_array_equal(mine[key][ti, :length], ref[key][ti, :length])
+        else:
+            np.testing.assert_array_equal(mine[key], ref[key], err_msg=key)
+
+
 def test_north_star_a100_game(archives):
     """Game 1 of the reference's A100 experiment with acp_prodigal 4x256 (5 s per move): every search's root table,
     best action and tree statistics, with the random streams carried from search to search."""
