@@ -78,12 +78,11 @@ def device_synchronize():
         raise RuntimeError(f"hipDeviceSynchronize failed with {rc}")
 
 
-def algorithmic_bytes(res, tree_steps, acp=True):
+def algorithmic_bytes(res, tree_steps, acp=True, mn_e=M * N + A, A=A, P=P):
     """Bytes the reference's arrays would move for the work counted on the device (element sizes of
     src/mctsnc.py:326-348): selection reads per level a leaf flag, the parent's visit count, the child row and the
     children's (ns, ns_wins); expansion reads the selected state and writes k children; each played-out node reads
     its state and reads + writes P generator states; backup updates k children and L + 1 path nodes."""
-    mn_e = M * N + A
     levels, children, expanded, played = res.stat_levels, res.stat_children, res.stat_expanded, res.stat_played
     select = levels * (1 + 4 + 4 * A) + 8 * children + tree_steps * (1 + 4) + 4 * (levels + tree_steps)
     expand = tree_steps * (mn_e + 6 + 4 * A + 2 * (A + 2)) + expanded * (mn_e + 18)
@@ -218,6 +217,7 @@ def bench_gomoku(args):
             e.run(roots[w][0], None, roots[w][1])
         playouts = mcts_steps = plies = 0
         dev = 0.0
+        alg = dict(select=0, expand=0, playout=0, backup=0, total=0)
         t0 = time.perf_counter()
         for k in range(steps):
             e.reseed()
@@ -226,6 +226,9 @@ def bench_gomoku(args):
             mcts_steps += e.steps
             plies += e.performance_info["playout_plies"]
             dev += e.time_device_loop
+            ab = algorithmic_bytes(e._result, e.steps * 4, acp=False, mn_e=225 + 1, A=225, P=128)
+            for key in alg:
+                alg[key] += ab[key]
         wall = time.perf_counter() - t0
     cpu = None
     if not args.no_cpu_baseline:
@@ -244,7 +247,14 @@ def bench_gomoku(args):
            "config": {"workload": "Gomoku 15x15, seeded roots with 0-20 random stones, ocp_thrifty n_trees=4 n_playouts=128 ucb_c=2.0 "
                                   "search_steps_limit=2000 device_memory=16GiB seed=0; one MCTSNC.run() per root, sequential"},
            "mcts_steps_per_s": mcts_steps / wall, "playout_plies_per_s": plies / dev, "device_loop_share": dev / wall,
-           "roofline": None, "cpu_baseline": cpu}
+           "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "kernel": "mctsnc::gomoku::search_kernel<false>", "algorithmic_bytes_per_launch": alg["total"] / steps,
+                        "avg_launch_ms": dev / steps * 1e3,
+                        "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
+                        "note": "four workgroups of two wavefronts: bound by the length of the longest playout "
+                                "(about 105 instructions per ply on a lone wavefront), not by memory"},
+           "cpu_baseline": cpu}
     e._release()
     print(json.dumps(out))
 
