@@ -137,3 +137,12 @@ def test_puct_library_exports_every_declared_symbol(tmp_path):
     src.write_text(f'#include "{header}"\nint main(void) {{ return PUCT_SELECT_BUSY == 4 ? 0 : 1; }}\n')
     subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-c", "-o", str(tmp_path / "probe.o"), str(src)])
     assert (puct.PACKED_KIND_SHIFT, puct.PACKED_SLOT_SHIFT, puct.PACKED_REASON_SHIFT) == (22, 14, 25)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits with an error instead of printing a figure."""
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
+    assert not r.stdout.strip().startswith("{")
