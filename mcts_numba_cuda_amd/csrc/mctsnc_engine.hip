@@ -419,7 +419,16 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
     const dim3 block(e0->block);
-    const size_t lds = c4::search_lds_bytes(c.board_m, c.board_n);
+    // All-children playouts with thousands of trees at once (large batches of searches): one workgroup per tree (see
+    // search_body), which does no work twice and keeps every CU busy from the queue; fewer trees: a team of one workgroup
+    // per column, which is much faster per step.  Measured switch-over: about 2000 trees (768 searches of 4 trees:
+    // 19 G playouts/s against 14; 256 searches: 6.4 against 12.7).  MCTSNC_SOLO_TREES moves it (0 = never).
+    int solo_from = 2000;
+    if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
+    const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
+    if (solo) args.G = 1;
+    const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
+    if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(c4::search_kernel_solo), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
     // all its workgroups must be resident together: a batch with more trees than resident sets starts one tree per
     // set and hands the remaining trees out through a queue as sets finish.
@@ -428,13 +437,14 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     if (e0->acp) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
-        const int resident_sets = (int)((int64_t)per_cu * cus / (8 * e0->G)) * 8;
-        if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * e0->G);
+        if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel_solo, e0->block, lds));
+        else HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
+        const int resident_sets = (int)((int64_t)per_cu * cus / (8 * args.G)) * 8;
+        if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * args.G);
         if (sets > resident_sets) { sets = resident_sets; args.queue = e0->d_abort + 1; }
-        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets (%d workgroups per CU resident)%s\n", n_refs, sets, per_cu, args.queue ? ", queue" : "");
+        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets of %d (%d workgroups per CU resident)%s\n", n_refs, sets, args.G, per_cu, args.queue ? ", queue" : "");
     }
-    const dim3 grid(e0->G * sets);
+    const dim3 grid(args.G * sets);
     static std::atomic<uint32_t> launch_counter{0};
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
@@ -445,8 +455,13 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
                 if (args.launch_seq == 0) args.launch_seq = ++launch_counter;   // 0 is what a reset header holds
                 HIP_TRY(hipMemcpyAsync(args.queue, &sets, sizeof(int32_t), hipMemcpyHostToDevice, stream));
             }
-            void *kargs[] = {&args};
-            HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+            if (solo) {   // nothing is exchanged between workgroups: an ordinary launch
+                hipLaunchKernelGGL(c4::search_kernel_solo, grid, block, lds, stream, args);
+                HIP_TRY(hipGetLastError());
+            } else {
+                void *kargs[] = {&args};
+                HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+            }
         } else {
             hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, lds, stream, args);
             HIP_TRY(hipGetLastError());
