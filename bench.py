@@ -303,6 +303,52 @@ def bench_puct_gomoku(args):
     print(json.dumps(out))
 
 
+def bench_c4_many(args):
+    """Many searches of the headline configuration (C4 6x7 acp_prodigal 4x256, 5000 steps each) in one run_batch pass: the
+    64 seeded roots repeated, every search with its own engine and pools (60 MiB each); one bench step = one pass."""
+    import contextlib
+    import io
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    roots = make_roots(N_ROOTS)
+    n = args.searches
+    steps = args.steps if args.steps != N_ROOTS else 3
+    with contextlib.redirect_stdout(io.StringIO()):
+        engines = []
+        for _ in range(n):
+            e = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=T, n_playouts=P,
+                       variant="acp_prodigal", device_memory=0.06, ucb_c=2.0, seed=0, verbose_info=False)
+            e.init_device_side_arrays()
+            engines.append(e)
+        chunk = [roots[i % len(roots)] for i in range(n)]
+        times = []
+        for k in range(max(args.warmup, 1) + steps):
+            for e in engines:
+                e.reseed()
+            t0 = time.perf_counter()
+            run_batch(engines, [c[0] for c in chunk], [c[1] for c in chunk], [c[2] for c in chunk])
+            if k >= max(args.warmup, 1):
+                times.append(time.perf_counter() - t0)
+        playouts = sum(e.performance_info["playouts"] for e in engines)
+        abytes = sum(algorithmic_bytes(e._result, e.steps * T)["total"] for e in engines)
+        dev = engines[0].time_device_loop
+        for e in engines:
+            e._release()
+    dt = sum(times) / len(times)
+    out = {"metric": "playouts/s, many concurrent C4 6x7 ACP-prodigal 4x256 searches in one pass on 1 MI355X", "value": playouts / dt,
+           "unit": "playouts/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1), "ms_per_step": dt * 1e3,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "int64 bitboards + int32 counters (UCB in f64 rounded to f32)", "data": "synthetic",
+           "config": {"workload": f"C4 6x7, {n} searches (the 64 seeded roots repeated) x acp_prodigal n_trees=4 n_playouts=256 "
+                                  "search_steps_limit=5000 device_memory=60MiB each, all in one run_batch pass"},
+           "searches_per_s": n / dt, "trees_in_flight": n * T, "mcts_steps_per_s_all_searches": n * STEPS / dt,
+           "roofline": {"bound": "hbm", "achieved": abytes / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": abytes / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "kernel": "mctsnc::c4::search_kernel_solo from 2000 trees on, mctsnc::c4::search_kernel<true> below",
+                        "algorithmic_bytes_per_launch": abytes, "avg_launch_ms": dev * 1e3},
+           "cpu_baseline": None}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -313,10 +359,11 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by) and exit")
-    ap.add_argument("--workload", default="c4", choices=("c4", "gomoku", "puct_select", "puct_gomoku"),
+    ap.add_argument("--workload", default="c4", choices=("c4", "c4_many", "gomoku", "puct_select", "puct_gomoku"),
                     help="c4: the headline MCTS-NC search (default); puct_select: the reference's deep-wide PUCT selection "
                          "benchmark through puct_select_winner_recalc_launch; puct_gomoku: the Gomoku PUCT search loop")
     ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
+    ap.add_argument("--searches", type=int, default=768, help="c4_many: concurrent searches in the pass")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (trees are independent and would shard over GPUs with one "
@@ -334,6 +381,8 @@ def main():
 
     if args.workload == "gomoku":
         return bench_gomoku(args)
+    if args.workload == "c4_many":
+        return bench_c4_many(args)
     if args.workload == "puct_select":
         return bench_puct_select(args)
     if args.workload == "puct_gomoku":
