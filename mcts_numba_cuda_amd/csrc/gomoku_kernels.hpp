@@ -84,6 +84,7 @@ struct SearchArgs {
     int32_t m, n;
     int32_t P;
     int32_t G;              // workgroups per tree
+    int32_t slots;          // playouts a workgroup runs at a time (<= its threads)
     int32_t span;           // XCDs a tree's workgroups are spread over (1 unless the launch has fewer than 8 trees)
     int32_t S;
     int32_t nsteps;
@@ -242,8 +243,11 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
 
     extern __shared__ unsigned char s_dyn[];
     const int list_dwords = (cells + 3) >> 2;
-    uint32_t *const s_list = reinterpret_cast<uint32_t *>(s_dyn);      // [list_dwords][nthreads]
-    uint32_t *const s_lines = s_list + (size_t)list_dwords * nthreads;  // [n_lines][nthreads]
+    // Playouts a round of the workgroup holds: a workgroup may have more threads than playouts (they speed up the
+    // expansion and the backup), its LDS is sized for the playouts.
+    const int nslots = args.slots;
+    uint32_t *const s_list = reinterpret_cast<uint32_t *>(s_dyn);      // [list_dwords][nslots]
+    uint32_t *const s_lines = s_list + (size_t)list_dwords * nslots;   // [n_lines][nslots]
     const uint32_t div_n = 65536u / (uint32_t)n + 1u;                   // (a * div_n) >> 16 == a / n for a < 1024, n <= 32
 
     __shared__ int32_t s_path[kMaxPath];
@@ -427,8 +431,8 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                 __syncthreads();
                 const int count0 = s_count;
                 const uint64_t *rng_base = ref.rng_playout + 2 * (size_t)(ACP ? paction * P : 0);
-                for (int round = 0; round * nthreads < P; round++) {
-                    const int t = round * nthreads + tid;  // playout index within the block of P
+                for (int round = 0; round * nslots < P; round++) {
+                    const int t = tid < nslots ? round * nslots + tid : P;  // playout index within the block of P
                     int outcome = 0; bool redo = false;
                     uint64_t s0 = 0, s1 = 0, s0_start = 0, s1_start = 0;
                     const uint32_t plies_start = plies;
@@ -438,13 +442,13 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                         {
                             const int used = (count0 + 3) >> 2;
 #pragma unroll 8
-                            for (int k = 0; k < used; k++) s_list[k * nthreads + tid] = s_tmpl[k];
+                            for (int k = 0; k < used; k++) s_list[k * nslots + tid] = s_tmpl[k];
 #pragma unroll 8
-                            for (int k = 0; k < n_lines; k++) s_lines[k * nthreads + tid] = s_ltmpl[k];
+                            for (int k = 0; k < n_lines; k++) s_lines[k * nslots + tid] = s_ltmpl[k];
                         }
                         uint8_t *const lb = reinterpret_cast<uint8_t *>(s_list + tid);   // byte i: lb[(i >> 2) * stride4 + (i & 3)]
                         uint32_t *const lp = s_lines + tid;
-                        const uint32_t nt = (uint32_t)nthreads, stride4 = nt << 2;
+                        const uint32_t nt = (uint32_t)nslots, stride4 = nt << 2;
                         int count = count0, outcome_if_win = pturn, status = count0 == 0 ? 2 : 0;
                         // byte selector that packs the mover's halves of two line words into one dword; flips with the side to move
                         uint32_t sel = pturn == 1 ? 0x05040100u : 0x07060302u;

@@ -79,6 +79,7 @@ struct mctsnc_engine {
     mctsnc_config cfg;
     bool inited = false;
     bool acp = false, thrifty = false;
+    int slots = 0;   // Gomoku: playouts a workgroup runs at a time (its LDS is sized for them); <= block
     int G = 1, block = 64, tpb_e1 = 64;
     c4::Node *d_nodes = nullptr;
     c4::TreeHdr *d_hdrs = nullptr;
@@ -533,14 +534,14 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     HIP_TRY(hipStreamSynchronize(stream));
 
     gomoku::SearchArgs args;
-    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
+    args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G; args.slots = e0->slots;
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
     // fewer than 8 trees (all-child-playouts): every tree is spread over 8 / next_pow2(trees) XCDs
     args.span = (e0->acp && n_refs < 8) ? 8 / next_pow2(n_refs) : 1;
     const dim3 block(e0->block);
-    const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->block);
+    const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots);
     // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
     // whole: more trees than the device holds rows of 8 * G workgroups for are searched by consecutive launches over
     // equal groups of trees, every group for the same number of steps before the budget is looked at again.
@@ -710,7 +711,10 @@ int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
         e->block = c.n_playouts < 64 ? 64 : c.n_playouts;
     } else {
         e->G = e->acp ? (c.max_actions < 32 ? c.max_actions : 32) : 1;  // workgroups per tree; each takes every G-th child
-        e->block = gomoku_block(c);
+        e->slots = gomoku_block(c);
+        // one workgroup per tree (one-child variants): all 256 threads, whatever the playout count -- creating up to 225
+        // children and re-evaluating the path are shared by all of them
+        e->block = e->acp ? e->slots : gomoku::kMaxThreads;
     }
     // tpb table of src/mctsnc.py:360-365 with cuda_tpb_default = 512: fixes which expand generators OCP uses
     const int tpb_board = next_pow2(c.board_m * c.board_n), tpb_extra = next_pow2(c.extra_info_memory), tpb_actions = next_pow2(c.max_actions);
@@ -790,7 +794,7 @@ int mctsnc_init_device(mctsnc_engine *e) {
         }
         HIP_TRY(hipMemcpy(e->g_refs, refs.data(), sizeof(gomoku::TreeRef) * T, hipMemcpyHostToDevice));
         // the playout state of a workgroup can need more LDS than the default limit allows
-        const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->block);
+        const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->slots);
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         if (e->acp) {
