@@ -240,6 +240,31 @@ def test_one_workgroup_per_tree_gives_the_same_trees(variant, monkeypatch):
             np.testing.assert_array_equal(eb.read_array("trees", ti), es.read_array("trees", ti))
 
 
+@pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
+def test_nearly_full_boards(variant):
+    """Roots with one to four empty cells on both games (trees of a handful of nodes, every playout a few plies, draws
+    by a full board), and a Gomoku root that already holds a five, which neither the reference nor the engine looks
+    for (only lines through the last stone placed are tested)."""
+    from helpers import random_gomoku_root
+    from oracle.oracle import Oracle
+    rng = np.random.default_rng(8)
+    params = dict(n_trees=2, n_playouts=32, variant=variant, device_memory=0.1, ucb_c=2.0, seed=3)
+    e = make_engine(params)
+    o = Oracle("c4", (6, 7), 7, 7, 2, 32, variant, ucb_c=2.0, seed=3, device_memory=0.1, threads=4)
+    for plies in (38, 40, 41):
+        board, fills, turn = random_c4_root(rng, plies)
+        compare_with_oracle(e, o, board, fills, turn, steps=30)
+    e = make_engine(params, board_shape=(6, 6), extra=0, actions=36, game="gomoku")
+    o = Oracle("gomoku", (6, 6), 0, 36, 2, 32, variant, ucb_c=2.0, seed=3, device_memory=0.1, threads=4)
+    for stones in (35, 34, 30):
+        board, turn = random_gomoku_root(rng, 6, 6, stones)
+        compare_with_oracle(e, o, board, None, turn, 20)
+    board = np.zeros((6, 6), np.int8)
+    board[2, 0:5] = 1
+    board[3, 0:4] = -1
+    compare_with_oracle(e, o, board, None, -1, 20)
+
+
 def test_run_batch_equals_single_runs():
     """Several engines searched concurrently in one device pass end in exactly the state separate runs leave."""
     from mcts_numba_cuda_amd import run_batch
