@@ -422,9 +422,10 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     const dim3 block(e0->block);
     // All-children playouts with thousands of trees at once (large batches of searches): one workgroup per tree (see
     // search_body), which does no work twice and keeps every CU busy from the queue; fewer trees: a team of one workgroup
-    // per column, which is much faster per step.  Measured switch-over: about 2000 trees (768 searches of 4 trees:
-    // 19 G playouts/s against 14; 256 searches: 6.4 against 12.7).  MCTSNC_SOLO_TREES moves it (0 = never).
-    int solo_from = 2000;
+    // per column, which is much faster per step.  Measured switch-over: about 2300 trees (768 searches of 4 trees:
+    // 19 G playouts/s against 14; 512 searches: 12.8 against 13.7; 256 searches: 6.4 against 12.7).
+    // MCTSNC_SOLO_TREES moves it (0 = never).
+    int solo_from = 2400;
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
     const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
     if (solo) args.G = 1;
