@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <cmath>
@@ -393,18 +394,32 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         if (rc) return rc;
         for (int t = 0; t < T; t++) { bb[2 * ((size_t)i * T + t)] = b2[0]; bb[2 * ((size_t)i * T + t) + 1] = b2[1]; tr[(size_t)i * T + t] = turns[i]; }
     }
-    // the refs / root / digest buffers of a batch are laid out engine after engine
+    // The refs / root / digest buffers of a batch hold the trees of the searches with the fewest stones on the board
+    // first: those have the longest playouts and the largest trees, and a pass with more trees than the device holds
+    // hands trees out in this order, so the long searches are not the ones that start last.
+    std::vector<int> order((size_t)n_refs);
+    for (int r = 0; r < n_refs; r++) order[r] = r;
+    if (n > 1) {
+        std::vector<int> stones((size_t)n);
+        for (int i = 0; i < n; i++) stones[i] = __builtin_popcountll(bb[2 * (size_t)i * T]) + __builtin_popcountll(bb[2 * (size_t)i * T + 1]);
+        std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return stones[a / T] < stones[b / T]; });
+        std::vector<uint64_t> bb2(bb.size());
+        std::vector<int32_t> tr2(tr.size());
+        for (int k = 0; k < n_refs; k++) { bb2[2 * (size_t)k] = bb[2 * (size_t)order[k]]; bb2[2 * (size_t)k + 1] = bb[2 * (size_t)order[k] + 1]; tr2[k] = tr[order[k]]; }
+        bb.swap(bb2); tr.swap(tr2);
+    }
     c4::TreeRef *d_refs = e0->d_refs;
     uint64_t *d_bb = e0->d_root_bb;
     int32_t *d_turns = e0->d_root_turns;
     c4::TreeDigest *d_digest = e0->d_digest;
     TempBuffers tmp;
     if (n > 1) {
-        std::vector<c4::TreeRef> refs((size_t)n_refs);
+        std::vector<c4::TreeRef> refs((size_t)n_refs), sorted((size_t)n_refs);
         for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->d_refs, sizeof(c4::TreeRef) * T, hipMemcpyDeviceToHost));
+        for (int k = 0; k < n_refs; k++) sorted[k] = refs[order[k]];
         int rc;
         if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 2 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) || (rc = tmp.alloc(&d_digest, n_refs))) return rc;
-        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
+        HIP_TRY(hipMemcpy(d_refs, sorted.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
     }
     hipStream_t stream = e0->stream;
     HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
@@ -422,10 +437,10 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     const dim3 block(e0->block);
     // All-children playouts with thousands of trees at once (large batches of searches): one workgroup per tree (see
     // search_body), which does no work twice and keeps every CU busy from the queue; fewer trees: a team of one workgroup
-    // per column, which is much faster per step.  Measured switch-over: about 2300 trees (768 searches of 4 trees:
-    // 19 G playouts/s against 14; 512 searches: 12.8 against 13.7; 256 searches: 6.4 against 12.7).
-    // MCTSNC_SOLO_TREES moves it (0 = never).
-    int solo_from = 2400;
+    // per column, which is much faster per step.  Measured switch-over: about 1300 trees (searches of 4 trees x 256
+    // playouts, G playouts/s: 768 searches 23.2 against 14.6 for teams, 384 searches 16.5 against 14.4, 256 searches
+    // 10.8 against 13.8).  MCTSNC_SOLO_TREES moves it (0 = never).
+    int solo_from = 1400;
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
     const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
     if (solo) args.G = 1;
@@ -479,9 +494,9 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     HIP_TRY(hipMemcpyAsync(dg.data(), d_digest, sizeof(c4::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
     std::vector<TreeSummary> ts((size_t)n_refs);
-    for (int r = 0; r < n_refs; r++) {
-        const c4::TreeDigest &d = dg[r];
-        TreeSummary &t = ts[r];
+    for (int k = 0; k < n_refs; k++) {
+        const c4::TreeDigest &d = dg[k];
+        TreeSummary &t = ts[order[k]];
         t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
         t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
         t.stat_expanded = d.stat_expanded; t.stat_played = d.stat_played;
