@@ -526,6 +526,20 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         if (rc) return rc;
         for (int t = 0; t < T; t++) { memcpy(&bb[16 * ((size_t)i * T + t)], b16, sizeof b16); tr[(size_t)i * T + t] = turns[i]; }
     }
+    // trees of the searches with the fewest stones on the board (the longest playouts) first, as for Connect 4; the
+    // groups of trees that consecutive launches take then hold searches of similar length
+    std::vector<int> order((size_t)n_refs);
+    for (int r = 0; r < n_refs; r++) order[r] = r;
+    if (n > 1) {
+        std::vector<int> stones((size_t)n, 0);
+        for (int i = 0; i < n; i++)
+            for (int w = 0; w < 16; w++) stones[i] += __builtin_popcount(bb[16 * (size_t)i * T + w]);
+        std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return stones[a / T] < stones[b / T]; });
+        std::vector<uint32_t> bb2(bb.size());
+        std::vector<int32_t> tr2(tr.size());
+        for (int k = 0; k < n_refs; k++) { memcpy(&bb2[16 * (size_t)k], &bb[16 * (size_t)order[k]], 16 * sizeof(uint32_t)); tr2[k] = tr[order[k]]; }
+        bb.swap(bb2); tr.swap(tr2);
+    }
     gomoku::TreeRef *d_refs = e0->g_refs;
     uint32_t *d_bb = e0->g_root_bb;
     int32_t *d_turns = e0->d_root_turns;
@@ -534,8 +548,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     int8_t *d_info = e0->g_child_info;
     TempBuffers tmp;
     if (n > 1) {
-        std::vector<gomoku::TreeRef> refs((size_t)n_refs);
-        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->g_refs, sizeof(gomoku::TreeRef) * T, hipMemcpyDeviceToHost));
+        std::vector<gomoku::TreeRef> unsorted((size_t)n_refs), refs((size_t)n_refs);
+        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(unsorted.data() + (size_t)i * T, engines[i]->g_refs, sizeof(gomoku::TreeRef) * T, hipMemcpyDeviceToHost));
+        for (int k = 0; k < n_refs; k++) refs[k] = unsorted[order[k]];
         int rc;
         if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 16 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) ||
             (rc = tmp.alloc(&d_digest, n_refs)) || (rc = tmp.alloc(&d_counts, (size_t)n_refs * A * 2)) || (rc = tmp.alloc(&d_info, (size_t)n_refs * A * 3))) return rc;
@@ -603,8 +618,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     HIP_TRY(hipMemcpyAsync(info.data(), d_info, info.size(), hipMemcpyDeviceToHost, stream));
     HIP_TRY(hipStreamSynchronize(stream));
     std::vector<TreeSummary> ts((size_t)n_refs);
-    for (int r = 0; r < n_refs; r++) {
-        const gomoku::TreeDigest &d = dg[r];
+    for (int k = 0; k < n_refs; k++) {
+        const int r = order[k];   // position k of the launch held tree r of the batch
+        const gomoku::TreeDigest &d = dg[k];
         TreeSummary &t = ts[r];
         t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
         t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
@@ -616,9 +632,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         }
         t.child_ns.resize(A); t.child_wins.resize(A); t.child_exists.resize(A); t.child_terminal.resize(A); t.child_outcome.resize(A);
         for (int a = 0; a < A; a++) {
-            t.child_ns[a] = counts[((size_t)r * A + a) * 2]; t.child_wins[a] = counts[((size_t)r * A + a) * 2 + 1];
-            t.child_exists[a] = (uint8_t)info[((size_t)r * A + a) * 3]; t.child_terminal[a] = (uint8_t)info[((size_t)r * A + a) * 3 + 1];
-            t.child_outcome[a] = info[((size_t)r * A + a) * 3 + 2];
+            t.child_ns[a] = counts[((size_t)k * A + a) * 2]; t.child_wins[a] = counts[((size_t)k * A + a) * 2 + 1];
+            t.child_exists[a] = (uint8_t)info[((size_t)k * A + a) * 3]; t.child_terminal[a] = (uint8_t)info[((size_t)k * A + a) * 3 + 1];
+            t.child_outcome[a] = info[((size_t)k * A + a) * 3 + 2];
         }
     }
     finish_results(engines, n, ts, turns, steps, t_start, t_red, time_loop, dev_time, out);

@@ -89,3 +89,26 @@ def test_gomoku_many_trees(variant, T, steps):
     for stones in (8, 1):
         board, turn = random_gomoku_root(rng, 15, 15, stones)
         compare_with_oracle(e, o, board, None, turn, steps)
+
+
+def test_gomoku_one_child_batch_equals_single_runs():
+    """Five one-child searches of positions with different numbers of stones in one pass (the library orders the trees
+    of a batch by stones on the board) against separate runs, twice, so that the generators carry over on both sides."""
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    rng = np.random.default_rng(29)
+
+    def mk():
+        e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, n_trees=3, n_playouts=64, variant="ocp_prodigal", device_memory=0.5,
+                   seed=6, verbose_info=False, game="gomoku")
+        e.init_device_side_arrays()
+        return e
+    roots = [random_gomoku_root(rng, 15, 15, stones) for stones in (14, 2, 9, 0, 21)]
+    batch, single = [mk() for _ in roots], [mk() for _ in roots]
+    for _ in range(2):
+        run_batch(batch, [r[0] for r in roots], None, [r[1] for r in roots], forced_search_steps_limit=40)
+        for e, r in zip(single, roots):
+            e.run(r[0], None, r[1], forced_search_steps_limit=40)
+        for eb, es in zip(batch, single):
+            assert eb.actions_info == es.actions_info
+            for name in ("trees", "ns", "ns_wins"):
+                np.testing.assert_array_equal(eb.read_array(name, 2), es.read_array(name, 2))
