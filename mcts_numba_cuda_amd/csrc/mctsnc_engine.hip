@@ -569,22 +569,20 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
-    // fewer than 8 trees (all-child-playouts): every tree is spread over 8 / next_pow2(trees) XCDs
-    args.span = (e0->acp && n_refs < 8) ? 8 / next_pow2(n_refs) : 1;
     const dim3 block(e0->block);
     const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots);
     // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
-    // whole: more trees than the device holds rows of 8 * G workgroups for are searched by consecutive launches over
-    // equal groups of trees, every group for the same number of steps before the budget is looked at again.
+    // whole: more trees than the device holds G workgroups each for are searched by consecutive launches over equal
+    // groups of trees, every group for the same number of steps before the budget is looked at again.
     int group = n_refs;
-    if (e0->acp && args.span == 1) {
+    if (e0->acp) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
         HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block, lds));
-        const int64_t rows = (int64_t)per_cu * cus / (8 * e0->G);
-        if (rows < 1) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * e0->G);
-        const int64_t n_groups = ((n_refs + 7) / 8 + rows - 1) / rows;
-        group = (int)(8 * (((n_refs + 7) / 8 + n_groups - 1) / n_groups));
+        const int64_t fit = (int64_t)per_cu * cus / e0->G;   // trees per launch
+        if (fit < 1) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of a tree at once", e0->G);
+        const int64_t n_groups = (n_refs + fit - 1) / fit;
+        group = (int)((n_refs + n_groups - 1) / n_groups);
         if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees, %d workgroups per tree, %d resident workgroups per CU: launches of %d trees\n", n_refs, e0->G, per_cu, group);
     }
     int64_t steps; double dev_time, time_loop;
@@ -593,12 +591,12 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         for (int start = 0; start < n_refs; start += group) {
             args.refs = d_refs + start;
             args.n_refs = std::min(group, n_refs - start);
+            const dim3 grid(e0->G * args.n_refs);
             if (e0->acp) {
-                const dim3 grid(args.span == 1 ? 8 * e0->G * ((args.n_refs + 7) / 8) : 8 * ((e0->G + args.span - 1) / args.span));
                 void *kargs[] = {&args};
                 HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
             } else {
-                hipLaunchKernelGGL(gomoku::search_kernel<false>, dim3(8 * ((args.n_refs + 7) / 8)), block, lds, stream, args);
+                hipLaunchKernelGGL(gomoku::search_kernel<false>, grid, block, lds, stream, args);
                 HIP_TRY(hipGetLastError());
             }
         }
@@ -835,9 +833,7 @@ int mctsnc_init_device(mctsnc_engine *e) {
             HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e->block, lds));
             HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
             const int64_t resident = (int64_t)per_cu * cus;
-            // the grid is 8 * G * ceil(T / 8) workgroups, or next_pow2(T) * G for fewer than 8 trees
-            // (more trees than the device holds workgroups: one workgroup per tree, several launches per step budget)
-            int64_t g_fit = resident / (T < 8 ? next_pow2(T) : 8 * ((T + 7) / 8));
+            const int64_t g_fit = resident / T;
             e->G = (int)std::min<int64_t>(std::max<int64_t>(g_fit, 1), A);
         }
     }
