@@ -13,6 +13,9 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                # UCB values must be bit-reproducible: no fused multiply-add contraction anywhere
                "-ffp-contract=off",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               # the playout loops are a few hundred bytes run by a lone wavefront: where they start relative to the
+               # instruction cache lines moved measured rates by 3 % between otherwise identical builds
+               "-falign-loops=64",
                "-Wno-unknown-warning-option"]
 
 

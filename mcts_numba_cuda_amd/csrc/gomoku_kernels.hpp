@@ -230,7 +230,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
     // to 40 % slower with tree counts that are not multiples of 8.)
     const int b = blockIdx.x;
     const int G = args.G;
-    const int r = b / G, g = b - r * G;
+    const int r = ACP ? b / G : b, g = ACP ? b - r * G : 0;
     if (r >= args.n_refs) return;
     const TreeRef ref = args.refs[r];
     Node *const nodes = ref.nodes;
