@@ -94,7 +94,9 @@ int mctsnc_init_device(mctsnc_engine *e);
 /* MCTSNC.run / _run_<variant> (src/mctsnc.py:409-434, :565-1257).  board: int8[m*n] row-major, values in
  * {-1, 0, +1}; extra: int8[extra_len] or NULL; turn: -1 or +1.  steps_limit / time_limit_s may be INFINITY;
  * forced_steps_limit < INFINITY overrides both (src/mctsnc.py:1112-1116).  Blocking. RNG streams carry over
- * from the previous run on the same engine, as in the reference. */
+ * from the previous run on the same engine, as in the reference.  Whatever the limits, a search ends after
+ * floor((2^31 - 1) / (n_playouts * max_actions)) steps (one-child variants: / n_playouts), before an int32 visit
+ * counter (the reference's dtype, src/mctsnc.py:334-335) could overflow. */
 int mctsnc_run(mctsnc_engine *e, const int8_t *board, const int8_t *extra, int32_t extra_len, int32_t turn,
                double steps_limit, double time_limit_s, double forced_steps_limit, mctsnc_result *out);
 
