@@ -343,7 +343,7 @@ def bench_c4_many(args):
            "searches_per_s": n / dt, "trees_in_flight": n * T, "mcts_steps_per_s_all_searches": n * STEPS / dt,
            "roofline": {"bound": "hbm", "achieved": abytes / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": abytes / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                        "kernel": "mctsnc::c4::search_kernel_solo from 1400 trees on, mctsnc::c4::search_kernel<true> below",
+                        "kernel": "mctsnc::c4::search_kernel_solo (batches of 960 trees or more), mctsnc::c4::search_kernel<true> below",
                         "algorithmic_bytes_per_launch": abytes, "avg_launch_ms": dev * 1e3},
            "cpu_baseline": None}
     print(json.dumps(out))

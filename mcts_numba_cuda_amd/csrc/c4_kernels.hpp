@@ -520,7 +520,10 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 }
             }
             if (timing) { const unsigned long long t2 = wall_clock64(); tk_expand += t2 - tk; tk = t2; }
-            // the playouts of the children, one child after the other, each with its column's generators
+            // The playouts of the children, each with its column's generators.  A workgroup of 2 P threads plays two
+            // children at a time: the children to play are dealt alternately to its two halves (whole wavefronts).
+            const int halves = (int)blockDim.x >= 2 * P && P >= kWave ? 2 : 1;
+            const int half = halves == 2 ? tid / P : 0, pl = halves == 2 ? tid - half * P : tid;   // pl: playout index
             const int rounds = (mode == kModeExpand) ? ncols : (mode == kModeFull ? 1 : 0);
             for (int a = 0; a < rounds; a++) {
                 uint64_t cur, opp; int turn_a;
@@ -532,16 +535,18 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 } else {  // pool exhausted: the selected node itself is played out, with the generators of column 0
                     turn_a = mover; cur = (mover == 1) ? leaf.bb_pos : leaf.bb_neg; opp = (mover == 1) ? leaf.bb_neg : leaf.bb_pos;
                 }
+                const bool my_turn = (__popc(solo_played) & (halves - 1)) == half;
                 solo_played |= 1u << a;
+                if (!my_turn) continue;
                 int outcome = 0;
-                uint64_t *const st = s_rng + 2 * ((size_t)a * P + tid);
+                uint64_t *const st = s_rng + 2 * ((size_t)a * P + pl);
                 uint64_t q0 = 0, q1 = 0;
                 const uint32_t plies_start = plies;
-                if (tid < P) {
+                if (pl < P) {
                     q0 = st[0]; q1 = st[1];
                     outcome = fast_playout(geo, cur, opp, turn_a, q0, q1, plies);
                 }
-                unsigned long long redo = __ballot(tid < P && outcome == 2);
+                unsigned long long redo = __ballot(pl < P && outcome == 2);
                 if (redo) {  // rare: replay the affected playouts one at a time with the exact emulation
                     if (lane == 0) {
                         uint32_t spins = 0;
@@ -563,8 +568,8 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                     if (lane == 0) atomicExch(&s_lock, 0u);
                 }
-                if (tid < P) { st[0] = q0; st[1] = q1; }
-                const unsigned long long bn = __ballot(tid < P && outcome == -1), bp = __ballot(tid < P && outcome == 1);
+                if (pl < P) { st[0] = q0; st[1] = q1; }
+                const unsigned long long bn = __ballot(pl < P && outcome == -1), bp = __ballot(pl < P && outcome == 1);
                 if (lane == 0) { s_red_solo[wave][a][0] = __popcll(bn); s_red_solo[wave][a][1] = __popcll(bp); }
             }
             st_played += __popc(solo_played);
@@ -684,7 +689,11 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
         if (SOLO && wave == 0) {  // the children's results: the wavefronts' counts, or the stored outcome times P
             if (lane < ncols) {
                 int neg = 0, pos = 0;
-                if ((solo_played >> lane) & 1u) { for (int wv = 0; wv < nwaves; wv++) { neg += s_red_solo[wv][lane][0]; pos += s_red_solo[wv][lane][1]; } }
+                if ((solo_played >> lane) & 1u) {  // the counts of the wavefronts of the half that played this child
+                    const int halves = (int)blockDim.x >= 2 * P && P >= kWave ? 2 : 1, per_half = nwaves / halves;
+                    const int first = (__popc(solo_played & ((1u << lane) - 1u)) & (halves - 1)) * per_half;
+                    for (int wv = first; wv < first + per_half; wv++) { neg += s_red_solo[wv][lane][0]; pos += s_red_solo[wv][lane][1]; }
+                }
                 else if (mode == kModeExpand && ((expmask >> lane) & 1u)) { neg = solo_outcome_l == -1 ? P : 0; pos = solo_outcome_l == 1 ? P : 0; }
                 s_gather[lane][0] = neg; s_gather[lane][1] = pos;
             }

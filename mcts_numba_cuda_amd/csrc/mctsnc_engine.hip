@@ -434,16 +434,24 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
-    const dim3 block(e0->block);
-    // All-children playouts with thousands of trees at once (large batches of searches): one workgroup per tree (see
-    // search_body), which does no work twice and keeps every CU busy from the queue; fewer trees: a team of one workgroup
-    // per column, which is much faster per step.  Measured switch-over: about 1300 trees (searches of 4 trees x 256
-    // playouts, G playouts/s: 768 searches 23.2 against 14.6 for teams, 384 searches 16.5 against 14.4, 256 searches
-    // 10.8 against 13.8).  MCTSNC_SOLO_TREES moves it (0 = never).
-    int solo_from = 1400;
+    dim3 block(e0->block);
+    // All-children playouts with many trees at once: one workgroup per tree (see search_body), which does no work twice and
+    // keeps every CU busy from the queue; fewer trees: a team of one workgroup per column, which is much faster per step.
+    // Measured switch-over (4 trees x 256 playouts per search, G playouts/s, one workgroup per tree against teams): a
+    // batch of searches of different roots, where the longest search sets the pace, from about 900 trees on (768
+    // searches 22 against 14.6, 256 searches 14.7 against 13.8, 192 searches 11.4 against 13.0); one search, whose trees
+    // all take about as long, from about 200 trees on (256 trees: 309 ms against 384 for seven roots; 128 trees: 307
+    // against 223).  MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
+    int solo_from = n > 1 ? 960 : 200;
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
     const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
-    if (solo) args.G = 1;
+    if (solo) {
+        args.G = 1;
+        // Twice the threads where that keeps whole wavefronts per child: two children are played at a time, which
+        // shortens a tree's step by a third.  Not for the largest passes, where only throughput counts and the idle half
+        // of a round costs 5 % (768 searches: 420 ms against 440; 512 searches: 338 against 316; 256: 300 against 220).
+        if (c.n_playouts >= 64 && 2 * c.n_playouts <= 512 && n_refs < 2560) block = dim3(2 * c.n_playouts);
+    }
     const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
     if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(c4::search_kernel_solo), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
@@ -454,7 +462,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     if (e0->acp) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel_solo, e0->block, lds));
+        if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel_solo, block.x, lds));
         else HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
         const int resident_sets = (int)((int64_t)per_cu * cus / (8 * args.G)) * 8;
         if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * args.G);
