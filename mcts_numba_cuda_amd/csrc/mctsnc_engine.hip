@@ -450,7 +450,9 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         // Twice the threads where that keeps whole wavefronts per child: two children are played at a time, which
         // shortens a tree's step by a third.  Not for the largest passes, where only throughput counts and the idle half
         // of a round costs 5 % (768 searches: 420 ms against 440; 512 searches: 338 against 316; 256: 300 against 220).
-        if (c.n_playouts >= 64 && 2 * c.n_playouts <= 512 && n_refs < 2560) block = dim3(2 * c.n_playouts);
+        bool two_at_a_time = n_refs < 2560;
+        if (const char *v = getenv("MCTSNC_SOLO_PAIRS")) two_at_a_time = atoi(v) != 0;   // for testing either form on small searches
+        if (c.n_playouts >= 64 && 2 * c.n_playouts <= 512 && two_at_a_time) block = dim3(2 * c.n_playouts);
     }
     const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
     if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(c4::search_kernel_solo), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
