@@ -108,6 +108,15 @@ __device__ __forceinline__ void atomic_store_relaxed(uint32_t *p, uint32_t v) {
 }
 __device__ __forceinline__ void fence_acquire_agent() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent"); }
 __device__ __forceinline__ void fence_release_agent() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent"); }
+
+// Publishing to workgroups on the same XCC without an L2 write-back.  The vector L1 of a CU is write-through and the
+// workgroups of one XCC share its L2, so a store is visible to them once it has been acknowledged: what a publish
+// needs is that every earlier store of the publishing wavefront has completed before the flag store is issued.  A
+// workgroup-scope release fence does NOT provide that (it lowers to no vector-memory wait when the workgroup runs on
+// one CU, and stores to different L2 channels can land in either order), hence the explicit counter wait: vmcnt counts
+// the wavefront's outstanding vector loads AND stores on gfx9.  Every wavefront that stored data a reader will look at
+// must execute it before the flag store (or before the workgroup barrier that precedes the flag store).
+__device__ __forceinline__ void wait_own_stores_at_l2() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 #endif
 
 }  // namespace mctsnc

@@ -764,9 +764,7 @@ int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
     return MCTSNC_OK;
 }
 
-int mctsnc_init_device(mctsnc_engine *e) {
-    if (!e) return fail(MCTSNC_E_INVALID, "null engine");
-    if (e->inited) free_device(e);
+static int init_device_impl(mctsnc_engine *e) {
     const mctsnc_config &c = e->cfg;
     int ndev = 0;
     HIP_TRY(hipGetDeviceCount(&ndev));
@@ -860,6 +858,14 @@ int mctsnc_init_device(mctsnc_engine *e) {
     return MCTSNC_OK;
 }
 
+int mctsnc_init_device(mctsnc_engine *e) {
+    if (!e) return fail(MCTSNC_E_INVALID, "null engine");
+    free_device(e);   // whatever an earlier (possibly failed) initialisation left behind
+    const int rc = init_device_impl(e);
+    if (rc != MCTSNC_OK) free_device(e);   // a failure half-way (e.g. out of memory for the node pool) keeps nothing allocated
+    return rc;
+}
+
 int mctsnc_reseed(mctsnc_engine *e) {
     if (!e || !e->inited) return fail(MCTSNC_E_STATE, "init_device has not been called");
     HIP_TRY(hipSetDevice(e->cfg.device));
@@ -888,7 +894,7 @@ int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on) {
 
 void mctsnc_destroy(mctsnc_engine *e) {
     if (!e) return;
-    if (e->inited) { (void)hipSetDevice(e->cfg.device); free_device(e); }
+    free_device(e);   // every pointer is checked for null, so this also cleans up after a failed initialisation
     delete e;
 }
 

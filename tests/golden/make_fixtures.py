@@ -1,6 +1,7 @@
 """Condenses the reference's recorded artefacts into the small fixtures kept in this folder.
 
 Inputs (data files of the reference, read as data, never executed):
+  * README.md -- two example runs with their full printouts (the only recorded Gomoku search there is).
   * extras/mctsnc_{ocp,acp}_thrifty_c4_1000steps.json  -- complete tree dumps written by the
     reference's MCTSNC._json_dump (src/mctsnc.py:2377-2462) after 1000 steps, T=4, P=128, seed 0.
   * experiments/*.zip -- tournament archives (src/utils.py:168-185): the stdout log holds, for every
@@ -14,6 +15,11 @@ Outputs:
                                       the ordered list of moves and MCTSNC / MCTS searches.
   * north_star_experiment.json.gz     all 100 games of the experiment with acp_prodigal 4x256 against the CPU
                                       player (moves and MCTSNC searches only), in the same format.
+  * readme_examples.json              the two complete MCTSNC runs printed in the reference's README.md ("Example
+                                      usage 1 (Connect 4)" and "Example usage 2 (Gomoku)"): the drawn root position,
+                                      the constructor parameters of the printed instance, the step count, every root
+                                      action row the printout shows (the Gomoku one elides most of its 210 rows), the
+                                      best action and the tree statistics.
 
 Usage: python tests/golden/make_fixtures.py [/root/reference]
 """
@@ -113,6 +119,65 @@ def condense_whole_experiment(ref_root, out):
         f.write(json.dumps({"archive": name, "engines": engines, "games": games}, separators=(",", ":")).encode())
 
 
+def condense_readme(ref_root, out):
+    """The two example runs of README.md.  Boards are drawn with the symbols of C4.SYMBOLS / Gomoku.SYMBOLS
+    (src/c4.py:24, src/gomoku.py:25: index = cell value + 1, so the hollow disc is -1 and the full disc +1); a C4
+    drawing lists row 0 first (src/c4.py:52-69), a Gomoku drawing lists row M-1 first and labels rows from 1
+    (src/gomoku.py:44-64).  Stored as rows of 'X' (+1), 'O' (-1), '.' (empty) in board index order."""
+    text = open(os.path.join(ref_root, "README.md"), encoding="utf-8").read()
+    sym = {"\u25CF": "X", "\u25CB": "O", ".": ".", "+": "."}
+    examples = {}
+    for name, title in (("c4", "## Example usage 1 (Connect 4)"), ("gomoku", "## Example usage 2 (Gomoku)")):
+        part = text[text.index(title):]
+        part = part[:part.index("\n## ", 5)]
+        blocks = re.findall(r"```bash\n(.*?)```", part, flags=re.S)
+        drawing, printout = blocks[0], blocks[1]
+        rows = []
+        if name == "c4":
+            for line in drawing.splitlines():
+                if line.startswith("|"):
+                    rows.append("".join(sym[ch] for ch in line.strip().strip("|").split("|")))
+        else:
+            labelled = {}
+            for line in drawing.splitlines():
+                mt = re.match(r"\s*(\d+)(\S+?)(\d+)\s*$", line)
+                if mt and mt.group(1) == mt.group(3):
+                    labelled[int(mt.group(1))] = "".join(sym[ch] for ch in mt.group(2))
+            rows = [labelled[i + 1] for i in range(len(labelled))]
+        n_pos = sum(r.count("X") for r in rows)
+        n_neg = sum(r.count("O") for r in rows)
+        turn = 1 if n_pos == n_neg else -1   # +1 moves first (src/mcts.py State.__init__: turn = 1)
+        assert n_pos - n_neg in (0, 1)
+        inst = re.search(r"MCTSNC RUN\.\.\. \[MCTSNC\((.*?)\)\]", printout).group(1)
+        params = parse_instance_fields(inst)
+        actions = {}
+        for mt in re.finditer(r"^\s+(\d+): (\{.*?\}),?$", printout, flags=re.M):
+            row = ast.literal_eval(mt.group(2))
+            actions[int(mt.group(1))] = {k: row[k] for k in ("name", "n_root", "win_flag", "n", "n_wins", "q", "ucb")}
+        best = ast.literal_eval(re.search(r"^\s+best: (\{.*?\})$", printout, flags=re.M).group(1))
+        trees = ast.literal_eval(re.search(r"^\s+trees: (\{.*?\})$", printout, flags=re.M).group(1))
+        examples[name] = {
+            "source": "README.md, " + title[3:],
+            "board_rows": rows, "turn": turn, "params": params,
+            "per_state_memory": int(re.search(r"per_state_memory: (\d+) B", printout).group(1)),
+            "max_tree_size": int(re.search(r"calculated max_tree_size: (\d+)", printout).group(1)),
+            "steps": int(re.search(r"^\s+steps: (\d+),", printout, flags=re.M).group(1)),
+            "playouts": int(re.search(r"^\s+playouts: (\d+),", printout, flags=re.M).group(1)),
+            "rows_elided": re.search(r"^\s+\.\.\.$", printout, flags=re.M) is not None,
+            "actions": actions, "best": best, "trees": trees,
+        }
+    json.dump(examples, open(out, "w"), indent=1)
+
+
+def parse_instance_fields(inst):
+    """'search_time_limit=5.0, ..., variant='acp_prodigal', ..., seed: 0' (MCTSNC.__str__, src/mctsnc.py:305) -> dict."""
+    out = {}
+    for item in inst.split(", "):
+        key, value = re.split(r"=|: ", item, maxsplit=1)
+        out[key] = value.strip("'") if value.startswith("'") else ("inf" if value == "inf" else float(value) if "." in value else int(value))
+    return out
+
+
 if __name__ == "__main__":
     ref = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
     for variant in ("ocp_thrifty", "acp_thrifty"):
@@ -120,4 +185,5 @@ if __name__ == "__main__":
                       os.path.join(HERE, f"dump_{variant}_c4_1000steps.npz"))
     condense_archives(ref, os.path.join(HERE, "archive_games.json"))
     condense_whole_experiment(ref, os.path.join(HERE, "north_star_experiment.json.gz"))
+    condense_readme(ref, os.path.join(HERE, "readme_examples.json"))
     print("fixtures written to", HERE)
