@@ -136,6 +136,23 @@ int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, c
                      const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
                      mctsnc_result *out);
 
+/* mctsnc_run_batch for callers that cannot allocate device memory while they run (tight serving loops, harnesses
+ * that forbid hipMalloc; it has no counterpart in the reference).  Same arguments, same results, n >= 1.  The per-call
+ * device buffers -- the gathered per-tree pointer records, the root positions and turns, the per-tree digests the
+ * final reductions read -- come out of a static device array of MCTSNC_NOALLOC_SCRATCH_BYTES that the library holds
+ * on every device it runs on until the process ends, instead of a hipMalloc / hipFree pair per call; the call makes
+ * no hipMalloc, hipFree or other allocating device-runtime call (the engines' own pools were allocated by
+ * mctsnc_init_device, which also looks up the array's address on the engine's device).  A batch whose buffers do not
+ * fit is rejected with MCTSNC_E_INVALID and a message that states both sizes (Connect 4: about 290 bytes per tree, i.e.
+ * some 14 000 trees; Gomoku: about 250 + 11 * max_actions bytes per tree, i.e. some 1500 trees of a 15x15 board).  All calls on one
+ * device share the one array: a call that finds it in use by another host thread returns MCTSNC_E_STATE rather
+ * than overwrite that call's buffers.  Every byte a call reads it has written first, so nothing needs clearing
+ * between calls. */
+#define MCTSNC_NOALLOC_SCRATCH_BYTES (4u << 20)
+int mctsnc_run_batch_noalloc(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
+                             const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
+                             mctsnc_result *out);
+
 /* Switches the per-stage device timers on (default) or off. */
 int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on);
 

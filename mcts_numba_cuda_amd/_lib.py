@@ -71,6 +71,8 @@ def lib():
         L.mctsnc_run_batch.restype = ctypes.c_int
         L.mctsnc_run_batch.argtypes = [ctypes.POINTER(vp), ctypes.c_int32, vp, vp, ctypes.c_int32, vp, ctypes.c_double,
                                        ctypes.c_double, ctypes.c_double, ctypes.POINTER(Result)]
+        L.mctsnc_run_batch_noalloc.restype = ctypes.c_int
+        L.mctsnc_run_batch_noalloc.argtypes = L.mctsnc_run_batch.argtypes
         L.mctsnc_read_size.restype = ctypes.c_int64
         L.mctsnc_read_size.argtypes = [vp, ctypes.c_int32, ctypes.c_int32]
         L.mctsnc_read.restype = ctypes.c_int

@@ -12,6 +12,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -95,6 +96,8 @@ struct mctsnc_engine {
     bool has_run = false;
     bool stage_timing = true;
     std::vector<uint64_t> rng_init_playout, rng_init_expand;  // the streams as seeded, kept for reseed()
+    std::vector<c4::TreeRef> h_refs;          // host copies of the per-tree pointer records (a batch gathers them)
+    std::vector<gomoku::TreeRef> hg_refs;
     // Gomoku pools
     gomoku::Node *g_nodes = nullptr;
     gomoku::Stat *g_stats = nullptr;
@@ -365,22 +368,82 @@ void finish_results(mctsnc_engine **engines, int n, const std::vector<TreeSummar
     }
 }
 
-// RAII holder for the temporary device buffers of a batched run
-struct TempBuffers {
-    std::vector<void *> ptrs;
-    ~TempBuffers() { for (void *p : ptrs) (void)hipFree(p); }
-    template <typename T> int alloc(T **out, size_t count) {
-        void *p = nullptr;
-        hipError_t err = hipMalloc(&p, sizeof(T) * count);
-        if (err != hipSuccess) return fail(MCTSNC_E_HIP, "hipMalloc of a batch buffer failed: %s", hipGetErrorString(err));
-        ptrs.push_back(p);
-        *out = static_cast<T *>(p);
+// The per-call device buffers of a batched run (the gathered per-tree pointer records, the roots, the per-tree digests)
+// are pieces of one block of device memory: a temporary allocation (mctsnc_run_batch) or the static scratch below
+// (mctsnc_run_batch_noalloc).  With a null base only the size is counted.
+struct Workspace {
+    unsigned char *base = nullptr;
+    size_t size = 0, used = 0;
+    template <typename T> T *take(size_t count) {
+        T *p = base ? reinterpret_cast<T *>(base + used) : nullptr;
+        used += (sizeof(T) * count + 255) & ~(size_t)255;
+        return p;
+    }
+};
+
+struct C4BatchBuffers { c4::TreeRef *refs; uint64_t *root_bb; int32_t *turns; c4::TreeDigest *digest; };
+C4BatchBuffers carve_c4(Workspace &w, size_t n_refs) {
+    C4BatchBuffers b;
+    b.refs = w.take<c4::TreeRef>(n_refs); b.root_bb = w.take<uint64_t>(2 * n_refs); b.turns = w.take<int32_t>(n_refs);
+    b.digest = w.take<c4::TreeDigest>(n_refs);
+    return b;
+}
+
+struct GomokuBatchBuffers { gomoku::TreeRef *refs; uint32_t *root_bb; int32_t *turns; gomoku::TreeDigest *digest; int32_t *counts; int8_t *info; };
+GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t A) {
+    GomokuBatchBuffers b;
+    b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(16 * n_refs); b.turns = w.take<int32_t>(n_refs);
+    b.digest = w.take<gomoku::TreeDigest>(n_refs); b.counts = w.take<int32_t>(n_refs * A * 2); b.info = w.take<int8_t>(n_refs * A * 3);
+    return b;
+}
+
+// A temporary block for one call (released when the call returns), or the caller's block.
+struct BlockHolder {
+    void *owned = nullptr;
+    ~BlockHolder() { if (owned) (void)hipFree(owned); }
+    int get(Workspace *fixed, size_t need, Workspace &out) {
+        if (fixed) {
+            if (need > fixed->size)
+                return fail(MCTSNC_E_INVALID, "this batch needs %zu bytes of device scratch; the static buffer of the entry point that allocates nothing holds %zu (MCTSNC_NOALLOC_SCRATCH_BYTES)", need, fixed->size);
+            out = *fixed; out.used = 0;
+            return MCTSNC_OK;
+        }
+        hipError_t err = hipMalloc(&owned, need);
+        if (err != hipSuccess) { owned = nullptr; return fail(MCTSNC_E_HIP, "hipMalloc of the batch buffers (%zu bytes) failed: %s", need, hipGetErrorString(err)); }
+        out.base = static_cast<unsigned char *>(owned); out.size = need; out.used = 0;
         return MCTSNC_OK;
     }
 };
 
+// ---- scratch of mctsnc_run_batch_noalloc -----------------------------------------------------------------------------
+// Device memory that exists from the moment the library is loaded: every device the library runs on holds its own copy
+// of this array, at its own address, until the process ends.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress; the address a kernel or a copy can use is what that call returns for the current device.
+static __device__ __align__(256) unsigned char scratch[MCTSNC_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+struct DeviceScratch {
+    std::atomic<unsigned char *> ptr{nullptr};
+    std::atomic<bool> busy{false};
+};
+DeviceScratch g_scratch[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+// Looks the array's address up once per device.  The device must be current.
+int scratch_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) return fail(MCTSNC_E_INVALID, "device %d is beyond the %d devices the static scratch is tracked for", device, kMaxDevices);
+    if (g_scratch[device].ptr.load(std::memory_order_acquire)) return MCTSNC_OK;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch[device].ptr.load(std::memory_order_acquire)) return MCTSNC_OK;
+    void *p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(MCTSNC_E_HIP, "hipGetSymbolAddress returned a null address for the static scratch on device %d", device);
+    g_scratch[device].ptr.store(static_cast<unsigned char *>(p), std::memory_order_release);
+    return MCTSNC_OK;
+}
+
 int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
-                const Budget &bud, mctsnc_result *out) {
+                const Budget &bud, mctsnc_result *out, Workspace *fixed) {
     mctsnc_engine *e0 = engines[0];
     const mctsnc_config &c = e0->cfg;
     const int T = c.n_trees, mn = c.board_m * c.board_n, A = c.max_actions;
@@ -408,19 +471,23 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         for (int k = 0; k < n_refs; k++) { bb2[2 * (size_t)k] = bb[2 * (size_t)order[k]]; bb2[2 * (size_t)k + 1] = bb[2 * (size_t)order[k] + 1]; tr2[k] = tr[order[k]]; }
         bb.swap(bb2); tr.swap(tr2);
     }
-    c4::TreeRef *d_refs = e0->d_refs;
-    uint64_t *d_bb = e0->d_root_bb;
-    int32_t *d_turns = e0->d_root_turns;
-    c4::TreeDigest *d_digest = e0->d_digest;
-    TempBuffers tmp;
-    if (n > 1) {
-        std::vector<c4::TreeRef> refs((size_t)n_refs), sorted((size_t)n_refs);
-        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(refs.data() + (size_t)i * T, engines[i]->d_refs, sizeof(c4::TreeRef) * T, hipMemcpyDeviceToHost));
-        for (int k = 0; k < n_refs; k++) sorted[k] = refs[order[k]];
-        int rc;
-        if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 2 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) || (rc = tmp.alloc(&d_digest, n_refs))) return rc;
-        HIP_TRY(hipMemcpy(d_refs, sorted.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
+    // one search with allocation allowed: the engine's own buffers; otherwise pieces of one block
+    C4BatchBuffers buf{e0->d_refs, e0->d_root_bb, e0->d_root_turns, e0->d_digest};
+    BlockHolder block_holder;
+    if (n > 1 || fixed) {
+        Workspace count, ws;
+        carve_c4(count, (size_t)n_refs);
+        int rc = block_holder.get(fixed, count.used, ws);
+        if (rc) return rc;
+        buf = carve_c4(ws, (size_t)n_refs);
+        std::vector<c4::TreeRef> sorted((size_t)n_refs);
+        for (int k = 0; k < n_refs; k++) sorted[k] = engines[order[k] / T]->h_refs[order[k] % T];
+        HIP_TRY(hipMemcpy(buf.refs, sorted.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
     }
+    c4::TreeRef *const d_refs = buf.refs;
+    uint64_t *const d_bb = buf.root_bb;
+    int32_t *const d_turns = buf.turns;
+    c4::TreeDigest *const d_digest = buf.digest;
     hipStream_t stream = e0->stream;
     HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
@@ -522,7 +589,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     return MCTSNC_OK;
 }
 
-int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const int32_t *turns, const Budget &bud, mctsnc_result *out) {
+int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const int32_t *turns, const Budget &bud, mctsnc_result *out, Workspace *fixed) {
     mctsnc_engine *e0 = engines[0];
     const mctsnc_config &c = e0->cfg;
     const int T = c.n_trees, cells = c.board_m * c.board_n, A = c.max_actions;
@@ -550,22 +617,24 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         for (int k = 0; k < n_refs; k++) { memcpy(&bb2[16 * (size_t)k], &bb[16 * (size_t)order[k]], 16 * sizeof(uint32_t)); tr2[k] = tr[order[k]]; }
         bb.swap(bb2); tr.swap(tr2);
     }
-    gomoku::TreeRef *d_refs = e0->g_refs;
-    uint32_t *d_bb = e0->g_root_bb;
-    int32_t *d_turns = e0->d_root_turns;
-    gomoku::TreeDigest *d_digest = e0->g_digest;
-    int32_t *d_counts = e0->g_child_counts;
-    int8_t *d_info = e0->g_child_info;
-    TempBuffers tmp;
-    if (n > 1) {
-        std::vector<gomoku::TreeRef> unsorted((size_t)n_refs), refs((size_t)n_refs);
-        for (int i = 0; i < n; i++) HIP_TRY(hipMemcpy(unsorted.data() + (size_t)i * T, engines[i]->g_refs, sizeof(gomoku::TreeRef) * T, hipMemcpyDeviceToHost));
-        for (int k = 0; k < n_refs; k++) refs[k] = unsorted[order[k]];
-        int rc;
-        if ((rc = tmp.alloc(&d_refs, n_refs)) || (rc = tmp.alloc(&d_bb, 16 * (size_t)n_refs)) || (rc = tmp.alloc(&d_turns, n_refs)) ||
-            (rc = tmp.alloc(&d_digest, n_refs)) || (rc = tmp.alloc(&d_counts, (size_t)n_refs * A * 2)) || (rc = tmp.alloc(&d_info, (size_t)n_refs * A * 3))) return rc;
-        HIP_TRY(hipMemcpy(d_refs, refs.data(), sizeof(gomoku::TreeRef) * n_refs, hipMemcpyHostToDevice));
+    GomokuBatchBuffers buf{e0->g_refs, e0->g_root_bb, e0->d_root_turns, e0->g_digest, e0->g_child_counts, e0->g_child_info};
+    BlockHolder block_holder;
+    if (n > 1 || fixed) {
+        Workspace count, ws;
+        carve_gomoku(count, (size_t)n_refs, (size_t)A);
+        int rc = block_holder.get(fixed, count.used, ws);
+        if (rc) return rc;
+        buf = carve_gomoku(ws, (size_t)n_refs, (size_t)A);
+        std::vector<gomoku::TreeRef> sorted((size_t)n_refs);
+        for (int k = 0; k < n_refs; k++) sorted[k] = engines[order[k] / T]->hg_refs[order[k] % T];
+        HIP_TRY(hipMemcpy(buf.refs, sorted.data(), sizeof(gomoku::TreeRef) * n_refs, hipMemcpyHostToDevice));
     }
+    gomoku::TreeRef *const d_refs = buf.refs;
+    uint32_t *const d_bb = buf.root_bb;
+    int32_t *const d_turns = buf.turns;
+    gomoku::TreeDigest *const d_digest = buf.digest;
+    int32_t *const d_counts = buf.counts;
+    int8_t *const d_info = buf.info;
     hipStream_t stream = e0->stream;
     HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint32_t) * 16 * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
@@ -649,15 +718,29 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     return MCTSNC_OK;
 }
 
+// use_static: take the per-call device buffers from the static scratch instead of allocating them.
 int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t *extras, int32_t extra_len, const int32_t *turns,
-             const Budget &bud, mctsnc_result *out) {
+             const Budget &bud, mctsnc_result *out, bool use_static) {
     int rc = check_batch(engines, n, turns);
     if (rc) return rc;
     mctsnc_engine *e0 = engines[0];
     const mctsnc_config &c = e0->cfg;
     HIP_TRY(hipSetDevice(c.device));
-    if (e0->is_gomoku()) return run_many_gomoku(engines, n, boards, turns, bud, out);
-    return run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out);
+    if (!use_static)
+        return e0->is_gomoku() ? run_many_gomoku(engines, n, boards, turns, bud, out, nullptr)
+                               : run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out, nullptr);
+    if ((rc = scratch_setup(c.device))) return rc;   // normally done by mctsnc_init_device already
+    DeviceScratch &ds = g_scratch[c.device];
+    // one array per device for all callers: a second call on the same device while one is running would overwrite its
+    // buffers, so it is turned away instead
+    if (ds.busy.exchange(true, std::memory_order_acquire))
+        return fail(MCTSNC_E_STATE, "the static scratch of device %d is in use by another mctsnc_run_batch_noalloc call", c.device);
+    Workspace ws;
+    ws.base = ds.ptr.load(std::memory_order_acquire); ws.size = MCTSNC_NOALLOC_SCRATCH_BYTES;
+    rc = e0->is_gomoku() ? run_many_gomoku(engines, n, boards, turns, bud, out, &ws)
+                         : run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out, &ws);
+    ds.busy.store(false, std::memory_order_release);
+    return rc;
 }
 
 int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t need) {
@@ -800,6 +883,7 @@ static int init_device_impl(mctsnc_engine *e) {
             refs[t].rng_expand = e->acp ? nullptr : e->d_rng_expand + 2 * (size_t)t;
         }
         HIP_TRY(hipMemcpy(e->d_refs, refs.data(), sizeof(c4::TreeRef) * T, hipMemcpyHostToDevice));
+        e->h_refs = refs;
     } else {
         const int A = c.max_actions;
         HIP_TRY(hipMalloc(&e->g_nodes, sizeof(gomoku::Node) * S * T));
@@ -831,6 +915,7 @@ static int init_device_impl(mctsnc_engine *e) {
             refs[t].path = e->g_path + (size_t)t * gomoku::kMaxPath;
         }
         HIP_TRY(hipMemcpy(e->g_refs, refs.data(), sizeof(gomoku::TreeRef) * T, hipMemcpyHostToDevice));
+        e->hg_refs = refs;
         // the playout state of a workgroup can need more LDS than the default limit allows
         const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->slots);
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -847,6 +932,7 @@ static int init_device_impl(mctsnc_engine *e) {
     }
     int rc = upload_rng(e);
     if (rc) return rc;
+    if ((rc = scratch_setup(c.device))) return rc;   // address of the static scratch on this device, looked up once
     if (e->acp) {
         // the step barrier between the workgroups of a tree needs all of them resident at once
         int coop = 0;
@@ -876,14 +962,21 @@ int mctsnc_run(mctsnc_engine *e, const int8_t *board, const int8_t *extra, int32
                double time_limit_s, double forced_steps_limit, mctsnc_result *out) {
     if (!e || !board || !out) return fail(MCTSNC_E_INVALID, "null argument");
     Budget b{steps_limit, time_limit_s, forced_steps_limit};
-    return run_many(&e, 1, board, extra, extra_len, &turn, b, out);
+    return run_many(&e, 1, board, extra, extra_len, &turn, b, out, false);
 }
 
 int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
                      const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit, mctsnc_result *out) {
     if (!engines || !boards || !turns || !out) return fail(MCTSNC_E_INVALID, "null argument");
     Budget b{steps_limit, time_limit_s, forced_steps_limit};
-    return run_many(engines, n, boards, extras, extra_len, turns, b, out);
+    return run_many(engines, n, boards, extras, extra_len, turns, b, out, false);
+}
+
+int mctsnc_run_batch_noalloc(mctsnc_engine **engines, int32_t n, const int8_t *boards, const int8_t *extras, int32_t extra_len,
+                             const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit, mctsnc_result *out) {
+    if (!engines || !boards || !turns || !out) return fail(MCTSNC_E_INVALID, "null argument");
+    Budget b{steps_limit, time_limit_s, forced_steps_limit};
+    return run_many(engines, n, boards, extras, extra_len, turns, b, out, true);
 }
 
 int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on) {

@@ -401,10 +401,12 @@ class MCTSNC:
             print(f"JSON DUMP DONE. [time: {t2 - t1} s]")
 
 
-def run_batch(engines, root_boards, root_extra_infos, root_turns, forced_search_steps_limit=np.inf):
+def run_batch(engines, root_boards, root_extra_infos, root_turns, forced_search_steps_limit=np.inf, allocate=True):
     """Runs one search on each of several identically configured, initialised ``MCTSNC`` instances concurrently in
     one device pass (no counterpart in the reference).  Every instance ends in the state a separate ``run`` call
-    would have left it in.  Returns the list of best actions."""
+    would have left it in.  Returns the list of best actions.  ``allocate=False`` goes through the entry point that
+    takes its per-call device buffers from the library's static scratch instead of allocating them (for callers that
+    must not allocate device memory while running; batches beyond the scratch size are rejected)."""
     n = len(engines)
     e0 = engines[0]
     for e in engines:
@@ -417,9 +419,9 @@ def run_batch(engines, root_boards, root_extra_infos, root_turns, forced_search_
     turns = np.ascontiguousarray(np.asarray(root_turns, dtype=np.int32))
     handles = (ctypes.c_void_p * n)(*[e._engine for e in engines])
     results = (_lib.Result * n)()
-    _lib.check(_lib.lib().mctsnc_run_batch(handles, n, boards.ctypes.data, extras.ctypes.data, extras.shape[1], turns.ctypes.data,
-                                           float(e0.search_steps_limit), float(e0.search_time_limit), float(forced_search_steps_limit),
-                                           results))
+    entry = _lib.lib().mctsnc_run_batch if allocate else _lib.lib().mctsnc_run_batch_noalloc
+    _lib.check(entry(handles, n, boards.ctypes.data, extras.ctypes.data, extras.shape[1], turns.ctypes.data,
+                     float(e0.search_steps_limit), float(e0.search_time_limit), float(forced_search_steps_limit), results))
     for e, r, t in zip(engines, results, turns):
         e._absorb_result(r, int(t))
     return [e.best_action for e in engines]
