@@ -138,13 +138,14 @@ int mctsnc_run_batch(mctsnc_engine **engines, int32_t n, const int8_t *boards, c
 
 /* mctsnc_run_batch for callers that cannot allocate device memory while they run (tight serving loops, harnesses
  * that forbid hipMalloc; it has no counterpart in the reference).  Same arguments, same results, n >= 1.  The per-call
- * device buffers -- the gathered per-tree pointer records, the root positions and turns, the per-tree digests the
- * final reductions read -- come out of a static device array of MCTSNC_NOALLOC_SCRATCH_BYTES that the library holds
+ * device buffers -- the gathered per-tree pointer records, the root positions and turns, the result blocks the
+ * final reductions write -- come out of a static device array of MCTSNC_NOALLOC_SCRATCH_BYTES that the library holds
  * on every device it runs on until the process ends, instead of a hipMalloc / hipFree pair per call; the call makes
  * no hipMalloc, hipFree or other allocating device-runtime call (the engines' own pools were allocated by
  * mctsnc_init_device, which also looks up the array's address on the engine's device).  A batch whose buffers do not
- * fit is rejected with MCTSNC_E_INVALID and a message that states both sizes (Connect 4: about 290 bytes per tree, i.e.
- * some 14 000 trees; Gomoku: about 250 + 11 * max_actions bytes per tree, i.e. some 1500 trees of a 15x15 board).  All calls on one
+ * fit is rejected with MCTSNC_E_INVALID and a message that states both sizes (Connect 4: 52 bytes per tree + 512 per
+ * search, i.e. some 5000 searches of 4 trees; Gomoku 15x15: 140 bytes per tree + 6400 per search, i.e. some 500
+ * searches of 8 trees).  All calls on one
  * device share the one array: a call that finds it in use by another host thread returns MCTSNC_E_STATE rather
  * than overwrite that call's buffers.  Every byte a call reads it has written first, so nothing needs clearing
  * between calls. */

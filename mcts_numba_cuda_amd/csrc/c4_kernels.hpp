@@ -950,41 +950,26 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) search_kernel_solo(SearchArgs args) { search_trees<true, true>(args); }
 
 
-// Per-tree digest for the final reductions (_reduce_over_trees_*, src/mctsnc.py:2222-2296).
-struct TreeDigest {
-    int32_t size, root_ns, max_depth, error;
-    int64_t depth_sum;
-    unsigned long long plies, u1_events, stat_levels, stat_children, stat_expanded, stat_played;
-    unsigned long long t_select, t_expand, t_playout, t_backup, t_exchange;
-    int32_t child_mask;
-    int32_t child_ns[kMaxCols], child_wins[kMaxCols];
-    int8_t child_terminal[kMaxCols], child_outcome[kMaxCols];
-    int16_t root_ae[16];
-};
-
-__global__ void digest_kernel(const TreeRef *refs, int n_refs, TreeDigest *out) {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= n_refs) return;
-    const TreeRef ref = refs[r];
-    const TreeHdr *h = ref.hdr;
-    const Node *root = ref.nodes;
-    TreeDigest d;
-    d.size = h->size; d.root_ns = h->root_ns; d.max_depth = h->max_depth; d.error = h->error; d.depth_sum = h->depth_sum;
-    d.plies = h->plies; d.u1_events = h->u1_events;
-    d.stat_levels = h->stat_levels; d.stat_children = h->stat_children; d.stat_expanded = h->stat_expanded; d.stat_played = h->stat_played;
-    d.t_select = h->t_select; d.t_expand = h->t_expand; d.t_playout = h->t_playout; d.t_backup = h->t_backup; d.t_exchange = h->t_exchange;
-    d.child_mask = (root->flags & kLeaf) ? 0 : root->child_mask;
-    for (int a = 0; a < kMaxCols; a++) {
-        d.child_ns[a] = 0; d.child_wins[a] = 0; d.child_terminal[a] = 0; d.child_outcome[a] = 2;
-        if ((d.child_mask >> a) & 1) {
-            const Node *c = ref.nodes + root->child_base + __popc(d.child_mask & ((1 << a) - 1));
-            d.child_ns[a] = root->child_ns[a]; d.child_wins[a] = root->child_wins[a];
-            d.child_terminal[a] = (c->flags & kTerminal) ? 1 : 0; d.child_outcome[a] = c->outcome;
-        }
+// Where the final reductions (reduce_kernels.hpp) find the root's visit count, the row memorised at the first step and
+// the counters of the root's children in this layout: a child's counters sit in the root's own record, slot = action.
+struct RootView {
+    using Ref = TreeRef;
+    static __device__ __forceinline__ int32_t root_ns(const Ref &r) { return r.hdr->root_ns; }
+    static __device__ __forceinline__ int16_t root_ae(const Ref &r, int i) { return r.hdr->root_ae[i]; }
+    static __device__ __forceinline__ void root_info(const Ref &r, int32_t &base, int32_t &kids) {
+        const Node *root = r.nodes;
+        base = root->child_base; kids = (root->flags & kLeaf) ? 0 : (int32_t)root->child_mask;   // kids: set of expanded actions
     }
-    for (int i = 0; i < 16; i++) d.root_ae[i] = h->root_ae[i];
-    out[r] = d;
-}
+    static __device__ __forceinline__ int action_slot(const Ref &, int a) { return a; }
+    static __device__ __forceinline__ bool has_child(int32_t kids, int, int a) { return (kids >> a) & 1; }
+    static __device__ __forceinline__ void child_counts(const Ref &r, int32_t, int, int a, int32_t &ns, int32_t &wins) {
+        ns = r.nodes->child_ns[a]; wins = r.nodes->child_wins[a];
+    }
+    static __device__ __forceinline__ void child_state(const Ref &r, int32_t base, int32_t kids, int, int a, bool &terminal, int &outcome) {
+        const Node *c = r.nodes + base + __popc((uint32_t)kids & ((1u << a) - 1u));
+        terminal = (c->flags & kTerminal) != 0; outcome = c->outcome;
+    }
+};
 
 }  // namespace c4
 }  // namespace mctsnc

@@ -736,47 +736,34 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
     }
 }
 
-// Per-tree digest for the final reductions (_reduce_over_trees_*, src/mctsnc.py:2222-2296): the header values and,
-// for every action of the root, whether a child exists, its counters and its terminal state.
-struct TreeDigest {
-    int32_t size, root_ns, max_depth, error;
-    int64_t depth_sum;
-    unsigned long long plies, u1_events, stat_levels, stat_children, stat_expanded, stat_played;
-    unsigned long long t_select, t_expand, t_playout, t_backup, t_exchange;
+// Where the final reductions (reduce_kernels.hpp) find the root's visit count, the row memorised at the first step and
+// the counters of the root's children in this layout: the children of the root are its empty cells in row-major order,
+// so the slot of an action is its rank among them; kids = number of children the root has (0 while it is a leaf).
+struct RootView {
+    using Ref = TreeRef;
+    static __device__ __forceinline__ int32_t root_ns(const Ref &r) { return r.stats[0].ns; }
+    static __device__ __forceinline__ int16_t root_ae(const Ref &r, int i) { return r.root_ae[i]; }
+    static __device__ __forceinline__ void root_info(const Ref &r, int32_t &base, int32_t &kids) {
+        const Node *root = r.nodes;
+        base = root->child_base; kids = (root->flags & kLeaf) ? 0 : root->n_children;
+    }
+    static __device__ __forceinline__ int action_slot(const Ref &r, int a) {
+        const Node *root = r.nodes;
+        if (bb_test(root->bb_pos, a) || bb_test(root->bb_neg, a)) return -1;
+        int rank = __popc(~(root->bb_pos[a >> 5] | root->bb_neg[a >> 5]) & ((1u << (a & 31)) - 1u));
+        for (int w = 0; w < (a >> 5); w++) rank += 32 - __popc(root->bb_pos[w] | root->bb_neg[w]);
+        return rank;
+    }
+    static __device__ __forceinline__ bool has_child(int32_t kids, int slot, int) { return slot >= 0 && slot < kids; }
+    static __device__ __forceinline__ void child_counts(const Ref &r, int32_t base, int slot, int, int32_t &ns, int32_t &wins) {
+        const Stat st = r.stats[base + slot];
+        ns = st.ns; wins = st.wins;
+    }
+    static __device__ __forceinline__ void child_state(const Ref &r, int32_t base, int32_t, int slot, int, bool &terminal, int &outcome) {
+        const Node *c = r.nodes + base + slot;
+        terminal = (c->flags & kTerminal) != 0; outcome = c->outcome;
+    }
 };
-
-__global__ void digest_kernel(const TreeRef *refs, int n_refs, int cells, TreeDigest *out, int32_t *child_counts /* [n_refs][A][2] */,
-                              int8_t *child_info /* [n_refs][A][3]: exists, terminal, outcome */) {
-    const int r = blockIdx.x;
-    if (r >= n_refs) return;
-    const TreeRef ref = refs[r];
-    const TreeHdr *h = ref.hdr;
-    const Node *root = ref.nodes;
-    if (threadIdx.x == 0) {
-        TreeDigest d;
-        d.size = h->size; d.root_ns = ref.stats[0].ns; d.max_depth = h->max_depth; d.error = h->error; d.depth_sum = h->depth_sum;
-        d.plies = h->plies; d.u1_events = h->u1_events; d.stat_levels = h->stat_levels; d.stat_children = h->stat_children;
-        d.stat_expanded = h->stat_expanded; d.stat_played = h->stat_played;
-        d.t_select = h->t_select; d.t_expand = h->t_expand; d.t_playout = h->t_playout; d.t_backup = h->t_backup; d.t_exchange = h->t_exchange;
-        out[r] = d;
-    }
-    const bool expanded = !(root->flags & kLeaf);
-    for (int a = threadIdx.x; a < cells; a += blockDim.x) {
-        int exists = 0, ns = 0, wins = 0, terminal = 0, outcome = 2;
-        if (expanded && !bb_test(root->bb_pos, a) && !bb_test(root->bb_neg, a)) {
-            int rank = __popc(~(root->bb_pos[a >> 5] | root->bb_neg[a >> 5]) & ((1u << (a & 31)) - 1u));
-            for (int w = 0; w < (a >> 5); w++) rank += 32 - __popc(root->bb_pos[w] | root->bb_neg[w]);
-            if (rank < root->n_children) {
-                const int child = root->child_base + rank;
-                exists = 1; ns = ref.stats[child].ns; wins = ref.stats[child].wins;
-                terminal = (ref.nodes[child].flags & kTerminal) ? 1 : 0; outcome = ref.nodes[child].outcome;
-            }
-        }
-        child_counts[((size_t)r * cells + a) * 2] = ns; child_counts[((size_t)r * cells + a) * 2 + 1] = wins;
-        child_info[((size_t)r * cells + a) * 3] = (int8_t)exists; child_info[((size_t)r * cells + a) * 3 + 1] = (int8_t)terminal;
-        child_info[((size_t)r * cells + a) * 3 + 2] = (int8_t)outcome;
-    }
-}
 
 }  // namespace gomoku
 }  // namespace mctsnc

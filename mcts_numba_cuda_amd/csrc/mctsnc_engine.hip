@@ -18,6 +18,7 @@
 
 #include "c4_kernels.hpp"
 #include "gomoku_kernels.hpp"
+#include "reduce_kernels.hpp"
 
 using namespace mctsnc;
 
@@ -87,7 +88,7 @@ struct mctsnc_engine {
     c4::TreeHdr *d_hdrs = nullptr;
     uint64_t *d_rng_playout = nullptr, *d_rng_expand = nullptr;
     c4::TreeRef *d_refs = nullptr;
-    c4::TreeDigest *d_digest = nullptr;
+    unsigned char *d_reduced = nullptr;   // what the final reductions leave for the host (one search)
     uint64_t *d_root_bb = nullptr;
     int32_t *d_root_turns = nullptr, *d_abort = nullptr;
     int64_t n_rng_playout = 0, n_rng_expand = 0;
@@ -103,24 +104,10 @@ struct mctsnc_engine {
     gomoku::Stat *g_stats = nullptr;
     gomoku::TreeHdr *g_hdrs = nullptr;
     gomoku::TreeRef *g_refs = nullptr;
-    gomoku::TreeDigest *g_digest = nullptr;
     int16_t *g_ae = nullptr, *g_root_ae = nullptr;
-    int32_t *g_poc = nullptr, *g_path = nullptr, *g_child_counts = nullptr;
-    int8_t *g_child_info = nullptr;
+    int32_t *g_poc = nullptr, *g_path = nullptr;
     uint32_t *g_root_bb = nullptr;
     bool is_gomoku() const { return cfg.game == MCTSNC_GAME_GOMOKU; }
-};
-
-// What the final reductions need from one tree, whatever the game.
-struct TreeSummary {
-    int32_t size = 0, root_ns = 0, max_depth = 0;
-    int64_t depth_sum = 0;
-    unsigned long long plies = 0, u1_events = 0, stat_levels = 0, stat_children = 0, stat_expanded = 0, stat_played = 0;
-    unsigned long long t_select = 0, t_expand = 0, t_playout = 0, t_backup = 0, t_exchange = 0;
-    std::vector<int16_t> root_ae;                       // A + 2
-    std::vector<int32_t> child_ns, child_wins;          // per action of the root
-    std::vector<uint8_t> child_exists, child_terminal;
-    std::vector<int8_t> child_outcome;
 };
 
 namespace {
@@ -164,20 +151,19 @@ void free_device(mctsnc_engine *e) {
     if (e->d_rng_playout) (void)hipFree(e->d_rng_playout);
     if (e->d_rng_expand) (void)hipFree(e->d_rng_expand);
     if (e->d_refs) (void)hipFree(e->d_refs);
-    if (e->d_digest) (void)hipFree(e->d_digest);
+    if (e->d_reduced) (void)hipFree(e->d_reduced);
     if (e->d_root_bb) (void)hipFree(e->d_root_bb);
     if (e->d_root_turns) (void)hipFree(e->d_root_turns);
     if (e->d_abort) (void)hipFree(e->d_abort);
-    void *gp[] = {e->g_nodes, e->g_stats, e->g_hdrs, e->g_refs, e->g_digest, e->g_ae, e->g_root_ae, e->g_poc, e->g_path,
-                  e->g_child_counts, e->g_child_info, e->g_root_bb};
+    void *gp[] = {e->g_nodes, e->g_stats, e->g_hdrs, e->g_refs, e->g_ae, e->g_root_ae, e->g_poc, e->g_path, e->g_root_bb};
     for (void *q : gp) if (q) (void)hipFree(q);
-    e->g_nodes = nullptr; e->g_stats = nullptr; e->g_hdrs = nullptr; e->g_refs = nullptr; e->g_digest = nullptr; e->g_ae = nullptr;
-    e->g_root_ae = nullptr; e->g_poc = nullptr; e->g_path = nullptr; e->g_child_counts = nullptr; e->g_child_info = nullptr; e->g_root_bb = nullptr;
+    e->g_nodes = nullptr; e->g_stats = nullptr; e->g_hdrs = nullptr; e->g_refs = nullptr; e->g_ae = nullptr;
+    e->g_root_ae = nullptr; e->g_poc = nullptr; e->g_path = nullptr; e->g_root_bb = nullptr;
     if (e->ev0) (void)hipEventDestroy(e->ev0);
     if (e->ev1) (void)hipEventDestroy(e->ev1);
     if (e->stream) (void)hipStreamDestroy(e->stream);
     e->d_nodes = nullptr; e->d_hdrs = nullptr; e->d_rng_playout = nullptr; e->d_rng_expand = nullptr; e->d_refs = nullptr;
-    e->d_digest = nullptr; e->d_root_bb = nullptr; e->d_root_turns = nullptr; e->d_abort = nullptr;
+    e->d_reduced = nullptr; e->d_root_bb = nullptr; e->d_root_turns = nullptr; e->d_abort = nullptr;
     e->ev0 = e->ev1 = nullptr; e->stream = nullptr;
     e->inited = false;
 }
@@ -207,66 +193,6 @@ int upload_rng(mctsnc_engine *e) {
 struct Budget {
     double steps_limit, time_limit, forced;
 };
-
-// Final reductions over trees and actions (src/mctsnc.py:2222-2375) from the per-tree summaries.
-void reduce_result(const mctsnc_engine *e, const TreeSummary *ts, int root_turn, mctsnc_result *out) {
-    const mctsnc_config &c = e->cfg;
-    const int A = c.max_actions, T = c.n_trees;
-    const int16_t *rae = ts[0].root_ae.data();
-    for (int i = 0; i < A + 2; i++) out->root_actions_expanded[i] = rae[i];
-    int nb = e->thrifty ? rae[A + 1] : A;
-    if (nb < 0) nb = 0;
-    if (nb > A) nb = A;
-    out->n_root_entries = nb;
-    for (int b = 0; b < A; b++) { out->root_ns[b] = 0; out->actions_ns[b] = 0; out->actions_ns_wins[b] = 0; out->actions_win_flags[b] = 0; }
-    for (int b = 0; b < nb; b++) {
-        const int action = e->thrifty ? rae[b] : b;
-        if (action < 0 || action >= A) continue;
-        if (e->thrifty || rae[action] != -1) {
-            for (int t = 0; t < T; t++) {
-                out->root_ns[b] += ts[t].root_ns;
-                if (ts[t].child_exists[action]) { out->actions_ns[b] += ts[t].child_ns[action]; out->actions_ns_wins[b] += ts[t].child_wins[action]; }
-            }
-        }
-        out->actions_win_flags[b] = ts[0].child_exists[action] && ts[0].child_terminal[action] && ts[0].child_outcome[action] == root_turn;
-    }
-    // strided max-argmax over (win_flag, n, n_wins) with the left slot kept on ties (:2318-2330)
-    const int size = next_pow2(A);
-    std::vector<int> idx(size);
-    std::vector<uint8_t> f(size, 0);
-    std::vector<int64_t> ns(size, 0), ws(size, 0);
-    for (int a = 0; a < size; a++) {
-        idx[a] = a;
-        if (a < nb) { f[a] = out->actions_win_flags[a]; ns[a] = out->actions_ns[a]; ws[a] = out->actions_ns_wins[a]; }
-    }
-    for (int stride = size >> 1; stride > 0; stride >>= 1)
-        for (int a = 0; a < stride; a++) {
-            const int b = a + stride;
-            if ((f[a] < f[b]) || (f[a] == f[b] && ns[a] < ns[b]) || (f[a] == f[b] && ns[a] == ns[b] && ws[a] < ws[b])) {
-                idx[a] = idx[b]; f[a] = f[b]; ns[a] = ns[b]; ws[a] = ws[b];
-            }
-        }
-    const int best = idx[0];
-    out->best_win_flag = f[0];
-    out->best_n = ns[0];
-    out->best_n_wins = ws[0];
-    out->best_action = e->thrifty ? ((best < A + 2) ? rae[best] : -1) : best;
-    out->depth_sum = 0; out->size_sum = 0; out->max_depth = -1; out->max_size = 0;
-    out->playout_plies = 0; out->u1_events = 0;
-    out->stat_levels = out->stat_children = out->stat_expanded = out->stat_played = 0;
-    const double tick = 1e-8;  // wall_clock64 counts at 100 MHz
-    out->time_select = ts[0].t_select * tick; out->time_expand = ts[0].t_expand * tick;
-    out->time_playout = ts[0].t_playout * tick; out->time_backup = ts[0].t_backup * tick;
-    out->time_exchange = ts[0].t_exchange * tick;
-    for (int t = 0; t < T; t++) {
-        out->stat_levels += ts[t].stat_levels; out->stat_children += ts[t].stat_children;
-        out->stat_expanded += ts[t].stat_expanded; out->stat_played += ts[t].stat_played;
-        out->depth_sum += ts[t].depth_sum; out->size_sum += ts[t].size;
-        if (ts[t].max_depth > out->max_depth) out->max_depth = ts[t].max_depth;
-        if (ts[t].size > out->max_size) out->max_size = ts[t].size;
-        out->playout_plies += ts[t].plies; out->u1_events += ts[t].u1_events;
-    }
-}
 
 // Root of a Gomoku search: bitboards with bit = row * n + column; any arrangement of stones is accepted, as in the
 // reference (its outcome test only looks through the last stone placed).
@@ -352,23 +278,52 @@ int budget_loop(mctsnc_engine *e0, const Budget &bud, Launch launch, int64_t &st
     return MCTSNC_OK;
 }
 
-void finish_results(mctsnc_engine **engines, int n, const std::vector<TreeSummary> &ts, const int32_t *turns, int64_t steps, double t_start,
-                    double t_red, double time_loop, double dev_time, mctsnc_result *out) {
-    const int T = engines[0]->cfg.n_trees;
-    for (int i = 0; i < n; i++) {
-        mctsnc_result *o = out + i;
+// Final reductions over trees and actions (src/mctsnc.py:2222-2375) on the device, one workgroup per search, and the
+// copy of their small result blocks into the callers' structs.  The trees of search j of the launch order are at
+// refs[j * T .. (j + 1) * T); search_of[j] is its index in the caller's arrays.
+template <class Game>
+int reduce_and_finish(mctsnc_engine **engines, int n, const typename Game::Ref *d_refs, unsigned char *d_reduced, const std::vector<int> &search_of,
+                      int64_t steps, double t_start, double time_loop, double dev_time, mctsnc_result *out) {
+    mctsnc_engine *e0 = engines[0];
+    const mctsnc_config &c = e0->cfg;
+    const int A = c.max_actions, T = c.n_trees;
+    const size_t stride = reduced_stride(A);
+    const double t_red = now_s();
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(reduce_kernel<Game>), dim3(n), dim3(kReduceThreads), 0, e0->stream, d_refs, T, A, e0->thrifty ? 1 : 0, d_reduced);
+    HIP_TRY(hipGetLastError());
+    std::vector<unsigned char> host(stride * (size_t)n);
+    HIP_TRY(hipMemcpyAsync(host.data(), d_reduced, host.size(), hipMemcpyDeviceToHost, e0->stream));
+    HIP_TRY(hipStreamSynchronize(e0->stream));
+    const double tick = 1e-8;  // wall_clock64 counts at 100 MHz
+    for (int j = 0; j < n; j++) {
+        const unsigned char *blk = host.data() + stride * (size_t)j;
+        ReducedHeader h;
+        memcpy(&h, blk, sizeof h);
+        mctsnc_result *o = out + search_of[j];
         memset(o, 0, sizeof *o);
-        reduce_result(engines[i], ts.data() + (size_t)i * T, turns[i], o);
         o->steps = steps;
-        engines[i]->has_run = true;
+        o->best_action = h.best_action; o->best_win_flag = h.best_win_flag; o->best_n = h.best_n; o->best_n_wins = h.best_n_wins;
+        o->n_root_entries = h.n_root_entries;
+        memcpy(o->root_ns, blk + reduced_off_root_ns(A), sizeof(int64_t) * A);
+        memcpy(o->actions_ns, blk + reduced_off_ns(A), sizeof(int64_t) * A);
+        memcpy(o->actions_ns_wins, blk + reduced_off_wins(A), sizeof(int64_t) * A);
+        memcpy(o->root_actions_expanded, blk + reduced_off_rae(A), sizeof(int16_t) * (A + 2));
+        memcpy(o->actions_win_flags, blk + reduced_off_flags(A), (size_t)A);
+        o->depth_sum = h.depth_sum; o->size_sum = h.size_sum; o->max_depth = h.max_depth; o->max_size = h.max_size;
+        o->playout_plies = h.plies; o->u1_events = h.u1_events;
+        o->stat_levels = h.stat_levels; o->stat_children = h.stat_children; o->stat_expanded = h.stat_expanded; o->stat_played = h.stat_played;
+        o->time_select = h.t_select * tick; o->time_expand = h.t_expand * tick; o->time_playout = h.t_playout * tick;
+        o->time_backup = h.t_backup * tick; o->time_exchange = h.t_exchange * tick;
+        engines[search_of[j]]->has_run = true;
     }
     const double t_end = now_s();
     for (int i = 0; i < n; i++) {
         out[i].time_loop = time_loop; out[i].time_reduce = t_end - t_red; out[i].time_total = t_end - t_start; out[i].time_device_loop = dev_time;
     }
+    return MCTSNC_OK;
 }
 
-// The per-call device buffers of a batched run (the gathered per-tree pointer records, the roots, the per-tree digests)
+// The per-call device buffers of a batched run (the gathered per-tree pointer records, the roots, the result blocks of the final reductions)
 // are pieces of one block of device memory: a temporary allocation (mctsnc_run_batch) or the static scratch below
 // (mctsnc_run_batch_noalloc).  With a null base only the size is counted.
 struct Workspace {
@@ -381,19 +336,19 @@ struct Workspace {
     }
 };
 
-struct C4BatchBuffers { c4::TreeRef *refs; uint64_t *root_bb; int32_t *turns; c4::TreeDigest *digest; };
-C4BatchBuffers carve_c4(Workspace &w, size_t n_refs) {
+struct C4BatchBuffers { c4::TreeRef *refs; uint64_t *root_bb; int32_t *turns; unsigned char *reduced; };
+C4BatchBuffers carve_c4(Workspace &w, size_t n_refs, size_t n, int A) {
     C4BatchBuffers b;
     b.refs = w.take<c4::TreeRef>(n_refs); b.root_bb = w.take<uint64_t>(2 * n_refs); b.turns = w.take<int32_t>(n_refs);
-    b.digest = w.take<c4::TreeDigest>(n_refs);
+    b.reduced = w.take<unsigned char>(n * reduced_stride(A));
     return b;
 }
 
-struct GomokuBatchBuffers { gomoku::TreeRef *refs; uint32_t *root_bb; int32_t *turns; gomoku::TreeDigest *digest; int32_t *counts; int8_t *info; };
-GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t A) {
+struct GomokuBatchBuffers { gomoku::TreeRef *refs; uint32_t *root_bb; int32_t *turns; unsigned char *reduced; };
+GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t n, int A) {
     GomokuBatchBuffers b;
     b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(16 * n_refs); b.turns = w.take<int32_t>(n_refs);
-    b.digest = w.take<gomoku::TreeDigest>(n_refs); b.counts = w.take<int32_t>(n_refs * A * 2); b.info = w.take<int8_t>(n_refs * A * 3);
+    b.reduced = w.take<unsigned char>(n * reduced_stride(A));
     return b;
 }
 
@@ -457,7 +412,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         if (rc) return rc;
         for (int t = 0; t < T; t++) { bb[2 * ((size_t)i * T + t)] = b2[0]; bb[2 * ((size_t)i * T + t) + 1] = b2[1]; tr[(size_t)i * T + t] = turns[i]; }
     }
-    // The refs / root / digest buffers of a batch hold the trees of the searches with the fewest stones on the board
+    // The refs / root buffers of a batch hold the trees of the searches with the fewest stones on the board
     // first: those have the longest playouts and the largest trees, and a pass with more trees than the device holds
     // hands trees out in this order, so the long searches are not the ones that start last.
     std::vector<int> order((size_t)n_refs);
@@ -472,14 +427,14 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         bb.swap(bb2); tr.swap(tr2);
     }
     // one search with allocation allowed: the engine's own buffers; otherwise pieces of one block
-    C4BatchBuffers buf{e0->d_refs, e0->d_root_bb, e0->d_root_turns, e0->d_digest};
+    C4BatchBuffers buf{e0->d_refs, e0->d_root_bb, e0->d_root_turns, e0->d_reduced};
     BlockHolder block_holder;
     if (n > 1 || fixed) {
         Workspace count, ws;
-        carve_c4(count, (size_t)n_refs);
+        carve_c4(count, (size_t)n_refs, (size_t)n, A);
         int rc = block_holder.get(fixed, count.used, ws);
         if (rc) return rc;
-        buf = carve_c4(ws, (size_t)n_refs);
+        buf = carve_c4(ws, (size_t)n_refs, (size_t)n, A);
         std::vector<c4::TreeRef> sorted((size_t)n_refs);
         for (int k = 0; k < n_refs; k++) sorted[k] = engines[order[k] / T]->h_refs[order[k] % T];
         HIP_TRY(hipMemcpy(buf.refs, sorted.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
@@ -487,7 +442,6 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     c4::TreeRef *const d_refs = buf.refs;
     uint64_t *const d_bb = buf.root_bb;
     int32_t *const d_turns = buf.turns;
-    c4::TreeDigest *const d_digest = buf.digest;
     hipStream_t stream = e0->stream;
     HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint64_t) * 2 * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
@@ -564,29 +518,10 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     }, steps, dev_time, time_loop);
     if (rc) return rc;
 
-    const double t_red = now_s();
-    hipLaunchKernelGGL(c4::digest_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_digest);
-    HIP_TRY(hipGetLastError());
-    std::vector<c4::TreeDigest> dg((size_t)n_refs);
-    HIP_TRY(hipMemcpyAsync(dg.data(), d_digest, sizeof(c4::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipStreamSynchronize(stream));
-    std::vector<TreeSummary> ts((size_t)n_refs);
-    for (int k = 0; k < n_refs; k++) {
-        const c4::TreeDigest &d = dg[k];
-        TreeSummary &t = ts[order[k]];
-        t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
-        t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
-        t.stat_expanded = d.stat_expanded; t.stat_played = d.stat_played;
-        t.t_select = d.t_select; t.t_expand = d.t_expand; t.t_playout = d.t_playout; t.t_backup = d.t_backup; t.t_exchange = d.t_exchange;
-        t.root_ae.assign(d.root_ae, d.root_ae + A + 2);
-        t.child_ns.resize(A); t.child_wins.resize(A); t.child_exists.resize(A); t.child_terminal.resize(A); t.child_outcome.resize(A);
-        for (int a = 0; a < A; a++) {
-            t.child_exists[a] = (d.child_mask >> a) & 1; t.child_ns[a] = d.child_ns[a]; t.child_wins[a] = d.child_wins[a];
-            t.child_terminal[a] = d.child_terminal[a]; t.child_outcome[a] = d.child_outcome[a];
-        }
-    }
-    finish_results(engines, n, ts, turns, steps, t_start, t_red, time_loop, dev_time, out);
-    return MCTSNC_OK;
+    // the trees of a search stay together and in order under the stable sort above: search j of the launch order
+    std::vector<int> search_of((size_t)n);
+    for (int j = 0; j < n; j++) search_of[j] = order[(size_t)j * T] / T;
+    return reduce_and_finish<c4::RootView>(engines, n, d_refs, buf.reduced, search_of, steps, t_start, time_loop, dev_time, out);
 }
 
 int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const int32_t *turns, const Budget &bud, mctsnc_result *out, Workspace *fixed) {
@@ -617,14 +552,14 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         for (int k = 0; k < n_refs; k++) { memcpy(&bb2[16 * (size_t)k], &bb[16 * (size_t)order[k]], 16 * sizeof(uint32_t)); tr2[k] = tr[order[k]]; }
         bb.swap(bb2); tr.swap(tr2);
     }
-    GomokuBatchBuffers buf{e0->g_refs, e0->g_root_bb, e0->d_root_turns, e0->g_digest, e0->g_child_counts, e0->g_child_info};
+    GomokuBatchBuffers buf{e0->g_refs, e0->g_root_bb, e0->d_root_turns, e0->d_reduced};
     BlockHolder block_holder;
     if (n > 1 || fixed) {
         Workspace count, ws;
-        carve_gomoku(count, (size_t)n_refs, (size_t)A);
+        carve_gomoku(count, (size_t)n_refs, (size_t)n, A);
         int rc = block_holder.get(fixed, count.used, ws);
         if (rc) return rc;
-        buf = carve_gomoku(ws, (size_t)n_refs, (size_t)A);
+        buf = carve_gomoku(ws, (size_t)n_refs, (size_t)n, A);
         std::vector<gomoku::TreeRef> sorted((size_t)n_refs);
         for (int k = 0; k < n_refs; k++) sorted[k] = engines[order[k] / T]->hg_refs[order[k] % T];
         HIP_TRY(hipMemcpy(buf.refs, sorted.data(), sizeof(gomoku::TreeRef) * n_refs, hipMemcpyHostToDevice));
@@ -632,9 +567,6 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     gomoku::TreeRef *const d_refs = buf.refs;
     uint32_t *const d_bb = buf.root_bb;
     int32_t *const d_turns = buf.turns;
-    gomoku::TreeDigest *const d_digest = buf.digest;
-    int32_t *const d_counts = buf.counts;
-    int8_t *const d_info = buf.info;
     hipStream_t stream = e0->stream;
     HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint32_t) * 16 * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
@@ -683,39 +615,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     }, steps, dev_time, time_loop);
     if (rc) return rc;
 
-    const double t_red = now_s();
-    hipLaunchKernelGGL(gomoku::digest_kernel, dim3(n_refs), dim3(256), 0, stream, d_refs, n_refs, cells, d_digest, d_counts, d_info);
-    HIP_TRY(hipGetLastError());
-    std::vector<gomoku::TreeDigest> dg((size_t)n_refs);
-    std::vector<int32_t> counts((size_t)n_refs * A * 2);
-    std::vector<int8_t> info((size_t)n_refs * A * 3);
-    std::vector<int16_t> rae((size_t)(A + 2));
-    HIP_TRY(hipMemcpyAsync(dg.data(), d_digest, sizeof(gomoku::TreeDigest) * n_refs, hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipMemcpyAsync(counts.data(), d_counts, counts.size() * sizeof(int32_t), hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipMemcpyAsync(info.data(), d_info, info.size(), hipMemcpyDeviceToHost, stream));
-    HIP_TRY(hipStreamSynchronize(stream));
-    std::vector<TreeSummary> ts((size_t)n_refs);
-    for (int k = 0; k < n_refs; k++) {
-        const int r = order[k];   // position k of the launch held tree r of the batch
-        const gomoku::TreeDigest &d = dg[k];
-        TreeSummary &t = ts[r];
-        t.size = d.size; t.root_ns = d.root_ns; t.max_depth = d.max_depth; t.depth_sum = d.depth_sum;
-        t.plies = d.plies; t.u1_events = d.u1_events; t.stat_levels = d.stat_levels; t.stat_children = d.stat_children;
-        t.stat_expanded = d.stat_expanded; t.stat_played = d.stat_played;
-        t.t_select = d.t_select; t.t_expand = d.t_expand; t.t_playout = d.t_playout; t.t_backup = d.t_backup; t.t_exchange = d.t_exchange;
-        t.root_ae.assign((size_t)A + 2, 0);
-        if (r % T == 0) {  // only tree 0 of an engine holds the memorised row the reductions use
-            HIP_TRY(hipMemcpy(t.root_ae.data(), engines[r / T]->g_root_ae, sizeof(int16_t) * (A + 2), hipMemcpyDeviceToHost));
-        }
-        t.child_ns.resize(A); t.child_wins.resize(A); t.child_exists.resize(A); t.child_terminal.resize(A); t.child_outcome.resize(A);
-        for (int a = 0; a < A; a++) {
-            t.child_ns[a] = counts[((size_t)k * A + a) * 2]; t.child_wins[a] = counts[((size_t)k * A + a) * 2 + 1];
-            t.child_exists[a] = (uint8_t)info[((size_t)k * A + a) * 3]; t.child_terminal[a] = (uint8_t)info[((size_t)k * A + a) * 3 + 1];
-            t.child_outcome[a] = info[((size_t)k * A + a) * 3 + 2];
-        }
-    }
-    finish_results(engines, n, ts, turns, steps, t_start, t_red, time_loop, dev_time, out);
-    return MCTSNC_OK;
+    std::vector<int> search_of((size_t)n);
+    for (int j = 0; j < n; j++) search_of[j] = order[(size_t)j * T] / T;
+    return reduce_and_finish<gomoku::RootView>(engines, n, d_refs, buf.reduced, search_of, steps, t_start, time_loop, dev_time, out);
 }
 
 // use_static: take the per-call device buffers from the static scratch instead of allocating them.
@@ -866,6 +768,7 @@ static int init_device_impl(mctsnc_engine *e) {
     HIP_TRY(hipMalloc(&e->d_rng_playout, sizeof(uint64_t) * 2 * e->n_rng_playout));
     if (!e->acp) HIP_TRY(hipMalloc(&e->d_rng_expand, sizeof(uint64_t) * 2 * T));
     HIP_TRY(hipMalloc(&e->d_root_turns, sizeof(int32_t) * T));
+    HIP_TRY(hipMalloc(&e->d_reduced, reduced_stride(c.max_actions)));
     HIP_TRY(hipMalloc(&e->d_abort, 2 * sizeof(int32_t)));   // [0] abort flag, [1] head of the tree queue of a batch launch
     const size_t rng_per_tree = (size_t)(e->acp ? c.max_actions * c.n_playouts : c.n_playouts);
     if (!e->is_gomoku()) {
@@ -873,7 +776,6 @@ static int init_device_impl(mctsnc_engine *e) {
         HIP_TRY(hipMalloc(&e->d_hdrs, sizeof(c4::TreeHdr) * T));
         HIP_TRY(hipMemset(e->d_hdrs, 0, sizeof(c4::TreeHdr) * T));
         HIP_TRY(hipMalloc(&e->d_refs, sizeof(c4::TreeRef) * T));
-        HIP_TRY(hipMalloc(&e->d_digest, sizeof(c4::TreeDigest) * T));
         HIP_TRY(hipMalloc(&e->d_root_bb, sizeof(uint64_t) * 2 * T));
         std::vector<c4::TreeRef> refs((size_t)T);
         for (int t = 0; t < T; t++) {
@@ -891,7 +793,6 @@ static int init_device_impl(mctsnc_engine *e) {
         HIP_TRY(hipMalloc(&e->g_hdrs, sizeof(gomoku::TreeHdr) * T));
         HIP_TRY(hipMemset(e->g_hdrs, 0, sizeof(gomoku::TreeHdr) * T));
         HIP_TRY(hipMalloc(&e->g_refs, sizeof(gomoku::TreeRef) * T));
-        HIP_TRY(hipMalloc(&e->g_digest, sizeof(gomoku::TreeDigest) * T));
         HIP_TRY(hipMalloc(&e->g_ae, sizeof(int16_t) * (A + 2) * T));
         HIP_TRY(hipMemset(e->g_ae, 0, sizeof(int16_t) * (A + 2) * T));
         HIP_TRY(hipMalloc(&e->g_root_ae, sizeof(int16_t) * (A + 2) * T));
@@ -899,8 +800,6 @@ static int init_device_impl(mctsnc_engine *e) {
         HIP_TRY(hipMalloc(&e->g_poc, sizeof(int32_t) * 2 * A * T));
         HIP_TRY(hipMemset(e->g_poc, 0, sizeof(int32_t) * 2 * A * T));
         HIP_TRY(hipMalloc(&e->g_path, sizeof(int32_t) * gomoku::kMaxPath * T));
-        HIP_TRY(hipMalloc(&e->g_child_counts, sizeof(int32_t) * 2 * A * T));
-        HIP_TRY(hipMalloc(&e->g_child_info, (size_t)3 * A * T));
         HIP_TRY(hipMalloc(&e->g_root_bb, sizeof(uint32_t) * 16 * T));
         std::vector<gomoku::TreeRef> refs((size_t)T);
         for (int t = 0; t < T; t++) {

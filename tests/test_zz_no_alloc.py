@@ -98,21 +98,27 @@ def test_two_calls_in_a_row_equal_the_allocating_entry_point(game, variant, n_tr
 
 def test_a_batch_beyond_the_scratch_is_rejected_with_both_sizes():
     from mcts_numba_cuda_amd import MCTSNC, _lib
+    n = 60   # 60 x 512 trees of a 9x9 board need 140 bytes per tree + 2560 per search = 4.5 MB, more than the 4 MiB of the static array
     engines = []
-    for _ in range(4):   # 4 x 512 trees of a 15x15 board need 5.6 MB, more than the 4 MiB the static array holds
-        e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=np.inf, n_trees=512, n_playouts=1, variant="ocp_prodigal",
-                   device_memory=0.25, verbose_info=False, game="gomoku")
+    for _ in range(n):
+        e = MCTSNC((9, 9), 0, 81, search_time_limit=np.inf, search_steps_limit=np.inf, n_trees=512, n_playouts=1, variant="ocp_prodigal",
+                   device_memory=0.05, verbose_info=False, game="gomoku")
         e.init_device_side_arrays()
         engines.append(e)
-    boards = np.zeros((4, 15, 15), np.int8)
-    extras = np.zeros((4, 1), np.int8)
-    turns = np.ones(4, np.int32)
+    boards = np.zeros((n, 9, 9), np.int8)
+    extras = np.zeros((n, 1), np.int8)
+    turns = np.ones(n, np.int32)
     rc, _ = call("mctsnc_run_batch_noalloc", engines, boards, extras, turns, 2)
     assert rc == -1
     msg = _lib.lib().mctsnc_last_error().decode()
     assert "bytes of device scratch" in msg and str(4 << 20) in msg
     # the same batch passes through the allocating entry point, and a batch that fits still passes afterwards
-    rc, _ = call("mctsnc_run_batch", engines, boards, extras, turns, 2)
+    rc, res_b = call("mctsnc_run_batch", engines, boards, extras, turns, 2)
     assert rc == 0
-    rc, _ = call("mctsnc_run_batch_noalloc", engines[:2], boards[:2], extras[:2], turns[:2], 2)
+    for e in engines:
+        e.reseed()
+    rc, res_a = call("mctsnc_run_batch_noalloc", engines[:50], boards[:50], extras[:50], turns[:50], 2)
     assert rc == 0
+    for a, b in zip(res_a, res_b):   # every engine has the same seed and root: one result, whichever entry point
+        for f in INT_FIELDS:
+            assert getattr(a, f) == getattr(b, f), f
