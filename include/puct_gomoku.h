@@ -67,7 +67,15 @@ void puct_gomoku_destroy(puct_gomoku_engine *engine);
  * puct_select_winner_recalc_launch, expansion / evaluation, the backup of puct_edge_backup_launch) — same results
  * whenever the selections of a step do not race (traversals == 1).  Selection differs from the plain launcher in one
  * point: progressive widening is capped by the node's number of empty cells instead of by the edge dimension, so a
- * fully expanded node is descended through rather than asked for another slot. */
+ * fully expanded node is descended through rather than asked for another slot.
+ * Node limit: a tree holds at most max_nodes nodes (<= 16384, the node field of the packed selection word,
+ * src/puct/puct_gpu_v3_cpp.cu:11-12).  The expansions a step selects in one tree are committed together or not at
+ * all: once they no longer all fit, none of that step is committed in that tree, each of those traversals evaluates
+ * the node it reached as a leaf instead (the evaluator's value of its position), backs that value up its path and
+ * gives its expansion ticket back (a traversal that was asked to widen the root itself has an empty path and leaves
+ * no visit).  The search then goes on over a tree that no longer grows: node_count stays within
+ * `traversals` of max_nodes and never exceeds it, nothing is left in flight, and result->expansions_committed stays
+ * nodes_total - trees. */
 int puct_gomoku_run(puct_gomoku_engine *engine, const int8_t *board, int32_t turn, int32_t steps, int32_t fused,
                     puct_gomoku_result *result);
 

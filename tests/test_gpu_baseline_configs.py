@@ -1,7 +1,9 @@
 """The benchmark configurations at their full sizes, engine against oracle: every node of every tree, the step scratch,
 the reduced root tables and the random streams must agree after the whole search (Connect 4 1x32 ocp_thrifty, 1000
 steps; Connect 4 8x256 acp_thrifty, 20000 steps, 16 GiB pools; Gomoku 15x15 4x128 ocp_thrifty, 2000 steps, 16 GiB
-pools).  The fourth configuration (Connect 4 4x256 acp_prodigal, 5000 steps) is covered by the recorded A100 games."""
+pools; Connect 4 4x256 acp_prodigal, 5000 steps, on the benchmark's own 64 seeded roots: four of them against the
+oracle, all of them in one batched pass against their sequential searches -- the same configuration is also covered
+by the recorded A100 games).  The fifth configuration (PUCT on Gomoku) is in test_gpu_puct_gomoku.py."""
 import numpy as np
 import pytest
 
@@ -38,3 +40,46 @@ def test_gomoku_ocp_thrifty_4x128_2000_steps():
     o = Oracle("gomoku", (15, 15), 0, 225, 4, 128, "ocp_thrifty", ucb_c=2.0, seed=0, device_memory=16.0, threads=16)
     compare_with_oracle(e, o, board, None, turn, steps=2000)
     assert e.performance_info["playouts"] == 2000 * 4 * 128
+
+
+def bench_roots():
+    import bench
+    assert (bench.T, bench.P, bench.STEPS, bench.DEVICE_MEMORY) == (4, 256, 5000, 2.0)
+    return bench.make_roots(bench.N_ROOTS)
+
+
+@pytest.mark.parametrize("k", [0, 21, 42, 63])
+def test_c4_acp_prodigal_4x256_5000_steps_on_a_benchmark_root(k):
+    params = dict(n_trees=4, n_playouts=256, variant="acp_prodigal", device_memory=2.0, ucb_c=2.0, seed=0)
+    board, fills, turn = bench_roots()[k]
+    e = make_engine(params)
+    o = Oracle("c4", (6, 7), 7, 7, 4, 256, "acp_prodigal", ucb_c=2.0, seed=0, device_memory=2.0, threads=16)
+    compare_with_oracle(e, o, board, fills, turn, steps=5000)
+    assert e.steps == 5000 and e.performance_info["playouts"] > 4 * 256 * 5000
+
+
+def test_c4_acp_prodigal_4x256_all_benchmark_roots_batched_equal_sequential():
+    """What bench.py times twice: the 64 roots one MCTSNC.run() after the other (streams restarted per root), and all
+    64 in one run_batch pass on 64 engines."""
+    from helpers import engine_result
+    from mcts_numba_cuda_amd import run_batch
+    params = dict(n_trees=4, n_playouts=256, variant="acp_prodigal", device_memory=2.0, ucb_c=2.0, seed=0)
+    roots = bench_roots()
+    one = make_engine(params)
+    one.search_steps_limit = 5000.0
+    sequential = []
+    for board, fills, turn in roots:
+        one.reseed()
+        one.run(board, fills, turn)
+        sequential.append((engine_result(one), [one.read_array("ns", t).copy() for t in range(4)]))
+    one._release()
+    engines = [make_engine(params) for _ in roots]
+    for e in engines:
+        e.search_steps_limit = 5000.0
+    run_batch(engines, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots])
+    for k, e in enumerate(engines):
+        assert e.steps == 5000
+        assert engine_result(e) == sequential[k][0], f"root {k}"
+        for t in range(4):
+            np.testing.assert_array_equal(e.read_array("ns", t), sequential[k][1][t], err_msg=f"root {k}, tree {t}")
+        e._release()

@@ -91,6 +91,61 @@ def test_concurrent_traversals_build_consistent_trees(shape, stones, trees, trav
     e.close()
 
 
+def test_baseline_config_at_full_size():
+    """The benchmark configuration for PUCT with virtual loss on Gomoku at its size: 15x15 empty board, 16 trees x 16
+    traversals = 256 leaves per step, 4000 steps, node limit 16384 per tree (which this search approaches but does not
+    reach: about 13 000 nodes per tree).  Racy by design, so what is checked are the invariants: structure of every
+    node of every tree, nothing in flight, conservation of visits from every edge to the child's edges."""
+    from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
+    trees, traversals, steps, max_nodes = 16, 16, 4000, 16384
+    board = np.zeros((15, 15), np.int8)
+    e = PUCTGomoku(trees=trees, traversals=traversals, max_nodes=max_nodes, path_depth=64, cpuct=1.5, c_pw=1.0, alpha_pw=0.5,
+                   recalc_attempts=16, dirichlet_alpha=0.3, seed=0)
+    best = e.run(board, 1, steps)
+    h = read_all(e)
+    print(f"nodes per tree: {h['node_count'].tolist()}", flush=True)
+    gc.check_trees(h, board, 1, 15, 15, max_nodes, 64, tree_not_full_required=True)
+    gc.check_visit_flow(h, 64)
+    sel = e.selections
+    assert sum(sel.values()) == steps * trees * traversals and sel["invalid"] == 0 and sel["depth_limit"] == 0
+    assert sum(gc.visits_below(h, t, 0) for t in range(trees)) == sel["expand"] + sel["terminal"]
+    assert e.result.steps == steps and e.result.nodes_total == int(h["node_count"].sum()) == e.result.expansions_committed + trees
+    assert e.result.expansions_committed == sel["expand"]        # every selected expansion was committed: no tree filled up
+    assert e.result.max_nodes_in_tree == int(h["node_count"].max()) > 8000
+    assert board.reshape(-1)[best] == 0 and e.root_n[best] == e.root_n.max() and int(e.root_n.sum()) == sel["expand"] + sel["terminal"]
+    e.close()
+
+
+@pytest.mark.parametrize("traversals", [16, 1])
+def test_node_limit_stops_growth_and_the_search_goes_on(traversals):
+    """With the benchmark's shape but room for 2048 nodes per tree, the trees fill up well before the last step.
+    From then on the expansions of a step are committed together or not at all, the traversals evaluate the node they
+    reached instead, and the search continues on trees that no longer grow."""
+    from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
+    trees, steps, max_nodes = 16, 1500 if traversals > 1 else 6000, 2048
+    board = np.zeros((15, 15), np.int8)
+    e = PUCTGomoku(trees=trees, traversals=traversals, max_nodes=max_nodes, path_depth=64, cpuct=1.5, c_pw=1.0, recalc_attempts=16, seed=2)
+    e.run(board, 1, steps)
+    h = read_all(e)
+    counts = h["node_count"]
+    assert np.all(counts <= max_nodes) and np.all(counts > max_nodes - traversals), counts.tolist()
+    gc.check_trees(h, board, 1, 15, 15, max_nodes, 64)     # structure, and nothing left in flight on any node
+    sel = e.selections
+    assert sum(sel.values()) == steps * trees * traversals and sel["invalid"] == 0
+    assert e.result.nodes_total == int(counts.sum()) == e.result.expansions_committed + trees
+    assert e.result.expansions_committed < sel["expand"]      # expansions selected after the trees were full were not committed ...
+    # ... but were evaluated and backed up along their paths: the root saw more visits than there are nodes, though not
+    # one per selection (a selection whose widening step asked the root itself for another child has an empty path)
+    root_visits = sum(gc.visits_below(h, t, 0) for t in range(trees))
+    assert e.result.expansions_committed < root_visits <= sel["expand"] + sel["terminal"] + sel["depth_limit"]
+    assert int(e.root_n.sum()) == root_visits
+    if traversals == 1:     # deterministic: equal to the sequential oracle, array for array
+        want = po.gomoku_search(board, 1, steps, trees=trees, traversals=1, max_nodes=max_nodes, path_depth=64, cpuct=1.5, c_pw=1.0,
+                                dirichlet_alpha=0.3, seed=2)
+        assert_same_trees(h, want)
+    e.close()
+
+
 def test_finds_the_winning_move():
     """Four in a row with both ends open for the player to move: every expansion of an end cell is a terminal win worth
     +1, so the search concentrates its visits there."""
