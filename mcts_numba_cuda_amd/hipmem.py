@@ -2,6 +2,7 @@
 package without any other GPU library in the process.  The runtime is the one libpuct_hip.so / libmctsnc_hip.so are
 linked against."""
 import ctypes
+import sys
 
 import numpy as np
 
@@ -74,6 +75,8 @@ class DeviceArray:
             hip().hipFree(ptr)
 
     def __del__(self):
+        if sys.is_finalizing():   # the process is going away and the HIP runtime with it: nothing to give back
+            return
         try:
             self.free()
         except Exception:
@@ -97,6 +100,8 @@ class Event:
         return float(ms.value)
 
     def __del__(self):
+        if sys.is_finalizing():
+            return
         try:
             if self._ev:
                 hip().hipEventDestroy(self._ev)

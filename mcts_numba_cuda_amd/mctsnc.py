@@ -6,10 +6,12 @@ forced_search_steps_limit)``, the attributes read by ``game_runner.py`` / ``main
 the reference, so an instance can stand where the numba.cuda one stood.  The search itself (selection, expansion,
 playouts, backup) runs inside one persistent HIP kernel; this module only validates, marshals and reports.
 """
+import atexit
 import ctypes
 import json
 import sys
 import time
+import weakref
 
 import numpy as np
 from numpy import inf
@@ -109,13 +111,28 @@ class MCTSNC:
         self.time_select = self.time_expand = self.time_playout = self.time_backup = 0.0
 
     def __del__(self):
+        # Engines still alive when the interpreter shuts down were already closed by the exit hook below; during
+        # finalisation itself nothing is released any more (the HIP runtime may be tearing down at that point).
+        if not sys.is_finalizing():
+            self._release()
+
+    def close(self):
+        """Frees the engine's device memory, stream and events now.  The instance can be initialised again with
+        init_device_side_arrays().  Also available as a context manager: ``with MCTSNC(...) as ai: ...``."""
         self._release()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+        return False
 
     def _release(self):
         eng = getattr(self, "_engine", None)
         if eng:
-            _lib.lib().mctsnc_destroy(eng)
             self._engine = None
+            _lib.lib().mctsnc_destroy(eng)
 
     def _set_cuda_constants(self):
         """The reference asks numba for MAX_THREADS_PER_BLOCK // 2 (src/mctsnc.py:278-281); 512 on every device it
@@ -177,6 +194,7 @@ class MCTSNC:
         handle = ctypes.c_void_p()
         _lib.check(L.mctsnc_create(ctypes.byref(cfg), ctypes.byref(handle)))
         self._engine = handle
+        _LIVE.add(self)
         try:
             _lib.check(L.mctsnc_init_device(self._engine))
         except Exception:
@@ -399,6 +417,21 @@ class MCTSNC:
         t2 = time.time()
         if self.verbose_info:
             print(f"JSON DUMP DONE. [time: {t2 - t1} s]")
+
+
+_LIVE = weakref.WeakSet()   # instances that hold a device-side engine
+
+
+@atexit.register
+def _close_all_engines():
+    """Interpreter exit: every engine still alive gives its device memory, stream and events back while the HIP
+    runtime is still fully up (Python's exit hooks run before the C runtime's), instead of from a destructor that
+    may run after the runtime's own teardown has begun."""
+    for e in list(_LIVE):
+        try:
+            e._release()
+        except Exception:
+            pass
 
 
 def run_batch(engines, root_boards, root_extra_infos, root_turns, forced_search_steps_limit=np.inf, allocate=True):

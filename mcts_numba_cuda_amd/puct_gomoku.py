@@ -1,6 +1,9 @@
 """Host side of the Gomoku PUCT search loop with virtual loss: a ctypes binding of the puct_gomoku_* entry points of
 libpuct_hip.so (C ABI: include/puct_gomoku.h).  No CPU fallback: without the library or a GPU every call raises."""
+import atexit
 import ctypes
+import sys
+import weakref
 
 import numpy as np
 
@@ -80,9 +83,18 @@ class PUCTGomoku:
         self._engine = ctypes.c_void_p()
         _check(_lib().puct_gomoku_create(ctypes.byref(self.cfg), ctypes.byref(self._engine)))
         self.result = None
+        _LIVE.add(self)
 
     def __del__(self):
+        if not sys.is_finalizing():   # engines alive at interpreter exit were closed by the exit hook below
+            self.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
         self.close()
+        return False
 
     def close(self):
         eng, self._engine = getattr(self, "_engine", None), None
@@ -122,3 +134,16 @@ class PUCTGomoku:
             raise EngineError(-1, f"array {name}: library reports {nbytes} bytes, expected {out.nbytes}")
         _check(_lib().puct_gomoku_read(self._engine, aid, out.ctypes.data, out.nbytes))
         return out
+
+
+_LIVE = weakref.WeakSet()
+
+
+@atexit.register
+def _close_all_engines():
+    """Interpreter exit: engines still alive are released while the HIP runtime is fully up."""
+    for e in list(_LIVE):
+        try:
+            e.close()
+        except Exception:
+            pass
