@@ -456,24 +456,27 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
     dim3 block(e0->block);
-    // All-children playouts with many trees at once: one workgroup per tree (see search_body), which does no work twice and
-    // keeps every CU busy from the queue; fewer trees: a team of one workgroup per column, which is much faster per step.
-    // Measured switch-over (4 trees x 256 playouts per search, G playouts/s, one workgroup per tree against teams): a
-    // batch of searches of different roots, where the longest search sets the pace, from about 900 trees on (768
-    // searches 22 against 14.6, 256 searches 14.7 against 13.8, 192 searches 11.4 against 13.0); one search, whose trees
-    // all take about as long, from about 200 trees on (256 trees: 309 ms against 384 for seven roots; 128 trees: 307
-    // against 223).  MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
-    int solo_from = n > 1 ? 960 : 200;
+    // All-children playouts with many trees at once: one workgroup per tree (see search_body), which does no work twice, lets
+    // no lane idle while others finish their playouts and keeps every CU busy from the queue; fewer trees: a team of one
+    // workgroup per column, whose step is two to four times shorter.  Measured switch-over (searches of 4 trees x 256
+    // playouts, 5000 steps, G playouts/s in one pass, one workgroup per tree against teams): a batch of searches of
+    // different roots, where the longest search sets the pace (a pass of up to 1024 trees lasts as long as its slowest
+    // search, 210 ms against 50 for a team), from about 1300 trees on (768 searches 25.7 against 14.9, 512 searches 23.2
+    // against 14.9, 384 searches 18.4 against 14.7, 256 searches 13.5 against 14.2, 192 searches 11.4 against 13.2); one
+    // search, whose trees all take about as long, from about 200 trees on.  MCTSNC_SOLO_TREES sets one threshold for
+    // both (0 = never).
+    int solo_from = n > 1 ? 1280 : 200;
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
     const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
     if (solo) {
         args.G = 1;
-        // Twice the threads where that keeps whole wavefronts per child: two children are played at a time, which
-        // shortens a tree's step by a third.  Not for the largest passes, where only throughput counts and the idle half
-        // of a round costs 5 % (768 searches: 420 ms against 440; 512 searches: 338 against 316; 256: 300 against 220).
-        bool two_at_a_time = n_refs < 2560;
-        if (const char *v = getenv("MCTSNC_SOLO_PAIRS")) two_at_a_time = atoi(v) != 0;   // for testing either form on small searches
-        if (c.n_playouts >= 64 && 2 * c.n_playouts <= 512 && two_at_a_time) block = dim3(2 * c.n_playouts);
+        // The workgroup plays all playouts of a step as one pool of jobs, with as many lanes as one node has playouts (64 to
+        // 512): lanes take further jobs as theirs end.  Fewer lanes make better use of each (768 searches: 25.7 G playouts/s
+        // with 256 threads, 21.6 with 512, 20.7 with 128) but lengthen the step of the slowest tree, which a pass waits for.
+        int threads = ((c.n_playouts + 63) / 64) * 64;
+        threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
+        if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 512 && t % 64 == 0) threads = t; }   // for experiments
+        block = dim3(threads);
     }
     const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
     if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(c4::search_kernel_solo), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

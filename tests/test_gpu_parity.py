@@ -202,17 +202,18 @@ def test_search_ends_before_visit_counters_overflow():
     assert e.time_total < 30.0
 
 
-@pytest.mark.parametrize("pairs", ["1", "0"], ids=["two-children-at-a-time", "one-child-at-a-time"])
+@pytest.mark.parametrize("threads", ["", "64", "192"], ids=["default-workgroup", "one-wavefront", "three-wavefronts"])
 @pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
-def test_one_workgroup_per_tree_gives_the_same_trees(variant, pairs, monkeypatch):
+def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypatch):
     """With many trees in one pass the all-children search of a tree is done by a single workgroup instead of one per
-    column (MCTSNC_SOLO_TREES sets from how many trees on), which plays two children at a time or, in the largest
-    passes, one (MCTSNC_SOLO_PAIRS).  Forced here for small searches: full state against the oracle over two runs, a
-    pool that fills up, late-game roots, and a batch against single runs."""
+    column (MCTSNC_SOLO_TREES sets from how many trees on), which runs all playouts of a step as one pool of jobs that
+    its lanes take one after the other (MCTSNC_SOLO_THREADS overrides its size).  Forced here for small searches: full
+    state against the oracle over two runs, a pool that fills up, late-game roots, and a batch against single runs."""
     from mcts_numba_cuda_amd import MCTSNC, run_batch
     from oracle.oracle import Oracle
     monkeypatch.setenv("MCTSNC_SOLO_TREES", "1")
-    monkeypatch.setenv("MCTSNC_SOLO_PAIRS", pairs)
+    if threads:
+        monkeypatch.setenv("MCTSNC_SOLO_THREADS", threads)
     rng = np.random.default_rng(41)
     for T, P, steps in ((3, 64, 300), (4, 256, 150), (2, 16, 200)):
         params = dict(n_trees=T, n_playouts=P, variant=variant, device_memory=0.25, ucb_c=2.0, seed=7)
