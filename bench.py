@@ -31,9 +31,41 @@ M, N, A = 6, 7, 7
 T, P, STEPS, DEVICE_MEMORY = 4, 256, 5000, 2.0
 N_ROOTS = 64
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per search-kernel launch from rocprofv3 --pmc FETCH_SIZE (x2, the factor a 1 GiB copy gives) and WRITE_SIZE
-# (x1), averaged over the first four roots: (5299.5 * 2 + 8909.5) KiB
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 20125389
+# Vector ALU peak of the device in wavefront instructions per second: 256 CUs x 4 SIMDs, each issuing one 64-lane
+# instruction per 4 clocks at 2.4 GHz.
+SIMDS, CLOCK_HZ = 1024, 2.4e9
+VALU_PEAK_G = SIMDS * CLOCK_HZ / 4 / 1e9
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def profile_json(name):
+    """The machine-readable block (first ```json fence) of a counter summary under profiles/, or None.  The summaries
+    are written from rocprofv3 --pmc runs of this script; each names the commit it was taken at."""
+    path = os.path.join(PROFILES, name)
+    if not os.path.exists(path):
+        return None
+    text = open(path).read()
+    start = text.find("```json")
+    if start < 0:
+        return None
+    end = text.find("```", start + 7)
+    try:
+        d = json.loads(text[start + 7:end])
+    except ValueError:
+        return None
+    d["file"] = "profiles/" + name
+    return d
+
+
+def valu_roofline(insts, seconds, source, what):
+    """Vector-ALU side of the roofline: SQ_INSTS_VALU (wavefront instructions, from the named counter summary) over the
+    kernel time measured in this run, against the device's issue peak."""
+    if not insts or not seconds:
+        return None
+    achieved = insts / seconds / 1e9
+    return {"bound": "valu", "achieved": achieved, "peak": VALU_PEAK_G, "unit": "G wavefront instructions/s", "frac": achieved / VALU_PEAK_G,
+            "formula": "SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel time x 2.4 GHz)", "what": what,
+            "counter_file": source.get("file"), "counter_commit": source.get("commit")}
 
 
 def has_four(board, token):
@@ -97,8 +129,6 @@ def algorithmic_bytes(res, tree_steps, acp=True, mn_e=M * N + A, A=A, P=P):
 # at the depth limit.  Published: 1.63 M / 0.64 M / 0.38 M selections/s (winner_recalc, device unstated).
 PUCT_SHAPES = {"eq64_d512": (16384, 64, 512), "eq128_d1024": (8192, 128, 1024), "eq256_d1024": (4096, 256, 1024)}
 PUCT_TRAVERSALS = 8
-# HBM bytes per selection launch from rocprofv3 --pmc FETCH_SIZE (x2) and WRITE_SIZE (x1), strict claim
-PUCT_TRAFFIC = {"eq256_d1024": int((45596114.7 * 2 + 2509333.3) * 1024)}
 
 
 def puct_wide_case(trees, actions, depth, warps):
@@ -185,10 +215,29 @@ def bench_puct_select(args):
                            "algorithmic_GB_per_s": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9,
                            "hbm_frac": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9 / HBM_PEAK_GBS},
            "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms / steps * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": alg_bytes / (ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": PUCT_TRAFFIC.get(args.puct_shape),
+                        "frac": alg_bytes / (ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": (profile_json(f"select_kernel_puct_{args.puct_shape}.md") or {}).get("traffic_bytes_per_launch"),
                         "kernel": "select_kernel", "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": ms / steps},
            "cpu_baseline": cpu}
     print(json.dumps(out))
+
+
+def cpu_oracle_baseline(roots):
+    """The CPU oracle (scalar restatement of the reference's kernels, OpenMP over playouts) on a bounded sample of the
+    headline workload: the first 8 roots, 400 MCTS steps each."""
+    from oracle.oracle import Oracle
+    cores = min(16, os.cpu_count() or 1)
+    n_sample_roots, sample_steps = 8, 400
+    cpu_playouts, dt = 0, 0.0
+    for b, f, t in roots[:n_sample_roots]:
+        o = Oracle("c4", (M, N), A, A, T, P, "acp_prodigal", ucb_c=2.0, seed=0, device_memory=DEVICE_MEMORY, threads=cores)
+        t1 = time.perf_counter()
+        o.run(b, f, t, sample_steps)
+        dt += time.perf_counter() - t1
+        cpu_playouts += int(o.result("root_ns").max())
+    return {"value": cpu_playouts / dt, "unit": "playouts/s", "cores": cores, "kind": "port",
+            "mcts_steps_per_s": n_sample_roots * sample_steps / dt,
+            "sample": f"first {n_sample_roots} roots of the workload, {sample_steps} MCTS steps each ({cpu_playouts} playouts), "
+                      "CPU oracle (scalar restatement of the reference's kernels) with OpenMP over playouts"}
 
 
 def bench_gomoku(args):
@@ -208,6 +257,7 @@ def bench_gomoku(args):
         roots.append((board, turn))
     steps = min(args.steps, len(roots)) if args.steps != N_ROOTS else 8
     quiet = io.StringIO()
+    prof = profile_json("search_kernel_gomoku_ocp_thrifty_4x128_counters.md")
     with contextlib.redirect_stdout(quiet):
         e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=2000, n_trees=4, n_playouts=128,
                    variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
@@ -230,6 +280,37 @@ def bench_gomoku(args):
             for key in alg:
                 alg[key] += ab[key]
         wall = time.perf_counter() - t0
+        # the workload as the batch it is: all 32 roots in one run_batch pass (128 workgroups instead of 4 at a time)
+        batched = None
+        if not args.no_batched:
+            from mcts_numba_cuda_amd import run_batch
+            engines = [e]
+            for _ in range(len(roots) - 1):
+                x = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=2000, n_trees=4, n_playouts=128,
+                           variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
+                x.init_device_side_arrays()
+                engines.append(x)
+            for rep in range(2):    # first pass warms the pools up
+                for x in engines:
+                    x.reseed()
+                t1 = time.perf_counter()
+                run_batch(engines, [r[0] for r in roots], None, [r[1] for r in roots])
+                bt = time.perf_counter() - t1
+            bp = sum(x.performance_info["playouts"] for x in engines)
+            bplies = sum(x.performance_info["playout_plies"] for x in engines)
+            bbytes = sum(algorithmic_bytes(x._result, x.steps * 4, acp=False, mn_e=225 + 1, A=225, P=128)["total"] for x in engines)
+            kt = engines[0].time_device_loop
+            batched = {"roots_per_pass": len(engines), "playouts_per_s": bp / bt, "searches_per_s": len(engines) / bt,
+                       "mcts_steps_per_s_all_roots": sum(x.steps for x in engines) / bt, "ms_per_pass": bt * 1e3, "kernel_ms": kt * 1e3,
+                       "playout_plies_per_s": bplies / kt, "algorithmic_GB_per_s": bbytes / kt / 1e9, "hbm_frac": bbytes / kt / 1e9 / HBM_PEAK_GBS,
+                       "valu": valu_roofline((prof or {}).get("batched_32_roots", {}).get("sq_insts_valu_per_pass"), kt, prof or {},
+                                             "one pass over the 32 roots, gomoku::search_kernel<false> with 128 workgroups")}
+            for x in engines[1:]:
+                x._release()
+    per_root = (prof or {}).get("sq_insts_valu_per_root")
+    roofline_valu = None
+    if per_root and len(per_root) >= steps:
+        roofline_valu = valu_roofline(sum(per_root[:steps]), dev, prof, "the timed single searches, gomoku::search_kernel<false> on 4 workgroups")
     cpu = None
     if not args.no_cpu_baseline:
         from oracle.oracle import Oracle
@@ -247,8 +328,9 @@ def bench_gomoku(args):
            "config": {"workload": "Gomoku 15x15, seeded roots with 0-20 random stones, ocp_thrifty n_trees=4 n_playouts=128 ucb_c=2.0 "
                                   "search_steps_limit=2000 device_memory=16GiB seed=0; one MCTSNC.run() per root, sequential"},
            "mcts_steps_per_s": mcts_steps / wall, "playout_plies_per_s": plies / dev, "device_loop_share": dev / wall,
+           "batched": batched, "roofline_valu": roofline_valu,
            "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                        "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
                         "kernel": "mctsnc::gomoku::search_kernel<false>", "algorithmic_bytes_per_launch": alg["total"] / steps,
                         "avg_launch_ms": dev / steps * 1e3,
                         "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
@@ -265,6 +347,7 @@ def bench_puct_gomoku(args):
     from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
     steps = args.steps if args.steps != N_ROOTS else 5
     search_steps = 4000
+    prof = profile_json("search_kernel_puct_gomoku_16_trees_x16.md")
     board = np.zeros((15, 15), np.int8)
     e = PUCTGomoku(trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0, alpha_pw=0.5,
                    recalc_attempts=16, dirichlet_alpha=0.3, seed=0)
@@ -272,6 +355,13 @@ def bench_puct_gomoku(args):
         e.run(board, 1, 200)
     sel = useful = nodes = 0
     dev = 0.0
+    alg = dict(select=0, expand=0, backup=0, total=0)
+    # legal cells of the nodes a search creates (priors are written for each): the trees are the same in every timed
+    # search but for races, so one look at the warm-up's arrays serves all
+    e.run(board, 1, search_steps)
+    counts, legal_arr, expanded_arr = e.read_array("node_count"), e.read_array("node_legal"), e.read_array("node_expanded")
+    created = sum(int(c) - 1 for c in counts)
+    legal_per_created = sum(int(legal_arr[t, 1:c][expanded_arr[t, 1:c] != -1].sum()) for t, c in enumerate(counts)) / max(created, 1)
     t0 = time.perf_counter()
     for _ in range(steps):
         e.run(board, 1, search_steps)
@@ -279,6 +369,19 @@ def bench_puct_gomoku(args):
         useful += e.performance_info["selections"] - e.selections["busy"]
         nodes += e.performance_info["nodes_total"]
         dev += e.result.time_device
+        # Algorithmic bytes with the element sizes of the reference's arrays (src/puct/puct_gpu_v2.py:69-103): a level read
+        # costs the node word, the ticket counter and five 4-byte fields per expanded edge; a selection writes its word,
+        # its length and 4 bytes per path entry; an expansion reads the parent's position and action, writes the child's
+        # position (128 B), turn, value, counters (17 B), links it (12 B) and writes 21 bytes per legal cell of the child
+        # (prior, action, child, N, W, in-flight); the backup reads 8 bytes and updates three 4-byte words per path edge.
+        r = e.result
+        path_edges = r.levels_read - sum(r.selections)          # every selection read one level more than it descended edges
+        legal_cells = legal_per_created * r.expansions_committed
+        b_sel = 8 * r.levels_read + 20 * r.edges_examined + 8 * sum(r.selections) + 4 * path_edges
+        b_exp = r.expansions_committed * (128 + 1 + 128 + 17 + 12) + 21 * legal_cells
+        b_bak = 32 * path_edges
+        for key, v in (("select", b_sel), ("expand", b_exp), ("backup", b_bak), ("total", b_sel + b_exp + b_bak)):
+            alg[key] += v
     wall = time.perf_counter() - t0
     cpu = None
     if not args.no_cpu_baseline:
@@ -298,7 +401,17 @@ def bench_puct_gomoku(args):
                                   "values, c_puct=1.5, c_pw=1.0, alpha_pw=0.5, 16 claim attempts, 4000 steps per search, "
                                   "node limit 16384 per tree"},
            "search_steps_per_s": steps * search_steps / wall, "selections_not_busy_per_s": useful / wall,
-           "nodes_created_per_search": nodes / steps, "device_share": dev / wall, "roofline": None, "cpu_baseline": cpu}
+           "nodes_created_per_search": nodes / steps, "device_share": dev / wall,
+           "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
+                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit")} if prof else None,
+                        "kernel": "puct::search_kernel (select, expand, backup of all 4000 steps in one launch)",
+                        "algorithmic_bytes_per_launch": alg["total"] / steps, "avg_launch_ms": dev / steps * 1e3,
+                        "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
+                        "note": "16 workgroups of 16 wavefronts: bound by the dependent L2 round trips of a level (edge rows, claim, "
+                                "recalculation) and the fp64 Gamma sampling of an expansion, not by memory"},
+           "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_launch"), dev / steps, prof or {}, "one search of 4000 steps"),
+           "cpu_baseline": cpu}
     e.close()
     print(json.dumps(out))
 
@@ -311,6 +424,7 @@ def bench_c4_many(args):
     from mcts_numba_cuda_amd import MCTSNC, run_batch
     roots = make_roots(N_ROOTS)
     n = args.searches
+    prof = profile_json("search_kernel_solo_c4_768_searches.md")
     steps = args.steps if args.steps != N_ROOTS else 3
     with contextlib.redirect_stdout(io.StringIO()):
         engines = []
@@ -345,7 +459,9 @@ def bench_c4_many(args):
                         "frac": abytes / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
                         "kernel": "mctsnc::c4::search_kernel_solo (batches of 960 trees or more), mctsnc::c4::search_kernel<true> below",
                         "algorithmic_bytes_per_launch": abytes, "avg_launch_ms": dev * 1e3},
-           "cpu_baseline": None}
+           "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_pass") if n == (prof or {}).get("searches") else None, dev, prof or {},
+                                          f"one pass over {n} searches"),
+           "cpu_baseline": None if args.no_cpu_baseline else cpu_oracle_baseline(roots)}
     print(json.dumps(out))
 
 
@@ -394,6 +510,7 @@ def main():
 
     roots = make_roots(max(N_ROOTS, 1))
     quiet = io.StringIO()
+    prof = profile_json("search_kernel_c4_acp_prodigal_4x256_counters.md")
 
     def new_engine():
         e = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=T, n_playouts=P,
@@ -449,8 +566,10 @@ def main():
             bp = sum(e.performance_info["playouts"] for e in engines)
             bbytes = sum(algorithmic_bytes(e._result, e.steps * T)["total"] for e in engines)
             batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": nb / bt,
-                       "mcts_steps_per_s_all_roots": nb * STEPS / bt, "ms_per_pass": bt * 1e3,
-                       "algorithmic_GB_per_s": bbytes / bt / 1e9, "hbm_frac": bbytes / bt / 1e9 / HBM_PEAK_GBS}
+                       "mcts_steps_per_s_all_roots": nb * STEPS / bt, "ms_per_pass": bt * 1e3, "kernel_ms": engines[0].time_device_loop * 1e3,
+                       "algorithmic_GB_per_s": bbytes / bt / 1e9, "hbm_frac": bbytes / bt / 1e9 / HBM_PEAK_GBS,
+                       "valu": valu_roofline((prof or {}).get("batched_64_roots", {}).get("sq_insts_valu_per_pass") if nb == N_ROOTS else None,
+                                             engines[0].time_device_loop, prof or {}, "one pass over the 64 roots, search_kernel<true>")}
             for e in engines[1:]:
                 e._release()
             del engines
@@ -468,7 +587,10 @@ def main():
             wbytes = algorithmic_bytes(wide._result, wide.steps * 512)["total"]
             trees_512 = {"n_trees": 512, "root": "empty board", "playouts_per_s": wide.performance_info["playouts"] / wt, "ms_per_search": wt * 1e3,
                          "mcts_steps_per_s": wide.steps / wt, "tree_steps_per_s": wide.steps * 512 / wt,
-                         "algorithmic_GB_per_s": wbytes / wt / 1e9, "hbm_frac": wbytes / wt / 1e9 / HBM_PEAK_GBS}
+                         "kernel_ms": wide.time_device_loop * 1e3,
+                         "algorithmic_GB_per_s": wbytes / wt / 1e9, "hbm_frac": wbytes / wt / 1e9 / HBM_PEAK_GBS,
+                         "valu": valu_roofline((prof or {}).get("trees_512", {}).get("sq_insts_valu_per_search"), wide.time_device_loop, prof or {},
+                                               "one search with 512 trees, search_kernel_solo")}
             wide._release()
         eng._release()      # free the pools now rather than at interpreter exit, after the HIP runtime has shut down
 
@@ -476,29 +598,25 @@ def main():
     launches = args.steps  # one search kernel launch per search at a fixed step budget
     roofline = {"bound": "hbm", "achieved": alg["total"] / dev_time / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": alg["total"] / dev_time / 1e9 / HBM_PEAK_GBS,
-                "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in the named file
+                "traffic": (prof or {}).get("traffic_bytes_per_launch"),
+                "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "launches": prof.get("traffic_launches")} if prof else None,
                 "kernel": "mctsnc::c4::search_kernel<true>", "algorithmic_bytes_per_launch": alg["total"] / launches,
                 "avg_launch_ms": dev_time / launches * 1e3,
                 "stage_bytes_per_launch": {k: v / launches for k, v in alg.items() if k != "total"},
                 "playout_plies_per_s": plies / dev_time,
                 "note": "latency-bound pointer chasing plus integer playouts on 28 workgroups: a few KB of tree data per step"}
 
+    # vector-ALU side: the counted instructions of the timed roots over their kernel time
+    per_root = (prof or {}).get("sq_insts_valu_per_root")
+    roofline_valu = None
+    if per_root and len(per_root) == len(roots):
+        roofline_valu = valu_roofline(sum(per_root[k % len(roots)] for k in range(args.steps)), dev_time, prof,
+                                      "the timed single searches, search_kernel<true> on 28 of 256 CUs")
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
-        from oracle.oracle import Oracle
-        cores = min(16, os.cpu_count() or 1)
-        n_sample_roots, sample_steps = 8, 400
-        cpu_playouts, dt = 0, 0.0
-        for b, f, t in roots[:n_sample_roots]:
-            o = Oracle("c4", (M, N), A, A, T, P, "acp_prodigal", ucb_c=2.0, seed=0, device_memory=DEVICE_MEMORY, threads=cores)
-            t1 = time.perf_counter()
-            o.run(b, f, t, sample_steps)
-            dt += time.perf_counter() - t1
-            cpu_playouts += int(o.result("root_ns").max())
-        cpu_baseline = {"value": cpu_playouts / dt, "unit": "playouts/s", "cores": cores, "kind": "port",
-                        "mcts_steps_per_s": n_sample_roots * sample_steps / dt,
-                        "sample": f"first {n_sample_roots} roots of the workload, {sample_steps} MCTS steps each ({cpu_playouts} playouts), "
-                                  "CPU oracle (scalar restatement of the reference's kernels) with OpenMP over playouts"}
+        cpu_baseline = cpu_oracle_baseline(roots)
 
     cpu_mcts = None
     if not args.no_cpu_baseline:
@@ -530,7 +648,7 @@ def main():
            "device_loop_share": dev_time / elapsed,
            "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
            "batched": batched, "trees_512": trees_512,
-           "roofline": roofline, "cpu_baseline": cpu_baseline, "cpu_mcts": cpu_mcts}
+           "roofline": roofline, "roofline_valu": roofline_valu, "cpu_baseline": cpu_baseline, "cpu_mcts": cpu_mcts}
     print(json.dumps(out))
 
 

@@ -55,6 +55,8 @@ typedef struct {
     int64_t nodes_total;             /* nodes over all trees after the search */
     int32_t max_nodes_in_tree;
     double time_total, time_device;  /* seconds */
+    int64_t levels_read;             /* tree levels the selections read (node word, ticket counter, edge rows) */
+    int64_t edges_examined;          /* expanded edges scored on those levels */
 } puct_gomoku_result;
 
 typedef struct puct_gomoku_engine puct_gomoku_engine;

@@ -190,6 +190,17 @@ int upload_rng(mctsnc_engine *e) {
     return MCTSNC_OK;
 }
 
+// MCTSNC_PLAIN_LAUNCH=1: launch the all-children kernels, whose workgroups wait for each other, as ordinary kernels
+// instead of cooperatively.  The grid is sized to what the device keeps resident either way, so on a device that runs
+// nothing else the workgroups are all resident and the search is the same; what is given up is the runtime's guarantee
+// of it when other kernels share the device (a workgroup that never gets scheduled ends the launch with
+// MCTSNC_E_DEVICE_SYNC through the bounded waits, it cannot hang).  For profilers that do not get along with the
+// runtime's cooperative queue.
+bool plain_launch_requested() {
+    const char *v = getenv("MCTSNC_PLAIN_LAUNCH");
+    return v && atoi(v) != 0;
+}
+
 struct Budget {
     double steps_limit, time_limit, forced;
 };
@@ -496,6 +507,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets of %d (%d workgroups per CU resident)%s\n", n_refs, sets, args.G, per_cu, args.queue ? ", queue" : "");
     }
     const dim3 grid(args.G * sets);
+    const bool plain_launch = plain_launch_requested();
     static std::atomic<uint32_t> launch_counter{0};
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
@@ -510,8 +522,13 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
                 hipLaunchKernelGGL(c4::search_kernel_solo, grid, block, lds, stream, args);
                 HIP_TRY(hipGetLastError());
             } else {
-                void *kargs[] = {&args};
-                HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+                if (plain_launch) {
+                    hipLaunchKernelGGL(c4::search_kernel<true>, grid, block, lds, stream, args);
+                    HIP_TRY(hipGetLastError());
+                } else {
+                    void *kargs[] = {&args};
+                    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+                }
             }
         } else {
             hipLaunchKernelGGL(c4::search_kernel<false>, grid, block, lds, stream, args);
@@ -599,6 +616,7 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         group = (int)((n_refs + n_groups - 1) / n_groups);
         if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees, %d workgroups per tree, %d resident workgroups per CU: launches of %d trees\n", n_refs, e0->G, per_cu, group);
     }
+    const bool plain_launch = plain_launch_requested();
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
         args.nsteps = nsteps;
@@ -607,8 +625,13 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
             args.n_refs = std::min(group, n_refs - start);
             const dim3 grid(e0->G * args.n_refs);
             if (e0->acp) {
-                void *kargs[] = {&args};
-                HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+                if (plain_launch) {
+                    hipLaunchKernelGGL(gomoku::search_kernel<true>, grid, block, lds, stream, args);
+                    HIP_TRY(hipGetLastError());
+                } else {
+                    void *kargs[] = {&args};
+                    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+                }
             } else {
                 hipLaunchKernelGGL(gomoku::search_kernel<false>, grid, block, lds, stream, args);
                 HIP_TRY(hipGetLastError());

@@ -44,6 +44,9 @@ struct SelectArgs {
     const int *node_capacity = nullptr;
     // Attempts of the winner-recalc claim per level; the reference has 2 compiled in.
     int recalc_attempts = kRecalcAttempts;
+    // Optional work counters, uint64 [trees, 8]: entry 6 of a tree's row gains the tree levels its traversals read,
+    // entry 7 the expanded edges examined on those levels (what the algorithmic byte count of a selection is made of).
+    unsigned long long *work = nullptr;
 };
 
 // ---- cross-lane reductions -------------------------------------------------------------------------------------
@@ -153,12 +156,14 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
 
     int final_packed = pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_UNKNOWN);
     int final_len = 0;
+    int levels = 0, edges_seen = 0;
 
     if (!valid_select_shape(a.path_depth, nodes, node_cnt, edges)) {
         final_packed = pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_SHAPE);
     } else {
         int node = 0, depth = 0;
         while (true) {
+            levels += 1;
             const size_t nrow = (size_t)tree * nodes + node;
             const size_t erow = nrow * edges;
 
@@ -196,6 +201,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
             }
 
             const int cur_expanded = node_info;
+            edges_seen += cur_expanded;
 #pragma unroll
             for (int i = 1; i < kPasses; ++i) {
                 n[i] = 0, f[i] = 0, c[i] = -1, p[i] = 0.0f, w[i] = 0.0f;
@@ -324,6 +330,10 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
     if (lane == 0) {
         a.out_selected_node[out] = final_packed;
         a.out_path_len[out] = final_len;
+        if (a.work != nullptr) {
+            atomicAdd(&a.work[(size_t)tree * 8 + 6], (unsigned long long)levels);
+            atomicAdd(&a.work[(size_t)tree * 8 + 7], (unsigned long long)edges_seen);
+        }
     }
 }
 

@@ -414,7 +414,7 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     g.sel = SelectArgs{c->cpuct, c->c_pw, c->alpha_pw, c->soft_winner, g.edge_child, g.edge_prior, g.edge_W, g.edge_N, g.edge_inflight,
                        g.node_expand_inflight, g.node_expanded, g.node_count, out_selected, out_path, out_len,
                        c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth, g.node_legal,
-                       c->recalc_attempts > 0 ? c->recalc_attempts : kRecalcAttempts};
+                       c->recalc_attempts > 0 ? c->recalc_attempts : kRecalcAttempts, g.tally};
     g.bk = BackupArgs{1, nullptr, g.edge_W, g.edge_N, g.edge_inflight, nullptr, g.node_expand_inflight, g.node_count,
                       out_selected, out_path, out_len, g.path_values, c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth};
     g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes; g.steps = 0;
@@ -501,6 +501,8 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
         }
         for (int k = 0; k < 5; ++k) res->selections[k] += (int64_t)tally[t * 8 + k];
         res->expansions_committed += (int64_t)tally[t * 8 + 5];
+        res->levels_read += (int64_t)tally[t * 8 + 6];
+        res->edges_examined += (int64_t)tally[t * 8 + 7];
         res->nodes_total += counts[t];
         if (counts[t] > res->max_nodes_in_tree) res->max_nodes_in_tree = counts[t];
     }

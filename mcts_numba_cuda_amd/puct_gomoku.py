@@ -32,7 +32,8 @@ class Result(ctypes.Structure):
     _fields_ = [("steps", ctypes.c_int64), ("best_action", ctypes.c_int32), ("best_n", ctypes.c_int64),
                 ("root_n", ctypes.c_int64 * 256), ("root_w", ctypes.c_double * 256), ("selections", ctypes.c_int64 * 5),
                 ("expansions_committed", ctypes.c_int64), ("nodes_total", ctypes.c_int64),
-                ("max_nodes_in_tree", ctypes.c_int32), ("time_total", ctypes.c_double), ("time_device", ctypes.c_double)]
+                ("max_nodes_in_tree", ctypes.c_int32), ("time_total", ctypes.c_double), ("time_device", ctypes.c_double),
+                ("levels_read", ctypes.c_int64), ("edges_examined", ctypes.c_int64)]
 
 
 class EngineError(RuntimeError):
@@ -120,6 +121,7 @@ class PUCTGomoku:
             "steps": int(res.steps), "selections": int(total), "selections_per_second": total / max(res.time_device, 1e-12),
             "steps_per_second": res.steps / max(res.time_device, 1e-12), "expansions": int(res.expansions_committed),
             "nodes_total": int(res.nodes_total), "max_nodes_in_tree": int(res.max_nodes_in_tree),
+            "levels_read": int(res.levels_read), "edges_examined": int(res.edges_examined),
             "times_[ms]": {"total": 1e3 * res.time_total, "device": 1e3 * res.time_device}}
         self.best_action = int(res.best_action)
         return self.best_action
