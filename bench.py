@@ -456,8 +456,9 @@ def bench_c4_many(args):
                                   "search_steps_limit=5000 device_memory=60MiB each, all in one run_batch pass"},
            "searches_per_s": n / dt, "trees_in_flight": n * T, "mcts_steps_per_s_all_searches": n * STEPS / dt,
            "roofline": {"bound": "hbm", "achieved": abytes / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": abytes / dev / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                        "kernel": "mctsnc::c4::search_kernel_solo (batches of 960 trees or more), mctsnc::c4::search_kernel<true> below",
+                        "frac": abytes / dev / 1e9 / HBM_PEAK_GBS,
+                        "traffic": (prof or {}).get("traffic_bytes_per_launch") if n == (prof or {}).get("searches") else None,
+                        "kernel": "mctsnc::c4::search_kernel_solo (batches of 1280 trees or more), mctsnc::c4::search_kernel<true> below",
                         "algorithmic_bytes_per_launch": abytes, "avg_launch_ms": dev * 1e3},
            "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_pass") if n == (prof or {}).get("searches") else None, dev, prof or {},
                                           f"one pass over {n} searches"),
