@@ -775,7 +775,12 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                     s_explore[lvl][a] = (n > 0) ? (double)args.ucb_c * __dsqrt_rn(det_log((double)N) / (double)n) : 0.0;
                 }
             }
-            if (!ACP || SOLO) __syncthreads();   // the workgroups of a team meet at the barrier that ends the exchange
+            if (!ACP || SOLO) {
+                // every wavefront of a workgroup that searches a tree alone stored child records earlier in the step; the
+                // next walk reads records past the L1, so the stores must have been acknowledged by the L2 (long since)
+                wait_own_stores_at_l2();
+                __syncthreads();
+            }   // (the workgroups of a team meet at the barrier that ends the exchange)
         }
         if (SOLO && wave == 0) {  // the children's results: the counts of the pool, or the stored outcome times P
             if (lane < ncols) {

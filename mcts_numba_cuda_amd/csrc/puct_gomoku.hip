@@ -282,10 +282,15 @@ __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const u
 }
 
 // Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one.  All wavefronts of a
-// tree run on one CU: stores leave its write-through L1 towards the L2 they all share (the workgroup-scope release waits
-// for that), but the L1 keeps lines that device-scope atomics of other wavefronts have changed underneath it, so the
-// acquire side drops the L1.  No L2 write-back is needed.
+// tree run on one CU and share its write-through L1 and the L2 behind it, so no L2 write-back is needed; what is needed
+// is (1) that every wavefront's stores and atomics of the phase have been acknowledged by the L2 before any wavefront
+// goes on -- a workgroup-scope release fence does not wait for that on one CU (it lowers to no vector-memory wait), and
+// a counter that another wavefront incremented could otherwise still be read with its old value after the barrier,
+// which once in some thousand searches handed out an expansion slot twice -- hence the explicit wait on the
+// wavefront's own outstanding vector memory operations; and (2) that the L1 drops the lines which device-scope atomics
+// of other wavefronts have changed underneath it: the agent-scope acquire.
 __device__ __forceinline__ void phase_barrier() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");

@@ -62,7 +62,7 @@ def check_trees(h, root_board, root_turn, m, n, max_nodes, path_depth, tree_not_
             child_visits = 0
             for s in range(ne):
                 child = int(h["edge_child"][t, node, s])
-                assert 0 < child < count and child not in seen_children
+                assert 0 < child < count and child not in seen_children, (t, node, s, child, count, ne)
                 seen_children.add(child)
                 a = acts[s]
                 cpos, cneg = cells_of(h["node_board"][t, child, :8], cells), cells_of(h["node_board"][t, child, 8:], cells)
