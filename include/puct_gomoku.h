@@ -70,6 +70,9 @@ void puct_gomoku_destroy(puct_gomoku_engine *engine);
  * whenever the selections of a step do not race (traversals == 1).  Selection differs from the plain launcher in one
  * point: progressive widening is capped by the node's number of empty cells instead of by the edge dimension, so a
  * fully expanded node is descended through rather than asked for another slot.
+ * Edge slots: an expansion puts the child into the node's next free edge slot at the time it is committed (slots are
+ * in descending prior order); the slot field of the selection word is the ticket that entitled the traversal to expand,
+ * and the tickets of one step are not always contiguous, the expanded edges of a node always are.
  * Node limit: a tree holds at most max_nodes nodes (<= 16384, the node field of the packed selection word,
  * src/puct/puct_gpu_v3_cpp.cu:11-12).  The expansions a step selects in one tree are committed together or not at
  * all: once they no longer all fit, none of that step is committed in that tree, each of those traversals evaluates

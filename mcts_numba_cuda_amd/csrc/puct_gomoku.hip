@@ -185,7 +185,7 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
     const size_t out = (size_t)tree * g.sel.warps + wave;
     const int raw = g.sel.out_selected_node[out];
     const int kind = (raw >> PUCT_PACKED_KIND_SHIFT) & PUCT_PACKED_KIND_MASK;
-    const int node = raw & PUCT_PACKED_NODE_MASK, slot = (raw >> PUCT_PACKED_SLOT_SHIFT) & PUCT_PACKED_EDGE_MASK;
+    const int node = raw & PUCT_PACKED_NODE_MASK, ticket_slot = (raw >> PUCT_PACKED_SLOT_SHIFT) & PUCT_PACKED_EDGE_MASK;
     const int plen = g.sel.out_path_len[out];
     const size_t trow = (size_t)tree * g.sel.nodes;
     const uint64_t tree_seed = psyn_tree_seed(g.seed, tree);
@@ -199,7 +199,7 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
         turn = g.node_turn[trow + node];
         wave_lds_fence();
     }
-    const int wants = (kind == PUCT_SELECT_EXPAND && slot < n_legal) ? 1 : 0;
+    const int wants = (kind == PUCT_SELECT_EXPAND && ticket_slot < n_legal) ? 1 : 0;
     if (lane == 0) {
         lds.want[wave] = wants;
         atomicAdd(&g.tally[(size_t)tree * 8 + kind], 1ull);
@@ -222,6 +222,14 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
     if (wants && fits) {
         const int child = base + before;
         const size_t erow = (trow + node) * kEdges;
+        // The edge slot the child goes into is the node's next free one, taken here, not the slot of the selection's
+        // ticket: tickets of one step can leave a hole (a traversal whose widening limit, computed from visit counts
+        // that include other traversals' virtual losses, is smaller gives its ticket back while one with a larger limit
+        // has already drawn the next), and the expanded edges of a node must stay contiguous.  With one traversal per
+        // tree the two are the same slot.
+        int slot_taken = 0;
+        if (lane == 0) slot_taken = atomicAdd(&g.node_expanded[trow + node], 1);
+        const int slot = __builtin_amdgcn_readfirstlane(slot_taken);
         const int action = g.edge_action[erow + slot];
         uint32_t *mine = board + (turn > 0 ? 0 : 8);
         if (lane == 0) mine[action >> 5] |= 1u << (action & 31);
@@ -241,7 +249,6 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
             g.edge_child[erow + slot] = child;
             g.edge_N[erow + slot] = 1;
             g.edge_W[erow + slot] = -v_child;
-            atomicAdd(&g.node_expanded[trow + node], 1);
         }
         if (!terminal) write_priors(g, tree, child, board, lane, bh, child_legal);
         u = -v_child;
@@ -284,11 +291,11 @@ __global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const u
 // Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one.  All wavefronts of a
 // tree run on one CU and share its write-through L1 and the L2 behind it, so no L2 write-back is needed; what is needed
 // is (1) that every wavefront's stores and atomics of the phase have been acknowledged by the L2 before any wavefront
-// goes on -- a workgroup-scope release fence does not wait for that on one CU (it lowers to no vector-memory wait), and
-// a counter that another wavefront incremented could otherwise still be read with its old value after the barrier,
-// which once in some thousand searches handed out an expansion slot twice -- hence the explicit wait on the
-// wavefront's own outstanding vector memory operations; and (2) that the L1 drops the lines which device-scope atomics
-// of other wavefronts have changed underneath it: the agent-scope acquire.
+// goes on -- a workgroup-scope release fence does not wait for that on one CU (it lowers to no vector-memory wait), and a
+// counter that another wavefront changed with a fire-and-forget atomic could otherwise still be read with its old value
+// after the barrier -- hence the explicit wait on the wavefront's own outstanding vector memory operations; and (2) that
+// the L1 drops the lines which device-scope atomics of other wavefronts have changed underneath it: the agent-scope
+// acquire.
 __device__ __forceinline__ void phase_barrier() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");

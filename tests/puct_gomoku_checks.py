@@ -62,7 +62,9 @@ def check_trees(h, root_board, root_turn, m, n, max_nodes, path_depth, tree_not_
             child_visits = 0
             for s in range(ne):
                 child = int(h["edge_child"][t, node, s])
-                assert 0 < child < count and child not in seen_children, (t, node, s, child, count, ne)
+                assert 0 < child < count and child not in seen_children, (
+                    t, node, s, child, count, ne, h["edge_child"][t, node, :ne + 3].tolist(), h["edge_n"][t, node, :ne + 3].tolist(),
+                    int(h["node_expand_inflight"][t, node]), int(h["node_legal"][t, node]))
                 seen_children.add(child)
                 a = acts[s]
                 cpos, cneg = cells_of(h["node_board"][t, child, :8], cells), cells_of(h["node_board"][t, child, 8:], cells)
