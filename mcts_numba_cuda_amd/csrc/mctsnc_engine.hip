@@ -39,7 +39,10 @@ int fail(int code, const char *fmt, ...) {
 #define HIP_TRY(expr)                                                                               \
     do {                                                                                            \
         hipError_t err__ = (expr);                                                                  \
-        if (err__ != hipSuccess) return fail(MCTSNC_E_HIP, "%s failed: %s", #expr, hipGetErrorString(err__)); \
+        if (err__ != hipSuccess) {                                                                  \
+            (void)hipGetLastError(); /* the runtime remembers the error: a later launch check must not find it */ \
+            return fail(MCTSNC_E_HIP, "%s failed: %s", #expr, hipGetErrorString(err__));          \
+        }                                                                                           \
     } while (0)
 
 double now_s() {
@@ -375,7 +378,7 @@ struct BlockHolder {
             return MCTSNC_OK;
         }
         hipError_t err = hipMalloc(&owned, need);
-        if (err != hipSuccess) { owned = nullptr; return fail(MCTSNC_E_HIP, "hipMalloc of the batch buffers (%zu bytes) failed: %s", need, hipGetErrorString(err)); }
+        if (err != hipSuccess) { (void)hipGetLastError(); owned = nullptr; return fail(MCTSNC_E_HIP, "hipMalloc of the batch buffers (%zu bytes) failed: %s", need, hipGetErrorString(err)); }
         out.base = static_cast<unsigned char *>(owned); out.size = need; out.used = 0;
         return MCTSNC_OK;
     }

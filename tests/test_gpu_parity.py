@@ -397,6 +397,17 @@ def test_device_scope_fences_give_the_same_trees(game, variant, monkeypatch):
         compare_with_oracle(e, o, board, None, turn, 12)
 
 
+def test_device_scope_fences_replay_a_recorded_game(archives, monkeypatch):
+    """The general path again (MCTSNC_AGENT_FENCES), over thousands of steps per search instead of hundreds: the first
+    game of the reference's experiment with acp_prodigal 4 x 256 (17 searches of 5000 to 5900 steps with carried random
+    streams) and of the one with acp_thrifty 8 x 256 (10 searches) must give the recorded root tables and tree statistics."""
+    monkeypatch.setenv("MCTSNC_AGENT_FENCES", "1")
+    for a in ("mctsnc_5_inf_4_256_acp_prodigal", "mctsnc_1_inf_8_256_acp_thrifty"):
+        key = replay.find_archive(archives, "mcts_5_inf_vanilla", a)
+        n = replay.replay_archive(archives[key], make_engine, engine_run_search, max_games=1)
+        assert n >= 3, key
+
+
 def test_time_limited_batch_over_several_launches_through_the_queue():
     """A time budget splits a batch into several kernel launches, each of which hands the trees beyond the resident
     workgroup sets out through the queue again: every search must end where a single search of as many steps ends."""

@@ -54,3 +54,33 @@ def test_an_engine_per_host_thread(games):
     for a, b in zip(alone, together):
         assert b is not None and a[0] == b[0]
         np.testing.assert_array_equal(a[1], b[1])
+
+
+def test_a_failed_initialisation_keeps_no_device_memory():
+    """An engine whose node pool cannot be allocated (512 trees x 2^24 nodes x 128 bytes is over a terabyte) must give
+    back what it had allocated before the failure (stream, events, 0.9 GB of generator states), both on the failing
+    call and on destroy; the free device memory afterwards is what it was before."""
+    import ctypes
+    from mcts_numba_cuda_amd import _lib
+    L = _lib.lib()
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    warm = _engine("c4")     # the runtime's own first-use allocations happen here, not inside the measurement
+    warm.close()
+    before = free_bytes()
+    cfg = _lib.Config(game=0, board_m=6, board_n=7, extra_info_memory=7, max_actions=7, n_trees=512, n_playouts=512, variant=3, ucb_c=2.0,
+                      seed=0, max_tree_size=2**24, device=0)
+    for _ in range(2):
+        h = ctypes.c_void_p()
+        assert L.mctsnc_create(ctypes.byref(cfg), ctypes.byref(h)) == 0
+        assert L.mctsnc_init_device(h) == -2 and b"hipMalloc" in L.mctsnc_last_error()
+        assert free_bytes() >= before - (8 << 20)          # nothing of the half-built engine is still held
+        assert L.mctsnc_init_device(h) == -2                # a second attempt on the same handle fails the same way
+        L.mctsnc_destroy(h)
+    assert free_bytes() >= before - (8 << 20)
