@@ -144,6 +144,7 @@ __device__ inline int exact_outcome(ExactScratch &s, int m, int n, int turn, int
     return 0;
 }
 
+template <class Game>
 __device__ inline int exact_playout(ExactScratch &s, int m, int n, const uint32_t *pos, const uint32_t *neg, int turn, int last_action,
                                     uint64_t &s0, uint64_t &s1, uint32_t &plies, uint32_t &u1) {
     for (int i = 0; i < 32 * 32; i++) s.board[i] = 0;
@@ -152,7 +153,7 @@ __device__ inline int exact_playout(ExactScratch &s, int m, int n, const uint32_
         const int v = bb_test(pos, c) ? 1 : (bb_test(neg, c) ? -1 : 0);
         s.board[(c / n) * 32 + (c % n)] = (int8_t)v;
     }
-    int outcome = (last_action >= 0) ? exact_outcome(s, m, n, turn, last_action) : 2;
+    int outcome = (last_action >= 0) ? Game::exact_outcome(s, m, n, turn, last_action) : 2;
     for (;;) {
         if (outcome != 2) return outcome;
         if (s.legal[512] == 0) {
@@ -174,7 +175,7 @@ __device__ inline int exact_playout(ExactScratch &s, int m, int n, const uint32_
         s.legal[512] = (int16_t)(count - 1);
         plies++;
         turn = -turn;
-        outcome = exact_outcome(s, m, n, turn, last_action);
+        outcome = Game::exact_outcome(s, m, n, turn, last_action);
     }
 }
 
@@ -190,6 +191,26 @@ __device__ __forceinline__ uint32_t exact_five_starts(uint32_t packed) {
     const u16x2 exact = five & ~(v << 1) & ~(v >> 5);
     return __builtin_bit_cast(uint32_t, exact);
 }
+
+// ------------------------------------------------------------------------------------------------------------------------
+// Gomoku as the game of the placement-game step skeleton below (search_kernel): what differs between games in which an
+// action places a stone on an empty cell of a board of up to 16 x 16 and a line of stones through the last one decides.
+// The reference's plugin functions (src/mctsnc_game_mechanics.py:56-87, Gomoku bodies :181-280) map onto it like this:
+// is_action_legal and legal_actions_playout (cell empty; row-major list, swap-remove) and take_action[_playout] (place
+// the stone) are the skeleton's own, being the same for every such game; compute_outcome is the game's:
+//   wins_through      at node creation: does the stone just placed at `cell` complete a winning line of `mine`
+//   winning_starts    in a playout: the same test on two 16-bit line words packed in one dword (bit s set = a winning run
+//                     starts at s), and reach(): the starts whose run covers position p of a line
+//   exact_outcome     the byte-array form used when a playout is replayed exactly
+// ------------------------------------------------------------------------------------------------------------------------
+struct Gomoku {
+    static __device__ __forceinline__ bool wins_through(const uint32_t *mine, int m, int n, int cell) { return five_through(mine, m, n, cell); }
+    static __device__ __forceinline__ uint32_t winning_starts(uint32_t packed) { return exact_five_starts(packed); }
+    static __device__ __forceinline__ uint32_t reach(uint32_t p) { return (0x1fu << p) >> 4; }   // starts of a run of five through position p
+    static __device__ __forceinline__ int exact_outcome(ExactScratch &s, int m, int n, int turn, int last_action) {
+        return gomoku::exact_outcome(s, m, n, turn, last_action);
+    }
+};
 
 struct LeafInfo {
     int32_t node, depth, turn, flags, outcome, size;
@@ -222,8 +243,9 @@ __host__ __device__ inline size_t playout_lds_bytes(int cells, int lines, int th
     return ((size_t)((cells + 3) / 4) + (size_t)lines) * sizeof(uint32_t) * threads;
 }
 
-template <bool ACP>
-__global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
+// The step skeleton for placement games: the whole search of the launch's trees by Game's rules.
+template <class Game, bool ACP>
+__global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args) {
     // The G workgroups of a tree are consecutive, and consecutive blockIdx values go to different XCDs: every tree is
     // spread over all XCDs, whatever the number of trees, and G can be any number that stays resident.  (Keeping a tree
     // inside one XCD and its L2 was measured too: 4 % slower with 8 trees, where both layouts allow the same G, and up
@@ -350,7 +372,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                 mine[a >> 5] |= 1u << (a & 31);
                 if (mover == 1) nd.bb_pos[a >> 5] |= 1u << (a & 31); else nd.bb_neg[a >> 5] |= 1u << (a & 31);
                 int outcome = 2;
-                if (five_through(mine, m, n, a)) outcome = mover;
+                if (Game::wins_through(mine, m, n, a)) outcome = mover;
                 else {
                     int occ = 0;
                     for (int w = 0; w < 8; w++) occ += __popc(nd.bb_pos[w] | nd.bb_neg[w]);
@@ -497,9 +519,9 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                             const uint32_t bit_j = (1u << jj) << sh;
                             w_row |= bit_j; w_col |= (1u << i) << sh; w_dia |= bit_j; w_ant |= bit_j;
                             *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
-                            const uint32_t win_j = (0x1fu << jj) >> 4, win_i = (0x1fu << i) >> 4;  // starts of a run of five through the stone
-                            const uint32_t hit = exact_five_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
-                            const uint32_t hit2 = exact_five_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
+                            const uint32_t win_j = Game::reach(jj), win_i = Game::reach(i);  // starts of a winning run through the stone
+                            const uint32_t hit = Game::winning_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
+                            const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
                             *slot_n = last_n;   // swap-remove of the next draw
                             if ((hit | hit2) != 0) { status = 1; outcome = outcome_if_win; rg = rg_now; }
                             else if (count == 0) { status = 2; outcome = 0; rg = rg_now; }
@@ -519,7 +541,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
                         for (int q = 0; q < nthreads; q++) {
                             if (tid == q && redo) {
                                 s0 = s0_start; s1 = s1_start; plies = plies_start;
-                                outcome = exact_playout(s_exact, m, n, s_cbb, s_cbb + 8, pturn, last_action, s0, s1, plies, u1);
+                                outcome = exact_playout<Game>(s_exact, m, n, s_cbb, s_cbb + 8, pturn, last_action, s0, s1, plies, u1);
                             }
                             __syncthreads();
                         }
@@ -737,6 +759,9 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel(SearchArgs args) {
         }
     }
 }
+
+// the kernels of this library: Gomoku's rules on the skeleton
+template <bool ACP> constexpr auto search_kernel = search_kernel_for<Gomoku, ACP>;
 
 // Where the final reductions (reduce_kernels.hpp) find the root's visit count, the row memorised at the first step and
 // the counters of the root's children in this layout: the children of the root are its empty cells in row-major order,
