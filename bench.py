@@ -568,6 +568,7 @@ def main():
             bbytes = sum(algorithmic_bytes(e._result, e.steps * T)["total"] for e in engines)
             batched = {"roots_per_pass": nb, "playouts_per_s": bp / bt, "searches_per_s": nb / bt,
                        "mcts_steps_per_s_all_roots": nb * STEPS / bt, "ms_per_pass": bt * 1e3, "kernel_ms": engines[0].time_device_loop * 1e3,
+                       "playout_plies_per_s": sum(e.performance_info["playout_plies"] for e in engines) / engines[0].time_device_loop,
                        "algorithmic_GB_per_s": bbytes / bt / 1e9, "hbm_frac": bbytes / bt / 1e9 / HBM_PEAK_GBS,
                        "valu": valu_roofline((prof or {}).get("batched_64_roots", {}).get("sq_insts_valu_per_pass") if nb == N_ROOTS else None,
                                              engines[0].time_device_loop, prof or {}, "one pass over the 64 roots, search_kernel<true>")}
@@ -588,7 +589,7 @@ def main():
             wbytes = algorithmic_bytes(wide._result, wide.steps * 512)["total"]
             trees_512 = {"n_trees": 512, "root": "empty board", "playouts_per_s": wide.performance_info["playouts"] / wt, "ms_per_search": wt * 1e3,
                          "mcts_steps_per_s": wide.steps / wt, "tree_steps_per_s": wide.steps * 512 / wt,
-                         "kernel_ms": wide.time_device_loop * 1e3,
+                         "kernel_ms": wide.time_device_loop * 1e3, "playout_plies_per_s": wide.performance_info["playout_plies"] / wide.time_device_loop,
                          "algorithmic_GB_per_s": wbytes / wt / 1e9, "hbm_frac": wbytes / wt / 1e9 / HBM_PEAK_GBS,
                          "valu": valu_roofline((prof or {}).get("trees_512", {}).get("sq_insts_valu_per_search"), wide.time_device_loop, prof or {},
                                                "one search with 512 trees, search_kernel_solo")}
