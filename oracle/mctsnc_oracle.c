@@ -12,16 +12,18 @@
  * reference's names, dtypes and index conventions (per tree instead of one
  * [T, S, ...] block, grown on demand instead of sized to max_tree_size).
  *
- * What pins this file (tests/test_oracle_golden.py, tests/test_oracle_units.py):
+ * What pins this file (tests/test_oracle_golden.py, tests/test_oracle_units.py, tests/test_readme_examples.py):
  *   - the reference's recorded full-tree dumps extras/mctsnc_{ocp,acp}_thrifty_c4_1000steps.json
  *     (parents, children of expanded nodes, depths, turns, ns, ns_wins, last-step scratch);
  *   - the reference's recorded A100 experiment logs (root tables, tree statistics,
  *     RNG carry-over across consecutive searches);
+ *   - the two complete runs printed in the reference's README.md: Connect 4 (8 trees x 128 playouts, all-children,
+ *     6373 steps) and Gomoku 15x15 (same settings, 442 steps, 94 359 552 playouts), every printed root row, the best
+ *     action and the tree statistics to the last digit: the Gomoku search end to end (legal list order, swap-remove,
+ *     exactly-five, stream layout with 225 actions, reduction over 225 actions);
  *   - independent brute-force / textbook checks of the game rules, the tournament
  *     arg-max and the RNG jump.
- * Parity unpinned (no recorded artefact exercises them): the Gomoku end-to-end
- * search (only its mechanics are checked against independent rules), and the
- * memory-exhausted (-3) paths.
+ * Parity unpinned (no recorded artefact exercises them): the memory-exhausted (-3) paths.
  *
  * Deliberate deviations from the reference where the reference reads or writes
  * out of bounds (they are deterministic definitions, listed for the record):
