@@ -572,9 +572,9 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
             // ---- the playouts of the step as one pool of jobs ----
             // Every playout (played-out node, generator t) is a job of its own: it uses its own generator, so the order
             // and the lane in which jobs run do not matter.  The jobs are dealt to the wavefronts in equal contiguous
-            // shares; a lane whose playout has ended takes the wavefront's next job in the same loop iteration, so lanes
-            // do not idle until the longest playout of the wavefront is over (with Connect 4's short, very unequal
-            // playouts they would for two thirds of the time).  What a playout starts from (stones, column fills, the
+            // shares; lanes whose playouts have ended take the wavefront's next jobs in the same loop, so lanes do not idle
+            // until the longest playout of the wavefront is over (with Connect 4's short, very unequal playouts they
+            // would for two thirds of the time).  What a playout starts from (stones, column fills, the
             // ascending list of legal columns) is worked out once per node here instead of once per playout.
             if (wave == 0) {
                 const int a = lane & 7;
@@ -620,55 +620,67 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 bool active = next + lane < last;
                 if (active) take_job(next + lane);
                 next += kWave;
-                while (__ballot(active) != 0ull) {
-                    int status = 0;   // 0 = game goes on, 1 = mover won, 2 = board full, 3 = ordinal == count
-                    if (active) { status = Game::ply(m, H, a, b, fills, list, count, rg); n++; }
-                    const unsigned long long done = __ballot(status != 0);
-                    if (done != 0ull) {
-                        const int col = (int)(job_turn_col >> 8), turn_a = (int)(int8_t)(job_turn_col & 0xffu);
-                        uint64_t *const st = s_rng + 2 * ((size_t)col * P + job_t);
-                        if (__ballot(status == 3) != 0ull) {  // rare: a draw rounded up to 1.0f; replay with the exact emulation, one playout at a time
-                            if (lane == 0) {
-                                uint32_t spins = 0;
-                                while (atomicCAS(&s_lock, 0u, 1u) != 0u) {
-                                    __builtin_amdgcn_s_sleep(4);
-                                    if (++spins > kSpinLimit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
-                                }
-                            }
-                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                            unsigned long long redo = __ballot(status == 3);
-                            while (redo) {
-                                const int l = (int)__ffsll((long long)redo) - 1;
-                                redo &= redo - 1ull;
-                                if (lane == l) {
-                                    const PoolChild pc = s_pool[__popc(solo_played & ((1u << col) - 1u))];
-                                    uint64_t q0 = st[0], q1 = st[1];   // the generator as it was when the playout started
-                                    const uint64_t cur = ((uint64_t)pc.a_hi << 32) | pc.a_lo, opp = ((uint64_t)pc.b_hi << 32) | pc.b_lo;
-                                    const uint64_t ppos = (turn_a == 1) ? cur : opp, pneg = (turn_a == 1) ? opp : cur;
-                                    const int outcome = Game::exact_playout(s_exact_solo, geo, ppos, pneg, turn_a, q0, q1, plies, u1);
-                                    st[0] = q0; st[1] = q1;
-                                    if (outcome != 0) atomicAdd(&s_cnt[col][outcome == 1 ? 1 : 0], 1);
-                                }
-                            }
-                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                            if (lane == 0) atomicExch(&s_lock, 0u);
-                        }
-                        if (status == 1 || status == 2) {
-                            st[0] = ((uint64_t)rg.s0h << 32) | rg.s0l; st[1] = ((uint64_t)rg.s1h << 32) | rg.s1l;
-                            plies += n;
-                            if (status == 1) {
-                                const int winner = (n & 1u) ? turn_a : -turn_a;   // the side that made the last move
-                                atomicAdd(&s_cnt[col][winner == 1 ? 1 : 0], 1);
-                            }
-                        }
-                        // the lanes that are done take the wavefront's next jobs in lane order
-                        const int mine = next + (int)__popcll(done & ((1ull << lane) - 1ull));
-                        if (status != 0) {
-                            active = mine < last;
-                            if (active) take_job(mine);
-                        }
-                        next += (int)__popcll(done);
+                // Finished lanes are served in batches: booking a result and fetching the next job costs about 40
+                // instructions for the whole wavefront whenever it runs, and with 64 lanes some lane finishes in almost
+                // every iteration; so it runs only once kRefill lanes are waiting (or all are), and not at all once the
+                // wavefront's jobs have run out, until its last playout has ended.  Measured, G playouts/s, thresholds 1 /
+                // 4 / 8 / 16: one search of 512 trees x 256 playouts 13.8 / 14.4 / 15.0 / 15.1, 768 searches of 4 trees
+                // 26.4 / 25.7 / 26.8 / 28.0.
+                constexpr int kRefill = 16;
+                int status = 0;        // of the lane's job: 0 = running, 1 = mover won, 2 = board full, 3 = ordinal == count
+                bool pending = false;  // the job has ended and its result is not booked yet
+                for (;;) {
+                    if (active) {
+                        status = Game::ply(m, H, a, b, fills, list, count, rg);
+                        n++;
+                        if (status != 0) { active = false; pending = true; }
                     }
+                    const unsigned long long idle = __ballot(!active);
+                    const int n_idle = (int)__popcll(idle);
+                    const bool jobs_left = next < last;
+                    if (!(n_idle == kWave || (jobs_left && n_idle >= kRefill))) continue;
+                    const int col = (int)(job_turn_col >> 8), turn_a = (int)(int8_t)(job_turn_col & 0xffu);
+                    uint64_t *const st = s_rng + 2 * ((size_t)col * P + job_t);
+                    if (__ballot(pending && status == 3) != 0ull) {  // rare: a draw rounded up to 1.0f; replay with the exact emulation, one playout at a time
+                        if (lane == 0) {
+                            uint32_t spins = 0;
+                            while (atomicCAS(&s_lock, 0u, 1u) != 0u) {
+                                __builtin_amdgcn_s_sleep(4);
+                                if (++spins > kSpinLimit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                            }
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+                        unsigned long long redo = __ballot(pending && status == 3);
+                        while (redo) {
+                            const int l = (int)__ffsll((long long)redo) - 1;
+                            redo &= redo - 1ull;
+                            if (lane == l) {
+                                const PoolChild pc = s_pool[__popc(solo_played & ((1u << col) - 1u))];
+                                uint64_t q0 = st[0], q1 = st[1];   // the generator as it was when the playout started
+                                const uint64_t cur = ((uint64_t)pc.a_hi << 32) | pc.a_lo, opp = ((uint64_t)pc.b_hi << 32) | pc.b_lo;
+                                const uint64_t ppos = (turn_a == 1) ? cur : opp, pneg = (turn_a == 1) ? opp : cur;
+                                const int outcome = Game::exact_playout(s_exact_solo, geo, ppos, pneg, turn_a, q0, q1, plies, u1);
+                                st[0] = q0; st[1] = q1;
+                                if (outcome != 0) atomicAdd(&s_cnt[col][outcome == 1 ? 1 : 0], 1);
+                            }
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                        if (lane == 0) atomicExch(&s_lock, 0u);
+                    }
+                    if (pending && (status == 1 || status == 2)) {
+                        st[0] = ((uint64_t)rg.s0h << 32) | rg.s0l; st[1] = ((uint64_t)rg.s1h << 32) | rg.s1l;
+                        plies += n;
+                        if (status == 1) {
+                            const int winner = (n & 1u) ? turn_a : -turn_a;   // the side that made the last move
+                            atomicAdd(&s_cnt[col][winner == 1 ? 1 : 0], 1);
+                        }
+                    }
+                    pending = false;
+                    if (!jobs_left) break;   // every lane is idle and there is nothing left to hand out
+                    // the idle lanes take the wavefront's next jobs in lane order
+                    const int mine = next + (int)__popcll(idle & ((1ull << lane) - 1ull));
+                    if (!active && mine < last) { take_job(mine); active = true; }
+                    next += n_idle;
                 }
             }
             st_played += __popc(solo_played);
@@ -1042,6 +1054,11 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
 // One workgroup per tree: the generators in LDS leave room for four workgroups per CU, i.e. four wavefronts per SIMD
 // and 128 vector registers (with 96 the playout loop spills).
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) search_kernel_solo(SearchArgs args) { search_trees<Connect4, true, true>(args); }
+
+// The same with up to 1024 threads (16 wavefronts: the four per SIMD that 128 registers allow, i.e. one workgroup per CU):
+// all children of a step at once with two playouts per lane, the form closest to a team's step a single workgroup can
+// take.  Only taken on request (MCTSNC_SOLO_THREADS above 512); see the design notes for what it measures.
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) search_kernel_solo_wide(SearchArgs args) { search_trees<Connect4, true, true>(args); }
 
 
 // Where the final reductions (reduce_kernels.hpp) find the root's visit count, the row memorised at the first step and

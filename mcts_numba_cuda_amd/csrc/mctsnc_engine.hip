@@ -477,23 +477,31 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     // different roots, where the longest search sets the pace (a pass of up to 1024 trees lasts as long as its slowest
     // search, 210 ms against 50 for a team), from about 1300 trees on (768 searches 25.7 against 14.9, 512 searches 23.2
     // against 14.9, 384 searches 18.4 against 14.7, 256 searches 13.5 against 14.2, 192 searches 11.4 against 13.2); one
-    // search, whose trees all take about as long, from about 200 trees on.  MCTSNC_SOLO_TREES sets one threshold for
-    // both (0 = never).
-    int solo_from = n > 1 ? 1280 : 200;
+    // search, whose trees all take about as long, from about 450 trees on (ms per search of 256 playouts, teams against
+    // one workgroup per tree: 256 trees 203 / 209, 384 trees 271 / 318, 512 trees 362 / 318 -- with up to two trees per
+    // CU a workgroup's step costs the same whether its CU holds one tree or two, teams grow with the number of trees).
+    // MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
+    int solo_from = n > 1 ? 1280 : 448;
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) solo_from = atoi(v);
     const bool solo = e0->acp && solo_from > 0 && n_refs >= solo_from;
     if (solo) {
         args.G = 1;
-        // The workgroup plays all playouts of a step as one pool of jobs, with as many lanes as one node has playouts (64 to
-        // 512): lanes take further jobs as theirs end.  Fewer lanes make better use of each (768 searches: 25.7 G playouts/s
-        // with 256 threads, 21.6 with 512, 20.7 with 128) but lengthen the step of the slowest tree, which a pass waits for.
+        // The workgroup plays all playouts of a step as one pool of jobs (lanes take further jobs as theirs end) with as many
+        // lanes as one node has playouts, twice as many while there are no more than two trees per CU (64 to 512).  Fewer
+        // lanes make better use of each but lengthen the step of the slowest tree, which a pass waits for; four workgroups
+        // per CU stay resident (LDS).  Measured, G playouts/s: 768 searches of 4 trees, 256 threads 25.7, 512 threads 21.6, 128
+        // threads 20.7; one search with 512 trees (two per CU), 512 threads 15.1, 256 threads 13.7, 1024 threads 11.1.
+        int cus_now = 0;
+        HIP_TRY(hipDeviceGetAttribute(&cus_now, hipDeviceAttributeMultiprocessorCount, c.device));
         int threads = ((c.n_playouts + 63) / 64) * 64;
+        if (n_refs <= 2 * cus_now) threads *= 2;
         threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
-        if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 512 && t % 64 == 0) threads = t; }   // for experiments
+        if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 1024 && t % 64 == 0) threads = t; }   // for experiments
         block = dim3(threads);
     }
     const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
-    if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(c4::search_kernel_solo), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const auto solo_kernel = block.x > 512 ? c4::search_kernel_solo_wide : c4::search_kernel_solo;
+    if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(solo_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
     // all its workgroups must be resident together: a batch with more trees than resident sets starts one tree per
     // set and hands the remaining trees out through a queue as sets finish.
@@ -502,7 +510,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     if (e0->acp) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel_solo, block.x, lds));
+        if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, solo_kernel, block.x, lds));
         else HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
         const int resident_sets = (int)((int64_t)per_cu * cus / (8 * args.G)) * 8;
         if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * args.G);
@@ -522,7 +530,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
                 HIP_TRY(hipMemcpyAsync(args.queue, &sets, sizeof(int32_t), hipMemcpyHostToDevice, stream));
             }
             if (solo) {   // nothing is exchanged between workgroups: an ordinary launch
-                hipLaunchKernelGGL(c4::search_kernel_solo, grid, block, lds, stream, args);
+                hipLaunchKernelGGL(solo_kernel, grid, block, lds, stream, args);
                 HIP_TRY(hipGetLastError());
             } else {
                 if (plain_launch) {

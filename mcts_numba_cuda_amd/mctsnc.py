@@ -247,7 +247,7 @@ class MCTSNC:
         self.best_win_flag = bool(res.best_win_flag)
         self.best_n = np.int64(res.best_n)
         self.best_n_wins = np.int64(res.best_n_wins)
-        self.best_q = float(self.best_n_wins / self.best_n) if self.best_n > 0 else float("nan")
+        self.best_q = float(self.best_n_wins / self.best_n) if self.best_n > 0 else np.nan
         self.time_total = res.time_total
         self.time_loop = res.time_loop
         self.time_device_loop = res.time_device_loop
@@ -275,8 +275,8 @@ class MCTSNC:
         entry["n"] = int(self._actions_ns[i])
         entry["n_wins"] = int(self._actions_ns_wins[i])
         # plain Python floats, so that the table prints as the reference's does whatever the numpy version
-        entry["q"] = entry["n_wins"] / entry["n"] if entry["n"] > 0 else float("nan")
-        entry["ucb"] = float(entry["q"] + self.ucb_c * np.sqrt(np.log(entry["n_root"]) / entry["n"])) if entry["n"] > 0 else float("inf")
+        entry["q"] = entry["n_wins"] / entry["n"] if entry["n"] > 0 else np.nan
+        entry["ucb"] = float(entry["q"] + self.ucb_c * np.sqrt(np.log(entry["n_root"]) / entry["n"])) if entry["n"] > 0 else np.inf
         return entry
 
     def _make_actions_info_thrifty(self):

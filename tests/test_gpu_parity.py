@@ -202,7 +202,7 @@ def test_search_ends_before_visit_counters_overflow():
     assert e.time_total < 30.0
 
 
-@pytest.mark.parametrize("threads", ["", "64", "192"], ids=["default-workgroup", "one-wavefront", "three-wavefronts"])
+@pytest.mark.parametrize("threads", ["", "64", "192", "896"], ids=["default-workgroup", "one-wavefront", "three-wavefronts", "fourteen-wavefronts"])
 @pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
 def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypatch):
     """With many trees in one pass the all-children search of a tree is done by a single workgroup instead of one per
