@@ -237,7 +237,7 @@ __device__ __forceinline__ bool bb_has_four(BB p, int H) {
 
 // What a playout of one node starts from: the stones of the side to move (a) and of the other side (b) as 32-bit halves,
 // the column fills and the ascending list of legal columns as 4-bit fields, the number of legal columns, and the side
-// to move (low byte) with the node's column.  Worked out once per node and step by the workgroup that searches a tree
+// to move (low byte) with the node's column (second byte) and the number of stones on the board (third byte).  Worked out once per node and step by the workgroup that searches a tree
 // alone, once per playout elsewhere.
 struct PoolChild { uint32_t a_lo, a_hi, b_lo, b_hi, fills, list; int32_t count; uint32_t turn_col; };
 
@@ -277,39 +277,43 @@ struct Connect4 {
             fills |= (uint32_t)h << (4 * c);
             if (h < g.m) { list |= (uint32_t)c << (4 * count); count++; }
         }
-        pc.fills = fills; pc.list = list; pc.count = count; pc.turn_col = (uint32_t)(turn & 0xff) | ((uint32_t)column << 8);
+        pc.fills = fills; pc.list = list; pc.count = count;
+        pc.turn_col = (uint32_t)(turn & 0xff) | ((uint32_t)column << 8) | ((uint32_t)__popcll(occ) << 16);
         return pc;
     }
 
-    // One random move of the side whose stones are `a`; afterwards a and b have changed places.  Returns 0 = game goes
-    // on, 1 = the mover won, 2 = board full, 3 = the drawn ordinal equals the count (the uniform rounded up to 1.0f).
-    static __device__ __forceinline__ int ply(int m, int H, BB &a, BB &b, uint32_t &fills, uint32_t &list, int &count, Rng32 &r) {
+    // One random move of the side whose stones are `me` (the other side's stones are not needed: the column fills say
+    // where a stone lands); the caller alternates the two sides.  Returns 0 = game goes on, 1 = the mover won, 2 = board
+    // full, 3 = the drawn ordinal equals the count (the uniform rounded up to 1.0f).
+    static __device__ __forceinline__ int ply(int m, int H, BB &me, uint32_t &fills, uint32_t &list, int &count, Rng32 &r) {
         uint32_t xl, xh;
         rng_next32(r, xl, xh);
         const float u = uniform_from_bits(xl, xh);
         const int ord = (int)(u * (float)count);  // single-precision product, as the reference's float32 * int16
         const int sh = ord * 4;
-        const int c = (int)((list >> sh) & 7u);
-        const int c4 = c * 4;
-        const int h = (int)((fills >> c4) & 15u);
-        const int pos = c * H + h;
-        const uint32_t bit = 1u << (pos & 31);
-        a.lo |= (pos < 32) ? bit : 0u;
-        a.hi |= (pos < 32) ? 0u : bit;
+        const uint32_t c = (list >> sh) & 7u;
+        const uint32_t c4 = c * 4u;
+        const uint32_t h = (fills >> c4) & 15u;
+        uint32_t pos;   // c * H + h at full rate (the compiler would take the 64-bit multiply-add, a quarter-rate instruction)
+        asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(pos) : "v"(c), "s"(H), "v"(h));
+        const uint32_t bit = 1u << (pos & 31u);
+        uint32_t upper = (uint32_t)((int32_t)(pos << 26) >> 31);   // all ones for a cell of the upper half
+        asm("" : "+v"(upper));                                      // (kept as a mask: two and-or instructions instead of compare and selects)
+        me.lo |= bit & ~upper;
+        me.hi |= bit & upper;
         fills += 1u << c4;
-        const bool full = (h + 1 == m);
+        const bool full = (h + 1u == (uint32_t)m);
         const uint32_t low = (1u << sh) - 1u;
         list = full ? ((list & low) | ((list >> 4) & ~low)) : list;  // a full column leaves the ascending list
         const bool hit = ord >= count;
         count -= full ? 1 : 0;
-        const bool win = bb_has_four(a, H);
-        const BB t = a; a = b; b = t;
-        return hit ? 3 : (win ? 1 : (count == 0 ? 2 : 0));
+        const bool win = bb_has_four(me, H);
+        if (!(hit || win || count == 0)) return 0;
+        return hit ? 3 : (win ? 1 : 2);
     }
 
     // cur: stones of the side to move, opp: the other side's.  Returns -1 / 0 / +1, or 2 when a draw of the uniform
-    // rounded up to 1.0f (the caller then replays the playout with exact_playout).  Lanes leave through the loop
-    // condition only.
+    // rounded up to 1.0f (the caller then replays the playout with exact_playout).
     static __device__ __forceinline__ int fast_playout(const Geometry &g, uint64_t cur, uint64_t opp, int turn,
                                                        uint64_t &s0, uint64_t &s1, uint32_t &plies) {
         const PoolChild pc = playout_start(g, cur, opp, turn, 0);
@@ -321,12 +325,14 @@ struct Connect4 {
         Rng32 r;
         r.s0l = (uint32_t)s0; r.s0h = (uint32_t)(s0 >> 32); r.s1l = (uint32_t)s1; r.s1h = (uint32_t)(s1 >> 32);
         int status;
-        uint32_t n = 0;
-        do {
-            status = ply(m, H, a, b, fills, list, count, r);
-            n++;
-        } while (status == 0);
+        for (;;) {   // the two sides in turn
+            status = ply(m, H, a, fills, list, count, r);
+            if (status != 0) break;
+            status = ply(m, H, b, fills, list, count, r);
+            if (status != 0) break;
+        }
         s0 = ((uint64_t)r.s0h << 32) | r.s0l; s1 = ((uint64_t)r.s1h << 32) | r.s1l;
+        const uint32_t n = (uint32_t)(__popc(a.lo) + __popc(a.hi) + __popc(b.lo) + __popc(b.hi)) - (pc.turn_col >> 16);   // plies made
         plies += n;
         const int mover = (n & 1u) ? turn : -turn;  // side that made the last move
         return status == 1 ? mover : (status == 2 ? 0 : 2);
@@ -428,6 +434,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
     typename Game::Exact &s_exact_solo = *reinterpret_cast<typename Game::Exact *>(s_rng + (size_t)args.n * args.P * 2);
     __shared__ PoolChild s_pool[kMaxCols];           // SOLO: the nodes played out in this step, ready to start a playout from
     __shared__ int32_t s_pool_n;                     // SOLO: how many of them,
+    __shared__ int32_t s_pool_next;                  // SOLO: the first playout job of the step that no wavefront has taken yet
     __shared__ uint32_t s_pool_mask;                 // SOLO: and which columns (bit 0 alone when the selected node itself is played out)
     __shared__ int32_t s_cnt[kMaxCols][2];           // SOLO: per played-out node, playouts won by -1 / by +1
     __shared__ uint32_t s_lock;                      // SOLO: the replay scratch is used by one wavefront at a time
@@ -571,11 +578,11 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
             if (timing) { const unsigned long long t2 = wall_clock64(); tk_expand += t2 - tk; tk = t2; }
             // ---- the playouts of the step as one pool of jobs ----
             // Every playout (played-out node, generator t) is a job of its own: it uses its own generator, so the order
-            // and the lane in which jobs run do not matter.  The jobs are dealt to the wavefronts in equal contiguous
-            // shares; lanes whose playouts have ended take the wavefront's next jobs in the same loop, so lanes do not idle
-            // until the longest playout of the wavefront is over (with Connect 4's short, very unequal playouts they
-            // would for two thirds of the time).  What a playout starts from (stones, column fills, the
-            // ascending list of legal columns) is worked out once per node here instead of once per playout.
+            // and the lane in which jobs run do not matter.  Every wavefront takes an equal share of every node's playouts;
+            // lanes whose playouts have ended take the wavefront's next jobs in the same loop, so lanes do not idle until
+            // the longest playout of the wavefront is over (with Connect 4's short, very unequal playouts they would for
+            // two thirds of the time).  What a playout starts from (stones, column fills, the ascending list of legal
+            // columns) is worked out once per node here instead of once per playout.
             if (wave == 0) {
                 const int a = lane & 7;
                 bool playable = false;
@@ -594,52 +601,59 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                     s_pool[__popc(pmask & ((1u << a) - 1u))] = Game::playout_start(geo, cur, opp, turn_a, a);
                     s_cnt[a][0] = 0; s_cnt[a][1] = 0;
                 }
-                if (lane == 0) { s_pool_n = __popc(pmask); s_pool_mask = pmask; }
+                if (lane == 0) { s_pool_n = __popc(pmask); s_pool_mask = pmask; s_pool_next = 0; }
             }
             __syncthreads();
             solo_played = s_pool_mask;
             {
-                const int n_nodes = s_pool_n, n_jobs = n_nodes * P;
-                const int pshift = 31 - __clz(P);                                    // P is a power of two
-                int next = (int)((long long)n_jobs * wave / nwaves);                // this wavefront's share: [next, last)
-                const int last = (int)((long long)n_jobs * (wave + 1) / nwaves);
+                const int n_jobs = s_pool_n * P;
+                const int pshift = 31 - __clz(P);   // P is a power of two
                 const int m = geo.m, H = geo.H;
                 BB a = {0, 0}, b = {0, 0};
-                uint32_t fills = 0, list = 0, n = 0, job_turn_col = 0, job_t = 0;
+                uint32_t fills = 0, list = 0, job_turn_col = 0, job_t = 0;
                 int count = 0;
                 Rng32 rg = {0, 0, 0, 0};
-                auto take_job = [&](int j) {   // j < last
+                auto take_job = [&](int j, BB &mover, BB &waiting) {   // j < n_jobs; mover: the stones of the side that moves next
                     const PoolChild pc = s_pool[j >> pshift];
                     job_t = (uint32_t)j & (uint32_t)(P - 1);
-                    a.lo = pc.a_lo; a.hi = pc.a_hi; b.lo = pc.b_lo; b.hi = pc.b_hi; fills = pc.fills; list = pc.list; count = pc.count;
-                    job_turn_col = pc.turn_col; n = 0;
-                    const uint64_t *st = s_rng + 2 * ((size_t)(pc.turn_col >> 8) * P + job_t);
+                    mover.lo = pc.a_lo; mover.hi = pc.a_hi; waiting.lo = pc.b_lo; waiting.hi = pc.b_hi; fills = pc.fills; list = pc.list; count = pc.count;
+                    job_turn_col = pc.turn_col;
+                    const uint64_t *st = s_rng + 2 * ((size_t)((pc.turn_col >> 8) & 0xffu) * P + job_t);
                     const uint64_t q0 = st[0], q1 = st[1];
                     rg.s0l = (uint32_t)q0; rg.s0h = (uint32_t)(q0 >> 32); rg.s1l = (uint32_t)q1; rg.s1h = (uint32_t)(q1 >> 32);
                 };
-                bool active = next + lane < last;
-                if (active) take_job(next + lane);
-                next += kWave;
+                // The wavefronts take jobs from one counter, in batches, as their lanes fall idle: how fast a wavefront gets
+                // through its playouts depends on how many wavefronts share its SIMD, which a workgroup cannot choose, and with
+                // fixed shares the step waited for the slowest one (8 wavefronts: 31 us against 22 for the first to finish).
+                auto grab = [&](int n) -> int {   // the first of n consecutive jobs (which may lie past the end)
+                    int first = 0;
+                    if (lane == 0) first = atomicAdd(&s_pool_next, n);
+                    return __builtin_amdgcn_readfirstlane(first);
+                };
+                int first = grab(kWave);
+                bool exhausted = first + kWave >= n_jobs;   // the counter has passed the end: nothing more to take
+                bool active = first + lane < n_jobs;
+                if (active) take_job(first + lane, a, b);
                 // Finished lanes are served in batches: booking a result and fetching the next job costs about 40
                 // instructions for the whole wavefront whenever it runs, and with 64 lanes some lane finishes in almost
                 // every iteration; so it runs only once kRefill lanes are waiting (or all are), and not at all once the
-                // wavefront's jobs have run out, until its last playout has ended.  Measured, G playouts/s, thresholds 1 /
+                // jobs have run out, until the wavefront's last playout has ended.  Measured, G playouts/s, thresholds 1 /
                 // 4 / 8 / 16: one search of 512 trees x 256 playouts 13.8 / 14.4 / 15.0 / 15.1, 768 searches of 4 trees
                 // 26.4 / 25.7 / 26.8 / 28.0.
                 constexpr int kRefill = 16;
                 int status = 0;        // of the lane's job: 0 = running, 1 = mover won, 2 = board full, 3 = ordinal == count
                 bool pending = false;  // the job has ended and its result is not booked yet
-                for (;;) {
+                // One iteration for the side whose stones are `me`, the same side in every lane (a job taken now starts
+                // with the next iteration, so its side to move goes where `other` is); true when the wavefront is done.
+                auto iteration = [&](BB &me, BB &other) -> bool {
                     if (active) {
-                        status = Game::ply(m, H, a, b, fills, list, count, rg);
-                        n++;
+                        status = Game::ply(m, H, me, fills, list, count, rg);
                         if (status != 0) { active = false; pending = true; }
                     }
                     const unsigned long long idle = __ballot(!active);
                     const int n_idle = (int)__popcll(idle);
-                    const bool jobs_left = next < last;
-                    if (!(n_idle == kWave || (jobs_left && n_idle >= kRefill))) continue;
-                    const int col = (int)(job_turn_col >> 8), turn_a = (int)(int8_t)(job_turn_col & 0xffu);
+                    if (!(n_idle == kWave || (!exhausted && n_idle >= kRefill))) return false;
+                    const int col = (int)((job_turn_col >> 8) & 0xffu), turn_a = (int)(int8_t)(job_turn_col & 0xffu);
                     uint64_t *const st = s_rng + 2 * ((size_t)col * P + job_t);
                     if (__ballot(pending && status == 3) != 0ull) {  // rare: a draw rounded up to 1.0f; replay with the exact emulation, one playout at a time
                         if (lane == 0) {
@@ -669,6 +683,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                     }
                     if (pending && (status == 1 || status == 2)) {
                         st[0] = ((uint64_t)rg.s0h << 32) | rg.s0l; st[1] = ((uint64_t)rg.s1h << 32) | rg.s1l;
+                        const uint32_t n = (uint32_t)(__popc(me.lo) + __popc(me.hi) + __popc(other.lo) + __popc(other.hi)) - (job_turn_col >> 16);   // plies made
                         plies += n;
                         if (status == 1) {
                             const int winner = (n & 1u) ? turn_a : -turn_a;   // the side that made the last move
@@ -676,11 +691,17 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                         }
                     }
                     pending = false;
-                    if (!jobs_left) break;   // every lane is idle and there is nothing left to hand out
-                    // the idle lanes take the wavefront's next jobs in lane order
-                    const int mine = next + (int)__popcll(idle & ((1ull << lane) - 1ull));
-                    if (!active && mine < last) { take_job(mine); active = true; }
-                    next += n_idle;
+                    if (exhausted) return true;   // every lane is idle and there is nothing left to hand out
+                    // the idle lanes take the next jobs in lane order
+                    first = grab(n_idle);
+                    exhausted = first + n_idle >= n_jobs;
+                    const int mine = first + (int)__popcll(idle & ((1ull << lane) - 1ull));
+                    if (!active && mine < n_jobs) { take_job(mine, other, me); active = true; }
+                    return __ballot(active) == 0ull;   // (the counter had passed the end already)
+                };
+                for (;;) {
+                    if (iteration(a, b)) break;
+                    if (iteration(b, a)) break;
                 }
             }
             st_played += __popc(solo_played);

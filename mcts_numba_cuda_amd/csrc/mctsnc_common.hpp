@@ -43,6 +43,9 @@ __host__ __device__ inline double det_log(double x) { return detm_log(x); }
 // exact in float64 (two conversions and one fused multiply-add, all exact), the narrowing rounds once to nearest even
 // as the reference's float32 cast does, and the scaling by 2^-64 is exact.  Five instructions per draw.
 __device__ __forceinline__ float uniform_from_bits(uint32_t lo, uint32_t hi) {
+    // (hi is usually the upper half of a 64-bit sum; without this the compiler converts that 64-bit value shifted down
+    // instead, a longer sequence with an addition of zero that it does not fold)
+    asm("" : "+v"(hi));
     const double d = __builtin_fma((double)hi, 4294967296.0, (double)(lo & 0xfffff800u));
     return (float)d * 0x1p-64f;
 }
