@@ -161,6 +161,20 @@ def test_other_connect4_boards(m, n, variant):
         compare_with_oracle(e, o, board, fills, turn, steps=250)
 
 
+@pytest.mark.parametrize("m,n", [(4, 5), (7, 8), (8, 7), (13, 4)])
+def test_other_connect4_boards_one_workgroup_per_tree(m, n, monkeypatch):
+    """The same boards' extremes with every tree searched by a single workgroup (the pool of playout jobs)."""
+    monkeypatch.setenv("MCTSNC_SOLO_TREES", "1")
+    rng = np.random.default_rng(100 * m + n + 1)
+    params = dict(n_trees=3, n_playouts=64, variant="acp_prodigal", device_memory=0.25, ucb_c=2.0, seed=9)
+    e = make_engine(params, board_shape=(m, n), extra=n, actions=n)
+    from oracle.oracle import Oracle
+    o = Oracle("c4", (m, n), n, n, 3, 64, "acp_prodigal", ucb_c=2.0, seed=9, device_memory=0.25, threads=8)
+    for plies in (2, m * n // 2):
+        board, fills, turn = random_c4_root(rng, plies, m, n)
+        compare_with_oracle(e, o, board, fills, turn, steps=250)
+
+
 @pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
 def test_small_playout_counts_and_exploration_constants(variant):
     """n_playouts below a wavefront (down to one playout per node), ucb_c = 0 (pure exploitation: ties everywhere) and
