@@ -606,7 +606,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
             __syncthreads();
             solo_played = s_pool_mask;
             {
-                const int n_jobs = s_pool_n * P;
+                const int n_jobs = __builtin_amdgcn_readfirstlane(s_pool_n) * P;   // (the same in every lane: kept in a scalar register)
                 const int pshift = 31 - __clz(P);   // P is a power of two
                 const int m = geo.m, H = geo.H;
                 BB a = {0, 0}, b = {0, 0};
@@ -632,8 +632,10 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 };
                 int first = grab(kWave);
                 bool exhausted = first + kWave >= n_jobs;   // the counter has passed the end: nothing more to take
-                bool active = first + lane < n_jobs;
-                if (active) take_job(first + lane, a, b);
+                // per lane: 0 = its playout is running; 1 = it ended with a win of the mover, 2 = with the board full, 3 = with
+                // a draw that equalled the count (to be replayed), all three not booked yet; 4 = no playout
+                int state = first + lane < n_jobs ? 0 : 4;
+                if (state == 0) take_job(first + lane, a, b);
                 // Finished lanes are served in batches: booking a result and fetching the next job costs about 40
                 // instructions for the whole wavefront whenever it runs, and with 64 lanes some lane finishes in almost
                 // every iteration; so it runs only once kRefill lanes are waiting (or all are), and not at all once the
@@ -641,21 +643,16 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                 // 4 / 8 / 16: one search of 512 trees x 256 playouts 13.8 / 14.4 / 15.0 / 15.1, 768 searches of 4 trees
                 // 26.4 / 25.7 / 26.8 / 28.0.
                 constexpr int kRefill = 16;
-                int status = 0;        // of the lane's job: 0 = running, 1 = mover won, 2 = board full, 3 = ordinal == count
-                bool pending = false;  // the job has ended and its result is not booked yet
                 // One iteration for the side whose stones are `me`, the same side in every lane (a job taken now starts
                 // with the next iteration, so its side to move goes where `other` is); true when the wavefront is done.
                 auto iteration = [&](BB &me, BB &other) -> bool {
-                    if (active) {
-                        status = Game::ply(m, H, me, fills, list, count, rg);
-                        if (status != 0) { active = false; pending = true; }
-                    }
-                    const unsigned long long idle = __ballot(!active);
-                    const int n_idle = (int)__popcll(idle);
-                    if (!(n_idle == kWave || (!exhausted && n_idle >= kRefill))) return false;
+                    if (state == 0) state = Game::ply(m, H, me, fills, list, count, rg);
+                    const unsigned long long idle = __ballot(state != 0);
+                    const int n_idle = __builtin_popcountll(idle);
+                    if (!(idle == ~0ull || (!exhausted && (uint32_t)n_idle >= (uint32_t)kRefill))) return false;
                     const int col = (int)((job_turn_col >> 8) & 0xffu), turn_a = (int)(int8_t)(job_turn_col & 0xffu);
                     uint64_t *const st = s_rng + 2 * ((size_t)col * P + job_t);
-                    if (__ballot(pending && status == 3) != 0ull) {  // rare: a draw rounded up to 1.0f; replay with the exact emulation, one playout at a time
+                    if (__ballot(state == 3) != 0ull) {  // rare: a draw rounded up to 1.0f; replay with the exact emulation, one playout at a time
                         if (lane == 0) {
                             uint32_t spins = 0;
                             while (atomicCAS(&s_lock, 0u, 1u) != 0u) {
@@ -664,7 +661,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                             }
                         }
                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-                        unsigned long long redo = __ballot(pending && status == 3);
+                        unsigned long long redo = __ballot(state == 3);
                         while (redo) {
                             const int l = (int)__ffsll((long long)redo) - 1;
                             redo &= redo - 1ull;
@@ -681,23 +678,23 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                         if (lane == 0) atomicExch(&s_lock, 0u);
                     }
-                    if (pending && (status == 1 || status == 2)) {
+                    if (state == 1 || state == 2) {
                         st[0] = ((uint64_t)rg.s0h << 32) | rg.s0l; st[1] = ((uint64_t)rg.s1h << 32) | rg.s1l;
                         const uint32_t n = (uint32_t)(__popc(me.lo) + __popc(me.hi) + __popc(other.lo) + __popc(other.hi)) - (job_turn_col >> 16);   // plies made
                         plies += n;
-                        if (status == 1) {
+                        if (state == 1) {
                             const int winner = (n & 1u) ? turn_a : -turn_a;   // the side that made the last move
                             atomicAdd(&s_cnt[col][winner == 1 ? 1 : 0], 1);
                         }
                     }
-                    pending = false;
+                    state = state != 0 ? 4 : 0;
                     if (exhausted) return true;   // every lane is idle and there is nothing left to hand out
                     // the idle lanes take the next jobs in lane order
                     first = grab(n_idle);
                     exhausted = first + n_idle >= n_jobs;
                     const int mine = first + (int)__popcll(idle & ((1ull << lane) - 1ull));
-                    if (!active && mine < n_jobs) { take_job(mine, other, me); active = true; }
-                    return __ballot(active) == 0ull;   // (the counter had passed the end already)
+                    if (state != 0 && mine < n_jobs) { take_job(mine, other, me); state = 0; }
+                    return __ballot(state == 0) == 0ull;   // (the counter had passed the end already)
                 };
                 for (;;) {
                     if (iteration(a, b)) break;
