@@ -474,24 +474,24 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     // no lane idle while others finish their playouts and keeps every CU busy from the queue; fewer trees: a team of one
     // workgroup per column, whose step is several times shorter.  Measured switch-over (searches of 4 trees x 256
     // playouts, 5000 steps, one workgroup per tree against teams).  A batch of searches of different roots, where the
-    // longest search sets the pace, G playouts/s in one pass: 192 searches 12.7 against 13.7, 256 searches 14.8 against
-    // 14.6, 320 searches 16.3 against 14.6, 384 searches 20.5 against 14.9, 512 searches 23.9 against 15.1, 768 searches 28
-    // against 15: from 1024 trees on.  One search, whose trees all take about as long, ms per search: a workgroup's step
-    // costs the same for any number of trees up to one per CU (175) and again up to two per CU (269), a team's search
-    // grows with the number of trees (192 trees 153, 256 trees 192, 320 trees 230, 384 trees 255, 448 trees 310, 512
-    // trees 340): from 1.6 trees per CU on, and between 0.9 and 1.  MCTSNC_SOLO_TREES sets one threshold for both
-    // (0 = never).
+    // longest search sets the pace, G playouts/s in one pass: 160 searches 12.6 against 13.2, 192 searches 14.0 against
+    // 13.7, 224 searches 13.9 against 14.0, 256 searches 15.1 against 14.2, 320 searches 17.5 against 14.7, 512 searches 26
+    // against 15, 768 searches 31 against 15: from 1024 trees on.  One search, whose trees all take about as long, ms per
+    // search: a workgroup's step costs the same for any number of trees up to one per CU (155) and again up to two per
+    // CU (250), a team's search grows with the number of trees (192 trees 153, 256 trees 191, 320 trees 230, 384 trees 255,
+    // 448 trees 309, 512 trees 339): from 1.4 trees per CU on, and between 0.8 and 1.  MCTSNC_SOLO_TREES sets one
+    // threshold for both (0 = never).
     int cus_now = 0;
     HIP_TRY(hipDeviceGetAttribute(&cus_now, hipDeviceAttributeMultiprocessorCount, c.device));
-    bool solo = e0->acp && (n > 1 ? n_refs >= 1024 : (10 * n_refs >= 16 * cus_now || (10 * n_refs >= 9 * cus_now && n_refs <= cus_now)));
+    bool solo = e0->acp && (n > 1 ? n_refs >= 1024 : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) { const int from = atoi(v); solo = e0->acp && from > 0 && n_refs >= from; }
     if (solo) {
         args.G = 1;
         // The workgroup plays all playouts of a step as one pool of jobs (lanes take further jobs as theirs end) with as many
         // lanes as one node has playouts, twice as many while there are no more than two trees per CU (64 to 512).  Fewer
         // lanes make better use of each but lengthen the step of the slowest tree, which a pass waits for; four workgroups
-        // per CU stay resident (LDS).  Measured, G playouts/s: 768 searches of 4 trees, 256 threads 25.7, 512 threads 21.6, 128
-        // threads 20.7; one search with 512 trees (two per CU), 512 threads 16.3, 256 threads 14.0, 1024 threads 11.1.
+        // per CU stay resident (LDS).  Measured, G playouts/s: 768 searches of 4 trees, 128 threads 23.7, 192 threads 27.7, 256
+        // threads 28.5, 384 threads 25.2, 512 threads 27.1; one search with 512 trees (two per CU), 512 threads 17.6, 256 threads 15.8, 1024 threads 11.1 (an earlier form).
         int threads = ((c.n_playouts + 63) / 64) * 64;
         if (n_refs <= 2 * cus_now) threads *= 2;
         threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
