@@ -103,8 +103,9 @@ class MCTSNC:
         self.device = int(device)
         self._engine = None
         self.max_tree_size = None
-        self.actions_info = None
-        self.performance_info = None
+        self._actions_info = None
+        self._performance_info = None
+        self._result = None
         self.best_action = self.best_win_flag = self.best_n = self.best_n_wins = self.best_q = None
         self.steps = 0
         self.time_total = self.time_loop = self.time_reduce_over_trees = self.time_reduce_over_actions = 0.0
@@ -239,7 +240,6 @@ class MCTSNC:
         return self.best_action
 
     def _absorb_result(self, res, root_turn):
-        A = self.state_max_actions
         self._result = res
         self._root_turn = root_turn
         self.steps = int(res.steps)
@@ -256,16 +256,50 @@ class MCTSNC:
         self.time_select, self.time_expand = res.time_select, res.time_expand
         self.time_playout, self.time_backup = res.time_playout, res.time_backup
         self.time_exchange = res.time_exchange
-        self._root_actions_expanded = np.array(res.root_actions_expanded[:A + 2], dtype=np.int16)
-        self._root_ns = np.array(res.root_ns[:A], dtype=np.int64)
-        self._actions_ns = np.array(res.actions_ns[:A], dtype=np.int64)
-        self._actions_ns_wins = np.array(res.actions_ns_wins[:A], dtype=np.int64)
-        self._actions_win_flags = np.array(res.actions_win_flags[:A], dtype=bool)
-        if "thrifty" in self.variant:
-            self._make_actions_info_thrifty()
-        else:
-            self._make_actions_info_prodigal()
-        self._make_performance_info()
+        # the root tables and the two dictionaries are built when first read (a pass over hundreds of engines would
+        # otherwise spend milliseconds on dictionaries nobody looks at)
+        self._tables = None
+        self._actions_info = None
+        self._performance_info = None
+
+    def _decode_tables(self):
+        if self._tables is None:
+            res, A = self._result, self.state_max_actions
+            self._tables = (np.array(res.root_actions_expanded[:A + 2], dtype=np.int16), np.array(res.root_ns[:A], dtype=np.int64),
+                            np.array(res.actions_ns[:A], dtype=np.int64), np.array(res.actions_ns_wins[:A], dtype=np.int64),
+                            np.array(res.actions_win_flags[:A], dtype=bool))
+        return self._tables
+
+    _root_actions_expanded = property(lambda self: self._decode_tables()[0])
+    _root_ns = property(lambda self: self._decode_tables()[1])
+    _actions_ns = property(lambda self: self._decode_tables()[2])
+    _actions_ns_wins = property(lambda self: self._decode_tables()[3])
+    _actions_win_flags = property(lambda self: self._decode_tables()[4])
+
+    @property
+    def actions_info(self):
+        """Root action table of the last search (src/mctsnc.py:496-563); None before the first."""
+        if self._actions_info is None and self._result is not None:
+            if "thrifty" in self.variant:
+                self._make_actions_info_thrifty()
+            else:
+                self._make_actions_info_prodigal()
+        return self._actions_info
+
+    @actions_info.setter
+    def actions_info(self, value):
+        self._actions_info = value
+
+    @property
+    def performance_info(self):
+        """Performance dictionary of the last search (src/mctsnc.py:448-494); None before the first."""
+        if self._performance_info is None and self._result is not None:
+            self._make_performance_info()
+        return self._performance_info
+
+    @performance_info.setter
+    def performance_info(self, value):
+        self._performance_info = value
 
     def _entry(self, i, a):
         entry = {}
