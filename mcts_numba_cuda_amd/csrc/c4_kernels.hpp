@@ -367,6 +367,12 @@ __global__ void reset_kernel(const TreeRef *refs, int n_refs, const uint64_t *ro
     h->t_select = 0; h->t_expand = 0; h->t_playout = 0; h->t_backup = 0; h->t_exchange = 0;
 }
 
+// Plies played in every tree since its reset, for the host to order a pass by what its searches cost.
+__global__ void plies_kernel(const TreeRef *refs, int n_refs, unsigned long long *out) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < n_refs) out[r] = refs[r].hdr->plies;
+}
+
 struct LeafInfo {
     uint64_t bb_pos, bb_neg;
     int32_t node, depth, turn, flags, outcome;
