@@ -481,20 +481,24 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
     dim3 block(e0->block);
-    // All-children playouts with many trees at once: one workgroup per tree (see search_body), which does no work twice, lets
-    // no lane idle while others finish their playouts and keeps every CU busy from the queue; fewer trees: a team of one
-    // workgroup per column, whose step is several times shorter.  Measured switch-over (searches of 4 trees x 256
-    // playouts, 5000 steps, one workgroup per tree against teams).  A batch of searches of different roots, where the
-    // longest search sets the pace, G playouts/s in one pass: 160 searches 12.6 against 13.2, 192 searches 14.0 against
-    // 13.7, 224 searches 13.9 against 14.0, 256 searches 15.1 against 14.2, 320 searches 17.5 against 14.7, 512 searches 26
-    // against 15, 768 searches 31 against 15: from 1024 trees on.  One search, whose trees all take about as long, ms per
-    // search: a workgroup's step costs the same for any number of trees up to one per CU (155) and again up to two per
-    // CU (250), a team's search grows with the number of trees (192 trees 153, 256 trees 191, 320 trees 230, 384 trees 255,
-    // 448 trees 309, 512 trees 339): from 1.4 trees per CU on, and between 0.8 and 1.  MCTSNC_SOLO_TREES sets one
-    // threshold for both (0 = never).
+    // All-children playouts, three forms of the same step (identical results).  A team of one workgroup per column with one
+    // lane per playout has the shortest step and is what one search or a few dozen run on.  One workgroup per tree (see
+    // search_body) does no work twice, lets no lane idle while others finish their playouts and keeps every CU busy from
+    // the queue: the form for many hundreds of trees.  Between the two, teams whose workgroups play their child's playouts
+    // as a pool of jobs on half as many lanes: half the wavefronts per tree, so twice as many trees resident, and no
+    // idle lanes, at a step 1.4 times as long.  Measured (searches of 4 trees x 256 playouts, 5000 steps, different
+    // roots, G playouts/s in one pass, teams / teams with pools / one workgroup per tree): 64 searches 12.5 / 9.2 / 6.7,
+    // 96 searches 14.4 / 13.8 / 9.3, 112 searches 14.4 / 14.7 / 9.7, 128 searches 14.6 / 17.0 / 10.7, 192 searches
+    // 15.1 / 19.8 / 14.3, 256 searches 15.2 / 21.1 / 15.5, 304 searches 15.3 / 21.0 / 21.0, 320 searches 15.3 / 21.4 / 22.9,
+    // 384 searches 15.5 / 21.4 / 26.1, 512 searches 15.5 / 21.9 / 37.9, 768 searches 15 / - / 40.5: pools from 1.75 trees
+    // per CU on, one workgroup per tree from 4.75.  One search, whose trees all take about as long, ms per search: a
+    // single workgroup's step costs the same for any number of trees up to one per CU (155) and again up to two per CU
+    // (250), a team's search grows with the number of trees (192 trees 153, 256 trees 191, 320 trees 230, 384 trees 255,
+    // 448 trees 309, 512 trees 339): one workgroup per tree from 1.4 trees per CU on, and between 0.8 and 1.
+    // MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
     int cus_now = 0;
     HIP_TRY(hipDeviceGetAttribute(&cus_now, hipDeviceAttributeMultiprocessorCount, c.device));
-    bool solo = e0->acp && (n > 1 ? n_refs >= 1024 : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
+    bool solo = e0->acp && (n > 1 ? 4 * n_refs >= 19 * cus_now : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) { const int from = atoi(v); solo = e0->acp && from > 0 && n_refs >= from; }
     if (solo) {
         args.G = 1;
@@ -509,8 +513,21 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 1024 && t % 64 == 0) threads = t; }   // for experiments
         block = dim3(threads);
     }
-    const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n);
+    // Teams with pools (see above): half as many lanes as playouts (with a quarter the step gets too long: 192 searches
+    // 17.5 against 19.7, 288 searches 15.5 against 21.1; with three quarters the gain is gone).  MCTSNC_TEAM_POOL=0/1
+    // forces the form off/on, MCTSNC_TEAM_POOL_THREADS sets the lanes.
+    bool team_pool = e0->acp && !solo && n > 1 && c.n_playouts >= 128 && 4 * n_refs >= 7 * cus_now;
+    if (const char *v = getenv("MCTSNC_TEAM_POOL")) team_pool = e0->acp && !solo && atoi(v) != 0;
+    if (team_pool) {
+        int threads = ((c.n_playouts / 2 + 63) / 64) * 64;
+        if (threads < 64) threads = 64;
+        if (const char *v = getenv("MCTSNC_TEAM_POOL_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 512 && t % 64 == 0) threads = t; }
+        block = dim3(threads);
+    }
+    const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts)
+                            : (team_pool ? c4::team_pool_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n));
     const auto solo_kernel = block.x > 512 ? c4::search_kernel_solo_wide : c4::search_kernel_solo;
+    const auto team_kernel = team_pool ? c4::search_kernel_team_pool : c4::search_kernel<true>;
     if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(solo_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
     // all its workgroups must be resident together: a batch with more trees than resident sets starts one tree per
@@ -521,7 +538,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
         if (solo) HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, solo_kernel, block.x, lds));
-        else HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, c4::search_kernel<true>, e0->block, lds));
+        else HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, team_kernel, block.x, lds));
         const int resident_sets = (int)((int64_t)per_cu * cus / (8 * args.G)) * 8;
         if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * args.G);
         if (sets > resident_sets) { sets = resident_sets; args.queue = e0->d_abort + 1; }
@@ -557,11 +574,11 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
                 HIP_TRY(hipGetLastError());
             } else {
                 if (plain_launch) {
-                    hipLaunchKernelGGL(c4::search_kernel<true>, grid, block, lds, stream, args);
+                    hipLaunchKernelGGL(team_kernel, grid, block, lds, stream, args);
                     HIP_TRY(hipGetLastError());
                 } else {
                     void *kargs[] = {&args};
-                    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(c4::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
+                    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(team_kernel), grid, block, kargs, (unsigned)lds, stream));
                 }
             }
         } else {

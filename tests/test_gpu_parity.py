@@ -258,6 +258,51 @@ def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypat
             np.testing.assert_array_equal(eb.read_array("trees", ti), es.read_array("trees", ti))
 
 
+@pytest.mark.parametrize("threads", ["", "64", "192"], ids=["half-the-playouts", "one-wavefront", "three-wavefronts"])
+@pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
+def test_teams_with_playout_pools_give_the_same_trees(variant, threads, monkeypatch):
+    """A pass of a few hundred trees runs teams whose workgroups play their child's playouts as a pool of jobs on fewer
+    lanes than playouts (MCTSNC_TEAM_POOL forces the form on or off, MCTSNC_TEAM_POOL_THREADS sets the lanes).  Forced here
+    for small searches: full state against the oracle over two runs, a pool that fills up, late-game roots, a playout
+    count smaller than a wavefront, and a batch through the queue against single runs without pools."""
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    from oracle.oracle import Oracle
+    monkeypatch.setenv("MCTSNC_TEAM_POOL", "1")
+    monkeypatch.setenv("MCTSNC_SOLO_TREES", "0")
+    if threads:
+        monkeypatch.setenv("MCTSNC_TEAM_POOL_THREADS", threads)
+    rng = np.random.default_rng(43)
+    for T, P, steps in ((3, 64, 300), (4, 256, 150), (2, 16, 200)):
+        params = dict(n_trees=T, n_playouts=P, variant=variant, device_memory=0.25, ucb_c=2.0, seed=7)
+        e = make_engine(params)
+        o = Oracle("c4", (6, 7), 7, 7, T, P, variant, ucb_c=2.0, seed=7, device_memory=0.25, threads=8)
+        for plies in (8, 24):
+            board, fills, turn = random_c4_root(rng, plies)
+            compare_with_oracle(e, o, board, fills, turn, steps=steps)
+    e = MCTSNC((6, 7), 7, 7, search_time_limit=np.inf, search_steps_limit=np.inf, n_trees=2, n_playouts=64, variant=variant,
+               device_memory=2.0, ucb_c=2.0, seed=4, verbose_info=False)
+    e.device_memory = float(2 * 95 * 50 + 2 * 8300)  # room for about 50 nodes per tree
+    e.init_device_side_arrays()
+    o = Oracle("c4", (6, 7), 7, 7, 2, 64, variant, ucb_c=2.0, seed=4, max_tree_size_override=e.max_tree_size, threads=4)
+    for plies in (5, 30):
+        board, fills, turn = random_c4_root(rng, plies)
+        compare_with_oracle(e, o, board, fills, turn, steps=200)
+    params = dict(n_trees=4, n_playouts=128, variant=variant, device_memory=0.1, ucb_c=2.0, seed=11)
+    roots = [random_c4_root(rng, int(rng.integers(4, 24))) for _ in range(96)]
+    batch = [make_engine(params) for _ in roots]
+    run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=300)
+    monkeypatch.setenv("MCTSNC_TEAM_POOL", "0")
+    es = make_engine(params)
+    for k in range(0, len(roots), 7):
+        eb, r = batch[k], roots[k]
+        es.reseed()
+        es.run(r[0], r[1], r[2], forced_search_steps_limit=300)
+        assert eb.actions_info == es.actions_info
+        for ti in range(4):
+            np.testing.assert_array_equal(eb.read_array("ns", ti), es.read_array("ns", ti))
+            np.testing.assert_array_equal(eb.read_array("trees", ti), es.read_array("trees", ti))
+
+
 @pytest.mark.parametrize("variant", ["ocp_thrifty", "ocp_prodigal", "acp_thrifty", "acp_prodigal"])
 def test_nearly_full_boards(variant):
     """Roots with one to four empty cells on both games (trees of a handful of nodes, every playout a few plies, draws
