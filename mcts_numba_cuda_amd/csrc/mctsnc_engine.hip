@@ -516,7 +516,9 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     // Teams with pools (see above): half as many lanes as playouts (with a quarter the step gets too long: 192 searches
     // 17.5 against 19.7, 288 searches 15.5 against 21.1; with three quarters the gain is gone).  MCTSNC_TEAM_POOL=0/1
     // forces the form off/on, MCTSNC_TEAM_POOL_THREADS sets the lanes.
-    bool team_pool = e0->acp && !solo && n > 1 && c.n_playouts >= 128 && 4 * n_refs >= 7 * cus_now;
+    // One search of more trees than CUs, below the point where one workgroup per tree takes over: 320 trees 217 ms against
+    // 231 for plain teams (256 trees 186 against 192, 192 trees 152 against 152, 128 trees 122 against 114).
+    bool team_pool = e0->acp && !solo && c.n_playouts >= 128 && (n > 1 ? 4 * n_refs >= 7 * cus_now : n_refs > cus_now);
     if (const char *v = getenv("MCTSNC_TEAM_POOL")) team_pool = e0->acp && !solo && atoi(v) != 0;
     if (team_pool) {
         int threads = ((c.n_playouts / 2 + 63) / 64) * 64;
