@@ -146,6 +146,20 @@ def test_widest_search_512_trees(variant):
         compare_with_oracle(e, o, board, fills, turn, steps=40)
 
 
+@pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
+def test_one_search_of_slightly_more_trees_than_cus(variant):
+    """288 trees x 128 playouts: between one and 1.4 trees per CU a single all-children search runs on teams whose
+    workgroups play their playouts as a pool of jobs (64 lanes for 128 playouts here)."""
+    rng = np.random.default_rng(78)
+    params = dict(n_trees=288, n_playouts=128, variant=variant, device_memory=1.0, ucb_c=2.0, seed=5)
+    e = make_engine(params)
+    from oracle.oracle import Oracle
+    o = Oracle("c4", (6, 7), 7, 7, 288, 128, variant, ucb_c=2.0, seed=5, device_memory=1.0, threads=8)
+    for plies in (12, 2):
+        board, fills, turn = random_c4_root(rng, plies)
+        compare_with_oracle(e, o, board, fills, turn, steps=30)
+
+
 @pytest.mark.parametrize("m,n", [(4, 5), (5, 6), (8, 7), (7, 8), (6, 8), (12, 4), (13, 4), (10, 5)])
 @pytest.mark.parametrize("variant", ["ocp_thrifty", "acp_prodigal"])
 def test_other_connect4_boards(m, n, variant):
