@@ -503,12 +503,13 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     if (solo) {
         args.G = 1;
         // The workgroup plays all playouts of a step as one pool of jobs (lanes take further jobs as theirs end) with as many
-        // lanes as one node has playouts, twice as many while there are no more than two trees per CU (64 to 512).  Fewer
+        // lanes as one node has playouts, twice as many while there are no more than six trees per CU (64 to 512).  Fewer
         // lanes make better use of each but lengthen the step of the slowest tree, which a pass waits for; four workgroups
-        // per CU stay resident (LDS).  Measured, G playouts/s: 768 searches of 4 trees, 128 threads 23.7, 192 threads 27.7, 256
-        // threads 28.5, 384 threads 25.2, 512 threads 27.1; one search with 512 trees (two per CU), 512 threads 17.6, 256 threads 15.8, 1024 threads 11.1 (an earlier form).
+        // of 256 threads per CU stay resident (LDS), two of 512 (registers).  Measured, G playouts/s, 256 / 512 threads:
+        // 320 searches of 4 trees 23.0 / 24.8, 384 searches 26.2 / 28.3, 448 searches 31.1 / 28.9, 512 searches 37.8 / 31.8,
+        // 768 searches 40.6 / 32.2 (192 threads 33.7, 384 threads 30.3); one search with 512 trees (two per CU) 15.8 / 17.6.
         int threads = ((c.n_playouts + 63) / 64) * 64;
-        if (n_refs <= 2 * cus_now) threads *= 2;
+        if (n_refs <= 6 * cus_now) threads *= 2;
         threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
         if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 1024 && t % 64 == 0) threads = t; }   // for experiments
         block = dim3(threads);
