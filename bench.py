@@ -458,7 +458,7 @@ def bench_c4_many(args):
            "roofline": {"bound": "hbm", "achieved": abytes / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": abytes / dev / 1e9 / HBM_PEAK_GBS,
                         "traffic": (prof or {}).get("traffic_bytes_per_launch") if n == (prof or {}).get("searches") else None,
-                        "kernel": "mctsnc::c4::search_kernel_solo (batches of 1216 trees or more), mctsnc::c4::search_kernel<true> below",
+                        "kernel": "mctsnc::c4::search_kernel_solo (batches of 896 trees or more), mctsnc::c4::search_kernel<true> below",
                         "algorithmic_bytes_per_launch": abytes, "avg_launch_ms": dev * 1e3},
            "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_pass") if n == (prof or {}).get("searches") else None, dev, prof or {},
                                           f"one pass over {n} searches"),

@@ -490,15 +490,16 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     // roots, G playouts/s in one pass, teams / teams with pools / one workgroup per tree): 64 searches 12.5 / 9.2 / 6.7,
     // 96 searches 14.4 / 13.8 / 9.3, 112 searches 14.4 / 14.7 / 9.7, 128 searches 14.6 / 17.0 / 10.7, 192 searches
     // 15.1 / 19.8 / 14.3, 256 searches 15.2 / 21.1 / 15.5, 304 searches 15.3 / 21.0 / 21.0, 320 searches 15.3 / 21.4 / 22.9,
-    // 384 searches 15.5 / 21.4 / 26.1, 512 searches 15.5 / 21.9 / 37.9, 768 searches 15 / - / 40.5: pools from 1.75 trees
-    // per CU on, one workgroup per tree from 4.75.  One search, whose trees all take about as long, ms per search: a
+    // 384 searches 15.5 / 21.4 / 26.1, 512 searches 15.5 / 21.9 / 37.9, 768 searches 15 / - / 40.5; with 512 instead of 256
+    // threads (see below) one workgroup per tree reaches 16.8 at 192 searches, 20.9 at 224, 25.9 at 256, 21.5 at 288, 22.7
+    // at 304, 28.5 at 384: pools from 1.75 trees per CU on, one workgroup per tree from 3.5.  One search, whose trees all take about as long, ms per search: a
     // single workgroup's step costs the same for any number of trees up to one per CU (155) and again up to two per CU
     // (250), a team's search grows with the number of trees (192 trees 153, 256 trees 191, 320 trees 230, 384 trees 255,
     // 448 trees 309, 512 trees 339): one workgroup per tree from 1.4 trees per CU on, and between 0.8 and 1.
     // MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
     int cus_now = 0;
     HIP_TRY(hipDeviceGetAttribute(&cus_now, hipDeviceAttributeMultiprocessorCount, c.device));
-    bool solo = e0->acp && (n > 1 ? 4 * n_refs >= 19 * cus_now : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
+    bool solo = e0->acp && (n > 1 ? 2 * n_refs >= 7 * cus_now : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
     if (const char *v = getenv("MCTSNC_SOLO_TREES")) { const int from = atoi(v); solo = e0->acp && from > 0 && n_refs >= from; }
     if (solo) {
         args.G = 1;
