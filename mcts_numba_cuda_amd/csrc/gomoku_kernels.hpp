@@ -98,8 +98,7 @@ __device__ __forceinline__ bool bb_test(const uint32_t *bb, int cell) { return (
 
 // compute_outcome_gomoku (src/mctsnc_game_mechanics.py:220-281) for the stone just placed at `cell` by `token`'s
 // owner, on bitboards: counts up to five stones on each side in the four directions; exactly four neighbours win.
-__device__ inline bool five_through(const uint32_t *mine, int m, int n, int cell) {
-    const int i = cell / n, j = cell - i * n;
+__device__ inline bool five_through(const uint32_t *mine, int m, int n, int i, int j) {
     const int DI[4] = {1, 0, 1, 1}, DJ[4] = {0, 1, -1, 1};
     for (int d = 0; d < 4; d++) {
         int total = 0;
@@ -198,13 +197,14 @@ __device__ __forceinline__ uint32_t exact_five_starts(uint32_t packed) {
 // The reference's plugin functions (src/mctsnc_game_mechanics.py:56-87, Gomoku bodies :181-280) map onto it like this:
 // is_action_legal and legal_actions_playout (cell empty; row-major list, swap-remove) and take_action[_playout] (place
 // the stone) are the skeleton's own, being the same for every such game; compute_outcome is the game's:
-//   wins_through      at node creation: does the stone just placed at `cell` complete a winning line of `mine`
+//   wins_through      at node creation: does a stone placed at (i, j) complete a winning line with the stones `mine`
+//                     (the mover's stones; only the neighbours of (i, j) are looked at, the cell itself is not)
 //   winning_starts    in a playout: the same test on two 16-bit line words packed in one dword (bit s set = a winning run
 //                     starts at s), and reach(): the starts whose run covers position p of a line
 //   exact_outcome     the byte-array form used when a playout is replayed exactly
 // ------------------------------------------------------------------------------------------------------------------------
 struct Gomoku {
-    static __device__ __forceinline__ bool wins_through(const uint32_t *mine, int m, int n, int cell) { return five_through(mine, m, n, cell); }
+    static __device__ __forceinline__ bool wins_through(const uint32_t *mine, int m, int n, int i, int j) { return five_through(mine, m, n, i, j); }
     static __device__ __forceinline__ uint32_t winning_starts(uint32_t packed) { return exact_five_starts(packed); }
     static __device__ __forceinline__ uint32_t reach(uint32_t p) { return (0x1fu << p) >> 4; }   // starts of a run of five through position p
     static __device__ __forceinline__ int exact_outcome(ExactScratch &s, int m, int n, int turn, int last_action) {
@@ -276,6 +276,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     __shared__ uint32_t s_bb[16];             // board of the selected node: [0..7] +1 stones, [8..15] -1 stones
     __shared__ uint32_t s_cbb[16];            // board of the child being played out
     __shared__ int16_t s_actions[kMaxCells];  // ordinal -> action of the selected node's expandable children
+    __shared__ int8_t s_out[kMaxCells];       // ordinal -> outcome of the child just created (2: the game goes on)
     __shared__ uint32_t s_tmpl[kMaxCells / 4];  // legal list template of the child being played out (bytes)
     __shared__ uint32_t s_ltmpl[kMaxLines];     // line words of both players (low / high half)
     __shared__ int32_t s_red[4][2];
@@ -361,23 +362,23 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
         if (mode == kModeExpand) {
             for (int j = (ACP ? g : 0) + (ACP ? G : 1) * tid; j < k_exp; j += (ACP ? G : 1) * nthreads) {
                 const int a = s_actions[j];
+                // every index below is a constant after unrolling: a record indexed at run time would live in scratch memory
+                const uint32_t a_word = (uint32_t)a >> 5, a_bit = 1u << (a & 31);
                 Node nd;
                 nd.child_base = -1; nd.parent = leaf.node; nd.n_children = 0; nd.best_child = -1; nd.depth = (int16_t)(L + 1); nd.turn = (int8_t)(-mover);
                 nd.pad0 = 0; nd.action = (int16_t)a; nd.pad1[0] = nd.pad1[1] = 0;
-                uint32_t mine[8];
+                int occ = 0;
+#pragma unroll
                 for (int w = 0; w < 8; w++) {
-                    nd.bb_pos[w] = s_bb[w]; nd.bb_neg[w] = s_bb[8 + w]; nd.pad2[w] = 0;
-                    mine[w] = (mover == 1) ? s_bb[w] : s_bb[8 + w];
+                    const uint32_t add = (uint32_t)w == a_word ? a_bit : 0u;
+                    nd.bb_pos[w] = s_bb[w] | (mover == 1 ? add : 0u); nd.bb_neg[w] = s_bb[8 + w] | (mover == 1 ? 0u : add); nd.pad2[w] = 0;
+                    occ += __popc(nd.bb_pos[w] | nd.bb_neg[w]);
                 }
-                mine[a >> 5] |= 1u << (a & 31);
-                if (mover == 1) nd.bb_pos[a >> 5] |= 1u << (a & 31); else nd.bb_neg[a >> 5] |= 1u << (a & 31);
+                const uint32_t ai = ((uint32_t)a * div_n) >> 16, aj = (uint32_t)a - ai * (uint32_t)n;
                 int outcome = 2;
-                if (Game::wins_through(mine, m, n, a)) outcome = mover;
-                else {
-                    int occ = 0;
-                    for (int w = 0; w < 8; w++) occ += __popc(nd.bb_pos[w] | nd.bb_neg[w]);
-                    if (occ == cells) outcome = 0;
-                }
+                if (Game::wins_through(mover == 1 ? s_bb : s_bb + 8, m, n, (int)ai, (int)aj)) outcome = mover;
+                else if (occ == cells) outcome = 0;
+                s_out[j] = (int8_t)outcome;
                 nd.outcome = (int8_t)outcome;
                 nd.flags = (uint8_t)(kLeaf | (outcome != 2 ? kTerminal : 0));
                 nodes[size + j] = nd;
@@ -409,15 +410,20 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             int pnode, last_action, pturn, paction;
             if (mode == kModeExpand) { pnode = size + j; last_action = s_actions[j]; pturn = -mover; paction = last_action; }
             else { pnode = leaf.node; last_action = -1; pturn = mover; paction = 0; }
-            const Node *pn = nodes + pnode;
             int job_neg = 0, job_pos = 0;
-            const int poutcome = (mode == kModeExpand) ? pn->outcome : 2;
+            const int poutcome = (mode == kModeExpand) ? s_out[j] : 2;   // this workgroup created the children it plays out
             if (poutcome != 2) {  // terminal child: stored outcome times P (src/mctsnc.py:1842-1846)
                 job_neg = poutcome == -1 ? P : 0; job_pos = poutcome == 1 ? P : 0;
             } else {
                 st_played++;
-                // templates: board, legal list in row-major order, line words of both players
-                if (tid < 16) s_cbb[tid] = (tid < 8) ? pn->bb_pos[tid] : pn->bb_neg[tid - 8];
+                // templates: board (the selected node's, plus the child's stone), legal list in row-major order, line words
+                // of both players
+                if (tid < 16) {
+                    uint32_t w = s_bb[tid];
+                    if (mode == kModeExpand && (tid >> 3) == (mover == 1 ? 0 : 1) && (tid & 7) == (last_action >> 5)) w |= 1u << (last_action & 31);
+                    s_cbb[tid] = w;
+                }
+                for (int ln = tid; ln < n_lines; ln += nthreads) s_ltmpl[ln] = 0;
                 __syncthreads();
                 if (wave == 0) {  // empty cells in row-major order as (row << 4 | column), compacted with ballots
                     uint8_t *tm = reinterpret_cast<uint8_t *>(s_tmpl);
@@ -431,23 +437,18 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     }
                     if (lane == 0) s_count = cnt;
                 }
-                for (int ln = tid; ln < n_lines; ln += nthreads) {
-                    uint32_t word = 0;
-                    for (int p = 0; p < 2; p++) {
-                        const uint32_t *bb = s_cbb + 8 * p;
-                        uint32_t v = 0;
-                        if (ln < m) { for (int jj = 0; jj < n; jj++) v |= (uint32_t)bb_test(bb, ln * n + jj) << jj; }
-                        else if (ln < m + n) { const int jj = ln - m; for (int ii = 0; ii < m; ii++) v |= (uint32_t)bb_test(bb, ii * n + jj) << ii; }
-                        else if (ln < m + n + (m + n - 1)) {
-                            const int d = ln - (m + n);  // d = i - j + (n - 1)
-                            for (int jj = 0; jj < n; jj++) { const int ii = d + jj - (n - 1); if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
-                        } else {
-                            const int e = ln - (m + n) - (m + n - 1);  // e = i + j
-                            for (int jj = 0; jj < n; jj++) { const int ii = e - jj; if (ii >= 0 && ii < m) v |= (uint32_t)bb_test(bb, ii * n + jj) << jj; }
-                        }
-                        word |= v << (16 * p);
+                // one thread per cell (the last wavefronts first: the first one makes the list): a stone sets its bit in
+                // the words of the four lines through it -- row i, column j, diagonal i - j, anti-diagonal i + j
+                for (int c = cells - 1 - tid; c >= 0; c -= nthreads) {
+                    const bool pos = bb_test(s_cbb, c), neg = bb_test(s_cbb + 8, c);
+                    if (pos | neg) {
+                        const uint32_t i = ((uint32_t)c * div_n) >> 16, jj = (uint32_t)c - i * (uint32_t)n, sh = neg ? 16u : 0u;
+                        const uint32_t bit_j = (1u << jj) << sh;
+                        atomicOr(&s_ltmpl[i], bit_j);
+                        atomicOr(&s_ltmpl[(uint32_t)m + jj], (1u << i) << sh);
+                        atomicOr(&s_ltmpl[(uint32_t)(m + n + n - 1) + i - jj], bit_j);
+                        atomicOr(&s_ltmpl[(uint32_t)(m + n + m + n - 1) + i + jj], bit_j);
                     }
-                    s_ltmpl[ln] = word;
                 }
                 __syncthreads();
                 const int count0 = s_count;
