@@ -96,23 +96,6 @@ struct SearchArgs {
 
 __device__ __forceinline__ bool bb_test(const uint32_t *bb, int cell) { return (bb[cell >> 5] >> (cell & 31)) & 1u; }
 
-// compute_outcome_gomoku (src/mctsnc_game_mechanics.py:220-281) for the stone just placed at `cell` by `token`'s
-// owner, on bitboards: counts up to five stones on each side in the four directions; exactly four neighbours win.
-__device__ inline bool five_through(const uint32_t *mine, int m, int n, int i, int j) {
-    const int DI[4] = {1, 0, 1, 1}, DJ[4] = {0, 1, -1, 1};
-    for (int d = 0; d < 4; d++) {
-        int total = 0;
-        for (int s = -1; s <= 1; s += 2)
-            for (int k = 1; k < 6; k++) {
-                const int ii = i + s * k * DI[d], jj = j + s * k * DJ[d];
-                if (ii < 0 || ii >= m || jj < 0 || jj >= n || !bb_test(mine, ii * n + jj)) break;
-                total++;
-            }
-        if (total == 4) return true;
-    }
-    return false;
-}
-
 // ---- exact emulation of one reference playout (used when a uniform draw rounded up to 1.0f) --------------------
 // The reference then reads one slot past its legal list (src/mctsnc.py:1882-1883): a stale entry, so a stone may be
 // overwritten and a list entry lost; when the list later runs empty while the board is not full, it is rebuilt from
@@ -197,14 +180,13 @@ __device__ __forceinline__ uint32_t exact_five_starts(uint32_t packed) {
 // The reference's plugin functions (src/mctsnc_game_mechanics.py:56-87, Gomoku bodies :181-280) map onto it like this:
 // is_action_legal and legal_actions_playout (cell empty; row-major list, swap-remove) and take_action[_playout] (place
 // the stone) are the skeleton's own, being the same for every such game; compute_outcome is the game's:
-//   wins_through      at node creation: does a stone placed at (i, j) complete a winning line with the stones `mine`
-//                     (the mover's stones; only the neighbours of (i, j) are looked at, the cell itself is not)
-//   winning_starts    in a playout: the same test on two 16-bit line words packed in one dword (bit s set = a winning run
-//                     starts at s), and reach(): the starts whose run covers position p of a line
+//   winning_starts    at node creation and in a playout: does the stone just placed complete a winning line
+//                     (src/mctsnc_game_mechanics.py:220-281: exactly four neighbours of its colour in a row with it), as a
+//                     test on two 16-bit line words packed in one dword (bit s set = a winning run starts at s),
+//                     and reach(): the starts whose run covers position p of a line
 //   exact_outcome     the byte-array form used when a playout is replayed exactly
 // ------------------------------------------------------------------------------------------------------------------------
 struct Gomoku {
-    static __device__ __forceinline__ bool wins_through(const uint32_t *mine, int m, int n, int i, int j) { return five_through(mine, m, n, i, j); }
     static __device__ __forceinline__ uint32_t winning_starts(uint32_t packed) { return exact_five_starts(packed); }
     static __device__ __forceinline__ uint32_t reach(uint32_t p) { return (0x1fu << p) >> 4; }   // starts of a run of five through position p
     static __device__ __forceinline__ int exact_outcome(ExactScratch &s, int m, int n, int turn, int last_action) {
@@ -278,7 +260,8 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     __shared__ int16_t s_actions[kMaxCells];  // ordinal -> action of the selected node's expandable children
     __shared__ int8_t s_out[kMaxCells];       // ordinal -> outcome of the child just created (2: the game goes on)
     __shared__ uint32_t s_tmpl[kMaxCells / 4];  // legal list template of the child being played out (bytes)
-    __shared__ uint32_t s_ltmpl[kMaxLines];     // line words of both players (low / high half)
+    __shared__ uint32_t s_ltmpl[kMaxLines];     // line words of both players (low / high half) of the child being played out
+    __shared__ uint32_t s_lleaf[kMaxLines];     // the same of the selected node
     __shared__ int32_t s_red[4][2];
     __shared__ unsigned long long s_lkey[kLevels];   // per level of a chunk of the backup's arg-max: best key,
     __shared__ double s_llog[kLevels];               // log of the node's visit count,
@@ -305,6 +288,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
 
     for (int step = 0; step < args.nsteps; step++) {
         if (timing) tk = wall_clock64();
+        for (int ln = tid; ln < n_lines; ln += nthreads) s_lleaf[ln] = 0;
         // ================= selection: follow the memoised best children =================
         if (wave == 0) {
             // one coalesced load of the 128-byte record per level (lane i: dword i), fields handed round with readlane
@@ -336,22 +320,30 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_select += t2 - tk; tk = t2; }
 
         // ================= expansion decision (src/mctsnc.py:1367-1681) =================
-        int mode, k_exp = 0;
+        int mode, k_exp = 0, empties = 0;
         if (leaf.flags & kTerminal) mode = kModeTerminal;
         else {
-            int empties = 0;
             for (int w = 0; w < 8; w++) empties += __popc(s_bb[w] | s_bb[8 + w]);
             empties = cells - empties;
             int room = S - size; if (room < 0) room = 0;
             k_exp = empties < room ? empties : room;
             mode = k_exp > 0 ? kModeExpand : kModeFull;
-            // ordinal -> action: the j-th empty cell in row-major order
+            // one thread per cell.  An empty cell: ordinal -> action, the j-th empty cell in row-major order (which is also
+            // the legal list of a playout from here).  A stone: its bit in the words of the four lines through it -- row i,
+            // column j, diagonal i - j, anti-diagonal i + j; low half: stones of +1, high half: stones of -1.
             for (int c = tid; c < cells; c += nthreads) {
-                const uint32_t occ_w = s_bb[c >> 5] | s_bb[8 + (c >> 5)];
+                const uint32_t neg_w = s_bb[8 + (c >> 5)], occ_w = s_bb[c >> 5] | neg_w;
                 if (!((occ_w >> (c & 31)) & 1u)) {
                     int rank = __popc(~occ_w & ((1u << (c & 31)) - 1u));
                     for (int w = 0; w < (c >> 5); w++) rank += 32 - __popc(s_bb[w] | s_bb[8 + w]);
                     s_actions[rank] = (int16_t)c;
+                } else {
+                    const uint32_t i = ((uint32_t)c * div_n) >> 16, jj = (uint32_t)c - i * (uint32_t)n, sh = ((neg_w >> (c & 31)) & 1u) << 4;
+                    const uint32_t bit_j = (1u << jj) << sh;
+                    atomicOr(&s_lleaf[i], bit_j);
+                    atomicOr(&s_lleaf[(uint32_t)m + jj], (1u << i) << sh);
+                    atomicOr(&s_lleaf[(uint32_t)(m + n + n - 1) + i - jj], bit_j);
+                    atomicOr(&s_lleaf[(uint32_t)(m + n + m + n - 1) + i + jj], bit_j);
                 }
             }
         }
@@ -374,9 +366,16 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     nd.bb_pos[w] = s_bb[w] | (mover == 1 ? add : 0u); nd.bb_neg[w] = s_bb[8 + w] | (mover == 1 ? 0u : add); nd.pad2[w] = 0;
                     occ += __popc(nd.bb_pos[w] | nd.bb_neg[w]);
                 }
+                // the mover's stones on the four lines through the new one, two lines to a dword as in the playouts
                 const uint32_t ai = ((uint32_t)a * div_n) >> 16, aj = (uint32_t)a - ai * (uint32_t)n;
+                const uint32_t sh = mover == 1 ? 0u : 16u, sel = mover == 1 ? 0x05040100u : 0x07060302u, bit_j = (1u << aj) << sh;
+                const uint32_t w_row = s_lleaf[ai] | bit_j, w_col = s_lleaf[(uint32_t)m + aj] | ((1u << ai) << sh);
+                const uint32_t w_dia = s_lleaf[(uint32_t)(m + n + n - 1) + ai - aj] | bit_j, w_ant = s_lleaf[(uint32_t)(m + n + m + n - 1) + ai + aj] | bit_j;
+                const uint32_t win_j = Game::reach(aj), win_i = Game::reach(ai);
+                const uint32_t hit = Game::winning_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
+                const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
                 int outcome = 2;
-                if (Game::wins_through(mover == 1 ? s_bb : s_bb + 8, m, n, (int)ai, (int)aj)) outcome = mover;
+                if ((hit | hit2) != 0) outcome = mover;
                 else if (occ == cells) outcome = 0;
                 s_out[j] = (int8_t)outcome;
                 nd.outcome = (int8_t)outcome;
@@ -416,39 +415,34 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 job_neg = poutcome == -1 ? P : 0; job_pos = poutcome == 1 ? P : 0;
             } else {
                 st_played++;
-                // templates: board (the selected node's, plus the child's stone), legal list in row-major order, line words
-                // of both players
+                // templates, all from the selected node's: board, line words and legal list, with the child's stone added
+                const bool with_stone = mode == kModeExpand;
                 if (tid < 16) {
                     uint32_t w = s_bb[tid];
-                    if (mode == kModeExpand && (tid >> 3) == (mover == 1 ? 0 : 1) && (tid & 7) == (last_action >> 5)) w |= 1u << (last_action & 31);
+                    if (with_stone && (tid >> 3) == (mover == 1 ? 0 : 1) && (tid & 7) == (last_action >> 5)) w |= 1u << (last_action & 31);
                     s_cbb[tid] = w;
                 }
-                for (int ln = tid; ln < n_lines; ln += nthreads) s_ltmpl[ln] = 0;
-                __syncthreads();
-                if (wave == 0) {  // empty cells in row-major order as (row << 4 | column), compacted with ballots
+                {
+                    const uint32_t la = with_stone ? (uint32_t)last_action : 0u;
+                    const uint32_t li = (la * div_n) >> 16, lj = la - li * (uint32_t)n, sh = mover == 1 ? 0u : 16u;
+                    for (int ln = tid; ln < n_lines; ln += nthreads) {
+                        uint32_t w = s_lleaf[ln];
+                        if (with_stone) {
+                            const uint32_t u = (uint32_t)ln;
+                            if (u == li || u == (uint32_t)(m + n + n - 1) + li - lj || u == (uint32_t)(m + n + m + n - 1) + li + lj) w |= (1u << lj) << sh;
+                            if (u == (uint32_t)m + lj) w |= (1u << li) << sh;
+                        }
+                        s_ltmpl[ln] = w;
+                    }
+                    // the list: the node's empty cells in row-major order as (row << 4 | column), without the child's own (ordinal j)
                     uint8_t *tm = reinterpret_cast<uint8_t *>(s_tmpl);
-                    int cnt = 0;
-                    for (int base = 0; base < cells; base += 64) {
-                        const int c = base + lane;
-                        const bool empty = c < cells && !bb_test(s_cbb, c) && !bb_test(s_cbb + 8, c);
-                        const unsigned long long mask = __ballot(empty);
-                        if (empty) { const uint32_t ci = ((uint32_t)c * div_n) >> 16; tm[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (uint8_t)((ci << 4) | ((uint32_t)c - ci * (uint32_t)n)); }
-                        cnt += __popcll(mask);
+                    const int cnt = empties - (with_stone ? 1 : 0);
+                    for (int k = tid; k < cnt; k += nthreads) {
+                        const uint32_t c = (uint32_t)s_actions[k + ((with_stone && k >= j) ? 1 : 0)];
+                        const uint32_t ci = (c * div_n) >> 16;
+                        tm[k] = (uint8_t)((ci << 4) | (c - ci * (uint32_t)n));
                     }
-                    if (lane == 0) s_count = cnt;
-                }
-                // one thread per cell (the last wavefronts first: the first one makes the list): a stone sets its bit in
-                // the words of the four lines through it -- row i, column j, diagonal i - j, anti-diagonal i + j
-                for (int c = cells - 1 - tid; c >= 0; c -= nthreads) {
-                    const bool pos = bb_test(s_cbb, c), neg = bb_test(s_cbb + 8, c);
-                    if (pos | neg) {
-                        const uint32_t i = ((uint32_t)c * div_n) >> 16, jj = (uint32_t)c - i * (uint32_t)n, sh = neg ? 16u : 0u;
-                        const uint32_t bit_j = (1u << jj) << sh;
-                        atomicOr(&s_ltmpl[i], bit_j);
-                        atomicOr(&s_ltmpl[(uint32_t)m + jj], (1u << i) << sh);
-                        atomicOr(&s_ltmpl[(uint32_t)(m + n + n - 1) + i - jj], bit_j);
-                        atomicOr(&s_ltmpl[(uint32_t)(m + n + m + n - 1) + i + jj], bit_j);
-                    }
+                    if (tid == 0) s_count = cnt;
                 }
                 __syncthreads();
                 const int count0 = s_count;
