@@ -272,6 +272,11 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     if (tid == 0) s_abort = 0;
     uint64_t e0 = 0, e1 = 0;
     if (!ACP && tid == 0) { e0 = ref.rng_expand[0]; e1 = ref.rng_expand[1]; }
+    // One-child playouts that fit one round use the same generators, thread for thread, in every step: their states
+    // stay in registers for the whole launch.
+    const bool keep_rng = !ACP && P <= nslots;
+    uint64_t k0 = 0, k1 = 0;
+    if (keep_rng && tid < P) { k0 = ref.rng_playout[2 * tid]; k1 = ref.rng_playout[2 * tid + 1]; }
     uint32_t plies = 0, u1 = 0;
     uint32_t st_levels = 0, st_children = 0, st_expanded = 0, st_played = 0;
     unsigned long long tk_select = 0, tk_expand = 0, tk_playout = 0, tk_backup = 0, tk_exchange = 0, tk = 0;
@@ -453,7 +458,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     uint64_t s0 = 0, s1 = 0, s0_start = 0, s1_start = 0;
                     const uint32_t plies_start = plies;
                     if (t < P) {
-                        s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1];
+                        if (keep_rng) { s0 = k0; s1 = k1; } else { s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1]; }
                         s0_start = s0; s1_start = s1;
                         {
                             const int used = (count0 + 3) >> 2;
@@ -464,6 +469,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                         }
                         uint8_t *const lb = reinterpret_cast<uint8_t *>(s_list + tid);   // byte i: lb[(i >> 2) * stride4 + (i & 3)]
                         uint32_t *const lp = s_lines + tid;
+                        const uint32_t line_shift = (uint32_t)(33 - __clz(nslots));   // log2(4 * nslots)
                         const uint32_t nt = (uint32_t)nslots, stride4 = nt << 2;
                         int count = count0, outcome_if_win = pturn, status = count0 == 0 ? 2 : 0;
                         // byte selector that packs the mover's halves of two line words into one dword; flips with the side to move
@@ -494,9 +500,11 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                             plies++;
                             const uint32_t i = a >> 4, jj = a & 15u;
                             const uint32_t sh = (sel & 2u) << 3;  // 0 for the +1 side, 16 for the -1 side
-                            uint32_t *const p_row = lp + __umul24(i, nt), *const p_col = lp + __umul24((uint32_t)m + jj, nt);
-                            uint32_t *const p_dia = lp + __umul24((uint32_t)(m + n + n - 1) + i - jj, nt);
-                            uint32_t *const p_ant = lp + __umul24((uint32_t)(m + n + m + n - 1) + i + jj, nt);
+                            // (the playouts of a round are a power of two: a line's words are 4 << log2 bytes apart)
+                            auto line_word = [&](uint32_t line) { return reinterpret_cast<uint32_t *>(reinterpret_cast<unsigned char *>(lp) + (line << line_shift)); };
+                            uint32_t *const p_row = line_word(i), *const p_col = line_word((uint32_t)m + jj);
+                            uint32_t *const p_dia = line_word((uint32_t)(m + n + n - 1) + i - jj);
+                            uint32_t *const p_ant = line_word((uint32_t)(m + n + m + n - 1) + i + jj);
                             // the four lines through a cell are four different words: read all, then write all
                             uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
                             __builtin_amdgcn_sched_barrier(0);   // the line reads are in flight while the next cell is drawn
@@ -541,7 +549,10 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                             __syncthreads();
                         }
                     }
-                    if (t < P) { uint64_t *w = const_cast<uint64_t *>(rng_base); w[2 * t] = s0; w[2 * t + 1] = s1; }
+                    if (t < P) {
+                        if (keep_rng) { k0 = s0; k1 = s1; }
+                        else { uint64_t *w = const_cast<uint64_t *>(rng_base); w[2 * t] = s0; w[2 * t + 1] = s1; }
+                    }
                     const unsigned long long bn = __ballot(t < P && outcome == -1), bp = __ballot(t < P && outcome == 1);
                     if (lane == 0) { s_red[wave][0] = __popcll(bn); s_red[wave][1] = __popcll(bp); }
                     __syncthreads();
@@ -741,6 +752,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     }
 
     if (!ACP && tid == 0) { ref.rng_expand[0] = e0; ref.rng_expand[1] = e1; }
+    if (keep_rng && tid < P) { uint64_t *w = const_cast<uint64_t *>(ref.rng_playout); w[2 * tid] = k0; w[2 * tid + 1] = k1; }
     for (int off = 32; off > 0; off >>= 1) { plies += __shfl_xor(plies, off); u1 += __shfl_xor(u1, off); }
     if (lane == 0) {
         if (plies) atomicAdd(&hdr->plies, (unsigned long long)plies);

@@ -221,6 +221,7 @@ int gomoku_encode_root(const mctsnc_config &c, const int8_t *board, uint32_t bb[
     return MCTSNC_OK;
 }
 
+// (a power of two, as n_playouts is: the kernel finds a playout's line words with a shift)
 int gomoku_block(const mctsnc_config &c) { return c.n_playouts < 64 ? 64 : (c.n_playouts > gomoku::kMaxThreads ? gomoku::kMaxThreads : c.n_playouts); }
 
 int check_batch(mctsnc_engine **engines, int n, const int32_t *turns) {
@@ -675,6 +676,7 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
 
     gomoku::SearchArgs args;
     args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G; args.slots = e0->slots;
+    if (e0->slots < 64 || (e0->slots & (e0->slots - 1))) return fail(MCTSNC_E_STATE, "playouts per round (%d) must be a power of two >= 64", e0->slots);
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
