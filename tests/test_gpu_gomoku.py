@@ -40,6 +40,23 @@ def test_gomoku_small_boards_deep_trees(variant):
         compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else steps // 3)
 
 
+@pytest.mark.parametrize("variant,steps", [("acp_prodigal", 6), ("ocp_thrifty", 150)])
+def test_gomoku_children_that_complete_lines(variant, steps):
+    """A root whose children decide games at creation: a cell that completes exactly five (open four in a row; a gapped
+    four; a diagonal that ends in the board's corner region), a cell that would make six (no win), and a four of the
+    other side that the grandchildren complete.  Outcomes and terminal flags of every node against the oracle."""
+    board = np.zeros((15, 15), np.int8)
+    board[7, 3:7] = 1                                   # open four: (7,2) and (7,7) win for +1
+    board[9, [2, 3, 5, 6, 7]] = 1                       # (9,4) makes six: not a win
+    board[3, [8, 9, 11, 12]] = 1                        # gapped four: (3,10) wins
+    for k in range(4):
+        board[10 + k, k] = 1                            # diagonal (10,0)..(13,3): (14,4) wins, the other end is off the board
+        board[1 + k, 12] = -1                           # four of -1 in a column: its replies at (0,12) and (5,12) win
+    board[[0, 0, 5, 12, 14], [0, 5, 2, 9, 14]] = -1     # a few more stones of -1
+    e, o = engines(variant, 2, 64, 15, 15, seed=9)
+    compare_with_oracle(e, o, board, None, 1, steps)
+
+
 def test_gomoku_tree_full_path():
     from mcts_numba_cuda_amd import MCTSNC
     from oracle.oracle import Oracle
