@@ -51,6 +51,16 @@ static_assert(sizeof(Node) == 128, "node record must be 128 bytes");
 
 struct Stat { int32_t ns, wins, action, pad; };
 
+// Loads through pointers known to point to device memory (GLOBAL instead of FLAT instructions where the compiler cannot
+// tell: a FLAT load is counted with the LDS operations as well, and waits for LDS data then wait for memory).
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ Stat load_stat(const Stat *p) {
+    const i32x4 v = *(const __attribute__((address_space(1))) i32x4 *)p;
+    Stat st; st.ns = v.x; st.wins = v.y; st.action = v.z; st.pad = v.w;
+    return st;
+}
+__device__ __forceinline__ int32_t load_i32(const int32_t *p) { return *(const __attribute__((address_space(1))) int32_t *)p; }
+
 struct __attribute__((aligned(128))) TreeHdr {
     int32_t size, po_neg, po_pos, max_depth;
     int64_t depth_sum;
@@ -225,6 +235,15 @@ __host__ __device__ inline size_t playout_lds_bytes(int cells, int lines, int th
     return ((size_t)((cells + 3) / 4) + (size_t)lines) * sizeof(uint32_t) * threads;
 }
 
+// Arg-max key of a child: UCB, then the reference's tie rule (smallest bit-reversed action index among the maxima; the
+// 8-bit reversal orders actions < 256 as the 9-bit one does), the child's ordinal in the low byte.
+__device__ __forceinline__ unsigned long long child_key(const Stat &st, double log_parent_n, float ucb_c, int q) {
+    const float ucb = (st.ns == 0) ? __builtin_inff() : ucb_value(st.wins, st.ns, log_parent_n, ucb_c);
+    const uint32_t rev = __brev((uint32_t)st.action) >> 24;
+    const unsigned long long kq = (((unsigned long long)__float_as_uint(ucb) + 1ull) << 16) | ((unsigned long long)(255u - rev) << 8);
+    return (kq << 8) | (unsigned long long)q;
+}
+
 // The step skeleton for placement games: the whole search of the launch's trees by Game's rules.
 template <class Game, bool ACP>
 __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args) {
@@ -266,6 +285,13 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     __shared__ unsigned long long s_lkey[kLevels];   // per level of a chunk of the backup's arg-max: best key,
     __shared__ double s_llog[kLevels];               // log of the node's visit count,
     __shared__ int32_t s_lbase[kLevels], s_lkc[kLevels];   // first child and number of children
+    // one-child variants, per path level, prepared while the playouts run: the best key among the node's children off
+    // the path, the log of its visit count after the step, its first child; and the counters before the step of the
+    // root ([0]) and of the path node one level down ([level + 1])
+    __shared__ unsigned long long s_pkey[ACP ? 1 : kMaxPath];
+    __shared__ double s_plog[ACP ? 1 : kMaxPath];
+    __shared__ int32_t s_pbase[ACP ? 1 : kMaxPath];
+    __shared__ Stat s_pstat[ACP ? 1 : kMaxPath + 1];
     __shared__ int32_t s_flag, s_chosen, s_abort, s_redo, s_count;
     __shared__ ExactScratch s_exact;
 
@@ -404,6 +430,36 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
         if (!ACP && mode == kModeExpand) chosen_j = s_chosen;
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_expand += t2 - tk; tk = t2; }
 
+        // ---- one-child variants: the backup's arg-max, as far as it does not depend on the playouts ----
+        // A step changes the counters of the path nodes and of the child it plays out, by amounts known but for the wins;
+        // all other children of the path nodes keep theirs, and a node's visit count after the step is known.  So the
+        // best key among each path node's children off the path can be worked out before the results are in: by the
+        // wavefronts that play no playouts, while the others play.  Wavefronts first .. first + count - 1 take the
+        // levels in turn; nothing here is read by anyone before the barriers that end the playouts.
+        const int n_levels = (mode == kModeExpand) ? L + 1 : L;   // path nodes that have children after this step
+        bool prepared = false;
+        const float ucb_c = args.ucb_c;
+        auto prepare_backup = [=](int first, int count) {   // (by value: captured by reference, every pointer of the kernel is a generic one to the compiler)
+            if (wave == first && lane == 0) s_pstat[0] = load_stat(stats + s_path[0]);
+            for (int l = wave - first; l < n_levels; l += count) {
+                const int node = s_path[l];
+                const bool fresh = l == L;   // the children created in this step
+                const int base = fresh ? size : load_i32(&nodes[node].child_base), cnt = fresh ? k_exp : load_i32(&nodes[node].n_children);
+                const double log_n = det_log((double)(load_i32(&stats[node].ns) + P));
+                const int on_path = fresh ? chosen_j : s_path[l + 1] - base;
+                unsigned long long best = 0ull;
+                for (int q = lane; q < cnt; q += 64) {
+                    Stat st;
+                    if (fresh) { st.ns = 0; st.wins = 0; st.action = s_actions[q]; st.pad = 0; }
+                    else st = load_stat(stats + base + q);
+                    if (q == on_path) { if (!fresh) s_pstat[l + 1] = st; }
+                    else { const unsigned long long key = child_key(st, log_n, ucb_c, q); best = key > best ? key : best; }
+                }
+                for (int off = 32; off > 0; off >>= 1) { const unsigned long long o = __shfl_xor(best, off); best = o > best ? o : best; }
+                if (lane == 0) { s_pkey[l] = best; s_plog[l] = log_n; s_pbase[l] = base; }
+            }
+        };
+
         // ================= playouts (src/mctsnc.py:1823-2081) =================
         // list of (child ordinal) jobs of this workgroup: OCP one job, ACP every G-th child, full tree: the selected node
         int tot_neg = 0, tot_pos = 0;
@@ -457,6 +513,10 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     int outcome = 0; bool redo = false;
                     uint64_t s0 = 0, s1 = 0, s0_start = 0, s1_start = 0;
                     const uint32_t plies_start = plies;
+                    if (!ACP && round == 0 && nthreads > nslots) {   // (the same for every thread)
+                        if (tid >= nslots) prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
+                        prepared = true;
+                    }
                     if (t < P) {
                         if (keep_rng) { s0 = k0; s1 = k1; } else { s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1]; }
                         s0_start = s0; s1_start = s1;
@@ -525,6 +585,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                             const uint32_t win_j = Game::reach(jj), win_i = Game::reach(i);  // starts of a winning run through the stone
                             const uint32_t hit = Game::winning_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
                             const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
+                            __builtin_amdgcn_sched_barrier(0);   // (the list reads have had the whole test to return)
                             *slot_n = last_n;   // swap-remove of the next draw
                             if ((hit | hit2) != 0) { status = 1; outcome = outcome_if_win; rg = rg_now; }
                             else if (count == 0) { status = 2; outcome = 0; rg = rg_now; }
@@ -620,6 +681,18 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 else { neg_tot = tot_neg; pos_tot = tot_pos; }
             }
             // path nodes (src/mctsnc.py:2095-2103, :2212-2219)
+            if (!ACP) {
+                if (!prepared) {   // no wavefront was free during the playouts, or there were none: all prepare now
+                    prepare_backup(0, nwaves);
+                    __syncthreads();
+                }
+                for (int l = tid; l <= L; l += nthreads) {   // counters before the step + this step's, without reading memory again
+                    Stat st = s_pstat[l];
+                    const int turn_l = (l & 1) ? -root_turn : root_turn;
+                    st.ns += n_tot; st.wins += (turn_l == 1) ? neg_tot : pos_tot;
+                    stats[s_path[l]] = st;
+                }
+            } else
             for (int l = tid; l <= L; l += nthreads) {
                 const int node = s_path[l];
                 const int turn_l = (l & 1) ? -root_turn : root_turn;
@@ -671,7 +744,24 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             // tie rule (smallest bit-reversed action index among the maxima).  Levels are taken kLevels at a time and
             // all their (level, child) pairs in one flat loop, each thread fetching its next pair's counters while it
             // evaluates the current one; the maxima meet in LDS.
-            const int n_levels = (mode == kModeExpand) ? L + 1 : L;
+            if (!ACP) {
+                // one-child variants: the best of the children off the path is known (prepare_backup); the child on
+                // the path competes with its counters after this step
+                for (int l = tid; l < n_levels; l += nthreads) {
+                    Stat pc; int q;
+                    if (l == L) {   // the child just created and played out
+                        q = chosen_j;
+                        pc.ns = P; pc.wins = (-mover == 1) ? neg_tot : pos_tot; pc.action = s_actions[chosen_j]; pc.pad = 0;
+                    } else {
+                        q = s_path[l + 1] - s_pbase[l];
+                        pc = s_pstat[l + 1];
+                        const int turn_c = ((l + 1) & 1) ? -root_turn : root_turn;
+                        pc.ns += n_tot; pc.wins += (turn_c == 1) ? neg_tot : pos_tot;
+                    }
+                    const unsigned long long key = child_key(pc, s_plog[l], args.ucb_c, q), best = key > s_pkey[l] ? key : s_pkey[l];
+                    nodes[s_path[l]].best_child = s_pbase[l] + (int)(best & 0xffull);
+                }
+            } else
             for (int l0 = 0; l0 < n_levels; l0 += kLevels) {
                 const int nl = min(kLevels, n_levels - l0);
                 if (tid < nl) {
@@ -698,10 +788,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     int k_next = 0, q_next = 0;
                     Stat nxt = {0, 0, 0, 0};
                     if (i_next < tot) { locate(i_next, k_next, q_next); nxt = stats[s_lbase[k_next] + q_next]; }
-                    const float ucb = (cur.ns == 0) ? __builtin_inff() : ucb_value(cur.wins, cur.ns, s_llog[k_cur], args.ucb_c);
-                    const uint32_t rev = __brev((uint32_t)cur.action) >> 24;  // 8-bit reversal; same order as the 9-bit one for actions < 256
-                    const unsigned long long kq = (((unsigned long long)__float_as_uint(ucb) + 1ull) << 16) | ((unsigned long long)(255u - rev) << 8);
-                    atomicMax(&s_lkey[k_cur], (kq << 8) | (unsigned long long)q_cur);  // ordinal carried in the low byte
+                    atomicMax(&s_lkey[k_cur], child_key(cur, s_llog[k_cur], args.ucb_c, q_cur));
                     i = i_next; k_cur = k_next; q_cur = q_next; cur = nxt;
                 }
                 __syncthreads();
