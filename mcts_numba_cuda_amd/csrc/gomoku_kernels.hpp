@@ -377,57 +377,66 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     atomicOr(&s_lleaf[(uint32_t)(m + n + m + n - 1) + i + jj], bit_j);
                 }
             }
-        }
-        __syncthreads();
-
-        // ================= children: creation (src/mctsnc.py:1690-1821) =================
-        // OCP: the single workgroup creates all children; ACP: workgroup g creates the ordinals j = g, g + G, ...
-        if (mode == kModeExpand) {
-            for (int j = (ACP ? g : 0) + (ACP ? G : 1) * tid; j < k_exp; j += (ACP ? G : 1) * nthreads) {
-                const int a = s_actions[j];
-                // every index below is a constant after unrolling: a record indexed at run time would live in scratch memory
-                const uint32_t a_word = (uint32_t)a >> 5, a_bit = 1u << (a & 31);
-                Node nd;
-                nd.child_base = -1; nd.parent = leaf.node; nd.n_children = 0; nd.best_child = -1; nd.depth = (int16_t)(L + 1); nd.turn = (int8_t)(-mover);
-                nd.pad0 = 0; nd.action = (int16_t)a; nd.pad1[0] = nd.pad1[1] = 0;
-                int occ = 0;
-#pragma unroll
-                for (int w = 0; w < 8; w++) {
-                    const uint32_t add = (uint32_t)w == a_word ? a_bit : 0u;
-                    nd.bb_pos[w] = s_bb[w] | (mover == 1 ? add : 0u); nd.bb_neg[w] = s_bb[8 + w] | (mover == 1 ? 0u : add); nd.pad2[w] = 0;
-                    occ += __popc(nd.bb_pos[w] | nd.bb_neg[w]);
-                }
-                // the mover's stones on the four lines through the new one, two lines to a dword as in the playouts
-                const uint32_t ai = ((uint32_t)a * div_n) >> 16, aj = (uint32_t)a - ai * (uint32_t)n;
-                const uint32_t sh = mover == 1 ? 0u : 16u, sel = mover == 1 ? 0x05040100u : 0x07060302u, bit_j = (1u << aj) << sh;
-                const uint32_t w_row = s_lleaf[ai] | bit_j, w_col = s_lleaf[(uint32_t)m + aj] | ((1u << ai) << sh);
-                const uint32_t w_dia = s_lleaf[(uint32_t)(m + n + n - 1) + ai - aj] | bit_j, w_ant = s_lleaf[(uint32_t)(m + n + m + n - 1) + ai + aj] | bit_j;
-                const uint32_t win_j = Game::reach(aj), win_i = Game::reach(ai);
-                const uint32_t hit = Game::winning_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
-                const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
-                int outcome = 2;
-                if ((hit | hit2) != 0) outcome = mover;
-                else if (occ == cells) outcome = 0;
-                s_out[j] = (int8_t)outcome;
-                nd.outcome = (int8_t)outcome;
-                nd.flags = (uint8_t)(kLeaf | (outcome != 2 ? kTerminal : 0));
-                nodes[size + j] = nd;
-                Stat st; st.ns = 0; st.wins = 0; st.action = a; st.pad = 0;
-                stats[size + j] = st;
-            }
-        }
-        int chosen_j = -1;
-        if (!ACP && mode == kModeExpand) {
-            if (tid == 0) {
+            if (!ACP && mode == kModeExpand && tid == 0) {   // the one child that is played out
                 const float u = rng_uniform(e0, e1);
                 int ord = (int)(int16_t)((double)u * (double)k_exp);  // float32 * int64 -> float64 in the reference (src/mctsnc.py:1435)
                 if (ord > k_exp - 1) ord = k_exp - 1;
                 s_chosen = ord;
             }
         }
-        __threadfence_block();
         __syncthreads();
-        if (!ACP && mode == kModeExpand) chosen_j = s_chosen;
+        const int chosen_j = (!ACP && mode == kModeExpand) ? s_chosen : -1;
+
+        // ================= children: creation (src/mctsnc.py:1690-1821) =================
+        // Outcome of the child that places a stone on cell a: the playouts' own test on the mover's stones on the four
+        // lines through the cell, two lines to a dword; a draw when it was the last empty cell.
+        auto child_outcome = [=](int a) -> int {
+            const uint32_t ai = ((uint32_t)a * div_n) >> 16, aj = (uint32_t)a - ai * (uint32_t)n;
+            const uint32_t sh = mover == 1 ? 0u : 16u, sel = mover == 1 ? 0x05040100u : 0x07060302u, bit_j = (1u << aj) << sh;
+            const uint32_t w_row = s_lleaf[ai] | bit_j, w_col = s_lleaf[(uint32_t)m + aj] | ((1u << ai) << sh);
+            const uint32_t w_dia = s_lleaf[(uint32_t)(m + n + n - 1) + ai - aj] | bit_j, w_ant = s_lleaf[(uint32_t)(m + n + m + n - 1) + ai + aj] | bit_j;
+            const uint32_t win_j = Game::reach(aj), win_i = Game::reach(ai);
+            const uint32_t hit = Game::winning_starts(__builtin_amdgcn_perm(w_dia, w_row, sel)) & (win_j | (win_j << 16));
+            const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
+            return (hit | hit2) != 0 ? mover : (empties == 1 ? 0 : 2);
+        };
+        // Records and counters of the children j0, j0 + stride, ...: the record as eight 16-byte stores (field layout of
+        // Node), typed as device memory; the counters of child `played` are left to the thread that stores its result.
+        auto create_children = [=](int j0, int stride, int played) {
+            typedef __attribute__((address_space(1))) i32x4 *DeviceQuads;
+            for (int j = j0; j < k_exp; j += stride) {
+                const int a = s_actions[j];
+                const uint32_t a_word = (uint32_t)a >> 5, a_bit = 1u << (a & 31);
+                const int outcome = child_outcome(a);
+                s_out[j] = (int8_t)outcome;
+                uint32_t bb[16];   // (constant indices after unrolling: registers)
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    const uint32_t add = (uint32_t)w == a_word ? a_bit : 0u;
+                    bb[w] = s_bb[w] | (mover == 1 ? add : 0u); bb[8 + w] = s_bb[8 + w] | (mover == 1 ? 0u : add);
+                }
+                const uint32_t flags = (uint32_t)kLeaf | (outcome != 2 ? (uint32_t)kTerminal : 0u);
+                const DeviceQuads rec = (DeviceQuads)(nodes + size + j);
+                const i32x4 zero = {0, 0, 0, 0};
+                rec[0] = i32x4{-1, leaf.node, 0, -1};   // child_base, parent, n_children, best_child
+                rec[1] = i32x4{(int32_t)(((uint32_t)(L + 1) & 0xffffu) | (((uint32_t)(-mover) & 0xffu) << 16) | (((uint32_t)outcome & 0xffu) << 24)),
+                               (int32_t)(flags | ((uint32_t)a << 16)), 0, 0};   // depth, turn, outcome; flags, action
+#pragma unroll
+                for (int q = 0; q < 4; q++) rec[2 + q] = i32x4{(int32_t)bb[4 * q], (int32_t)bb[4 * q + 1], (int32_t)bb[4 * q + 2], (int32_t)bb[4 * q + 3]};
+                rec[6] = zero; rec[7] = zero;
+                if (j != played) *(DeviceQuads)(stats + size + j) = i32x4{0, 0, a, 0};
+            }
+        };
+        // OCP: the single workgroup creates all children; ACP: workgroup g creates the ordinals j = g, g + G, ...
+        // One-child variants with wavefronts that play no playouts leave the creation to those, while the others play:
+        // the playouts need the chosen child's outcome only, which every thread works out for itself.
+        const int chosen_outcome = (!ACP && mode == kModeExpand) ? child_outcome(s_actions[chosen_j]) : 2;
+        const bool deferred = !ACP && mode == kModeExpand && nthreads > nslots && chosen_outcome == 2;
+        if (mode == kModeExpand && !deferred) {
+            create_children((ACP ? g : 0) + (ACP ? G : 1) * tid, (ACP ? G : 1) * nthreads, -1);
+            __threadfence_block();
+            __syncthreads();
+        }
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_expand += t2 - tk; tk = t2; }
 
         // ---- one-child variants: the backup's arg-max, as far as it does not depend on the playouts ----
@@ -471,7 +480,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             if (mode == kModeExpand) { pnode = size + j; last_action = s_actions[j]; pturn = -mover; paction = last_action; }
             else { pnode = leaf.node; last_action = -1; pturn = mover; paction = 0; }
             int job_neg = 0, job_pos = 0;
-            const int poutcome = (mode == kModeExpand) ? s_out[j] : 2;   // this workgroup created the children it plays out
+            const int poutcome = (mode == kModeExpand) ? (ACP ? (int)s_out[j] : chosen_outcome) : 2;   // (all-children variants: this workgroup created the children it plays out)
             if (poutcome != 2) {  // terminal child: stored outcome times P (src/mctsnc.py:1842-1846)
                 job_neg = poutcome == -1 ? P : 0; job_pos = poutcome == 1 ? P : 0;
             } else {
@@ -514,7 +523,10 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     uint64_t s0 = 0, s1 = 0, s0_start = 0, s1_start = 0;
                     const uint32_t plies_start = plies;
                     if (!ACP && round == 0 && nthreads > nslots) {   // (the same for every thread)
-                        if (tid >= nslots) prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
+                        if (tid >= nslots) {
+                            if (deferred) create_children(tid - nslots, nthreads - nslots, chosen_j);
+                            prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
+                        }
                         prepared = true;
                     }
                     if (t < P) {
