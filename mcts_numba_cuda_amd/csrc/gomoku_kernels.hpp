@@ -522,7 +522,17 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     int outcome = 0; bool redo = false;
                     uint64_t s0 = 0, s1 = 0, s0_start = 0, s1_start = 0;
                     const uint32_t plies_start = plies;
-                    if (!ACP && round == 0 && nthreads > nslots) {   // (the same for every thread)
+                    const bool helped = !ACP && round == 0 && nthreads > nslots;   // (the same for every thread)
+                    if (helped) {
+                        // all wavefronts fill the playouts' columns from the templates, each its share of the dwords
+                        const int col = tid & (nslots - 1), part = tid / nslots, parts = nthreads / nslots, used = (count0 + 3) >> 2;
+                        if (col < P) {
+#pragma unroll 4
+                            for (int k = part; k < used; k += parts) s_list[k * nslots + col] = s_tmpl[k];
+#pragma unroll 4
+                            for (int k = part; k < n_lines; k += parts) s_lines[k * nslots + col] = s_ltmpl[k];
+                        }
+                        __syncthreads();
                         if (tid >= nslots) {
                             if (deferred) create_children(tid - nslots, nthreads - nslots, chosen_j);
                             prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
@@ -532,7 +542,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                     if (t < P) {
                         if (keep_rng) { s0 = k0; s1 = k1; } else { s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1]; }
                         s0_start = s0; s1_start = s1;
-                        {
+                        if (!helped) {
                             const int used = (count0 + 3) >> 2;
 #pragma unroll 8
                             for (int k = 0; k < used; k++) s_list[k * nslots + tid] = s_tmpl[k];
