@@ -26,6 +26,7 @@ constexpr int kMaxCells = 256;    // m * n <= 256, m, n <= 16
 constexpr int kMaxPath = 258;     // a tree can be m * n + 1 levels deep
 constexpr int kMaxLines = 96;     // 3 * (m + n) - 2 <= 94
 constexpr int kLevels = 8;         // path levels whose arg-max the backup evaluates together
+constexpr int kPrepLevels = 48;    // path levels whose arg-max the one-child variants prepare during the playouts (deeper paths: as above)
 constexpr int kMaxThreads = 256;  // playouts beyond this run in several rounds of the same workgroup
 constexpr uint8_t kLeaf = 1, kTerminal = 2;
 constexpr int kModeExpand = 0, kModeTerminal = 1, kModeFull = 2;
@@ -101,6 +102,7 @@ struct SearchArgs {
     float ucb_c;
     int32_t stage_timing;
     int32_t agent_fences;   // never take the same-XCC shortcuts (full device-scope release and acquire every step)
+    int32_t prep_levels;    // one-child variants: paths up to this many levels have their backup prepared during the playouts (<= kPrepLevels)
     int32_t *abort_flag;
 };
 
@@ -288,10 +290,11 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     // one-child variants, per path level, prepared while the playouts run: the best key among the node's children off
     // the path, the log of its visit count after the step, its first child; and the counters before the step of the
     // root ([0]) and of the path node one level down ([level + 1])
-    __shared__ unsigned long long s_pkey[ACP ? 1 : kMaxPath];
-    __shared__ double s_plog[ACP ? 1 : kMaxPath];
-    __shared__ int32_t s_pbase[ACP ? 1 : kMaxPath];
-    __shared__ Stat s_pstat[ACP ? 1 : kMaxPath + 1];
+    // (sized so that two workgroups with 128 playouts each still fit the LDS of a CU)
+    __shared__ unsigned long long s_pkey[ACP ? 1 : kPrepLevels];
+    __shared__ double s_plog[ACP ? 1 : kPrepLevels];
+    __shared__ int32_t s_pbase[ACP ? 1 : kPrepLevels];
+    __shared__ Stat s_pstat[ACP ? 1 : kPrepLevels + 1];
     __shared__ int32_t s_flag, s_chosen, s_abort, s_redo, s_count;
     __shared__ ExactScratch s_exact;
 
@@ -446,6 +449,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
         // wavefronts that play no playouts, while the others play.  Wavefronts first .. first + count - 1 take the
         // levels in turn; nothing here is read by anyone before the barriers that end the playouts.
         const int n_levels = (mode == kModeExpand) ? L + 1 : L;   // path nodes that have children after this step
+        const bool can_prepare = !ACP && L < args.prep_levels;
         bool prepared = false;
         const float ucb_c = args.ucb_c;
         auto prepare_backup = [=](int first, int count) {   // (by value: captured by reference, every pointer of the kernel is a generic one to the compiler)
@@ -535,9 +539,9 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                         __syncthreads();
                         if (tid >= nslots) {
                             if (deferred) create_children(tid - nslots, nthreads - nslots, chosen_j);
-                            prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
+                            if (can_prepare) prepare_backup(nslots >> 6, nwaves - (nslots >> 6));
                         }
-                        prepared = true;
+                        prepared = can_prepare;
                     }
                     if (t < P) {
                         if (keep_rng) { s0 = k0; s1 = k1; } else { s0 = rng_base[2 * t]; s1 = rng_base[2 * t + 1]; }
@@ -703,7 +707,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 else { neg_tot = tot_neg; pos_tot = tot_pos; }
             }
             // path nodes (src/mctsnc.py:2095-2103, :2212-2219)
-            if (!ACP) {
+            if (can_prepare) {
                 if (!prepared) {   // no wavefront was free during the playouts, or there were none: all prepare now
                     prepare_backup(0, nwaves);
                     __syncthreads();
@@ -766,7 +770,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             // tie rule (smallest bit-reversed action index among the maxima).  Levels are taken kLevels at a time and
             // all their (level, child) pairs in one flat loop, each thread fetching its next pair's counters while it
             // evaluates the current one; the maxima meet in LDS.
-            if (!ACP) {
+            if (can_prepare) {
                 // one-child variants: the best of the children off the path is known (prepare_backup); the child on
                 // the path competes with its counters after this step
                 for (int l = tid; l < n_levels; l += nthreads) {

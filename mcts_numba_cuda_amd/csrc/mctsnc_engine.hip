@@ -680,6 +680,8 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
     args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
+    args.prep_levels = gomoku::kPrepLevels;
+    if (const char *v = getenv("MCTSNC_PREP_LEVELS")) args.prep_levels = std::max(0, std::min(atoi(v), gomoku::kPrepLevels));   // for testing the path deep trees take
     const dim3 block(e0->block);
     const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots);
     // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
