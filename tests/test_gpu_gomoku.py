@@ -70,6 +70,15 @@ def test_gomoku_one_child_backup_of_paths_too_deep_to_prepare(monkeypatch, level
         compare_with_oracle(e, o, board, None, turn, steps)
 
 
+@pytest.mark.parametrize("P", [1, 8, 32, 256])
+def test_gomoku_one_child_other_playout_counts(P):
+    """A one-child workgroup has 256 threads whatever the playout count: with fewer playouts the other wavefronts help
+    (LDS columns, children, the backup's arg-max), with 256 every wavefront plays and none is left to help."""
+    e, o = engines("ocp_thrifty", 2, P, 9, 9, seed=4)
+    board, turn = random_gomoku_root(np.random.default_rng(P), 9, 9, 6)
+    compare_with_oracle(e, o, board, None, turn, 60 if P < 256 else 25)
+
+
 def test_gomoku_tree_full_path():
     from mcts_numba_cuda_amd import MCTSNC
     from oracle.oracle import Oracle
