@@ -221,8 +221,15 @@ int gomoku_encode_root(const mctsnc_config &c, const int8_t *board, uint32_t bb[
     return MCTSNC_OK;
 }
 
-// (a power of two, as n_playouts is: the kernel finds a playout's line words with a shift)
-int gomoku_block(const mctsnc_config &c) { return c.n_playouts < 64 ? 64 : (c.n_playouts > gomoku::kMaxThreads ? gomoku::kMaxThreads : c.n_playouts); }
+// Playouts a Gomoku workgroup runs at a time (a power of two, as n_playouts is: the kernel finds a playout's line words
+// with a shift): as many as there are playouts, up to 256, and no more than fit the LDS of a CU beside the kernel's own
+// 8 KB (16 x 16 boards: 128; more playouts then run in rounds).
+int gomoku_block(const mctsnc_config &c) {
+    int slots = c.n_playouts < 64 ? 64 : (c.n_playouts > gomoku::kMaxThreads ? gomoku::kMaxThreads : c.n_playouts);
+    const size_t lds_of_a_cu = 160 * 1024, kernels_own = 8 * 1024;
+    while (slots > 64 && gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, slots) + kernels_own > lds_of_a_cu) slots /= 2;
+    return slots;
+}
 
 int check_batch(mctsnc_engine **engines, int n, const int32_t *turns) {
     if (n < 1) return fail(MCTSNC_E_INVALID, "no engines given");

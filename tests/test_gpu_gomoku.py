@@ -110,6 +110,15 @@ def test_gomoku_sixteen_wide_boards(variant):
         compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else max(3, steps // 10))
 
 
+@pytest.mark.parametrize("variant,steps", [("ocp_prodigal", 20), ("acp_thrifty", 3)])
+def test_gomoku_largest_board_with_256_playouts(variant, steps):
+    """On 16x16 the lists and line words of 256 playouts do not fit the LDS of a CU: the workgroup then holds 128 at a
+    time and plays 256 in two rounds."""
+    e, o = engines(variant, 2, 256, 16, 16, seed=8)
+    board, turn = random_gomoku_root(np.random.default_rng(3), 16, 16, 30)
+    compare_with_oracle(e, o, board, None, turn, steps)
+
+
 def test_gomoku_all_child_playouts_in_rounds():
     """n_playouts = 512 with all-child-playouts: every child's playouts run in two rounds of 256, one tree spread over
     all XCDs."""
