@@ -3,15 +3,32 @@
  *
  * The reference has no such loop: its PUCT kernels stop at selection (src/puct/puct_gpu_v3_cpp.cu:277-448) and backup
  * (src/puct/puct_gpu_v2.py:847-927) on synthetic trees.  This engine puts the step between them — committing the
- * claimed expansion slot, creating the child position, evaluating it — around those two kernels, for Gomoku with the
- * rules of the reference's game plugin (five in a row exactly, src/mctsnc_game_mechanics.py:181-280), a synthetic
- * evaluator (Dirichlet priors over the legal cells and a value, both pure functions of the position) and the
- * reference's array layout and sizes (src/puct/puct_gpu_v2.py:69-103: [trees, nodes, edges] arrays, nodes <= 16384,
- * edges <= 256).
+ * claimed expansion slot, creating the child position, evaluating it — around the same selection and backup rules, for
+ * Gomoku with the rules of the reference's game plugin (five in a row exactly,
+ * src/mctsnc_game_mechanics.py:181-280) and a synthetic evaluator (Dirichlet priors over the legal cells and a value,
+ * both pure functions of the position).
  *
- * One step = every tree runs `traversals` selections at once (one 64-lane wavefront each, virtual loss between
- * them), then expands / evaluates the selected leaves, then backs the values up.  All steps of a search run inside one
- * kernel launch, one workgroup per tree.
+ * One step = every tree runs `traversals` selections with virtual loss between them, then expands / evaluates the
+ * selected leaves, then backs the values up.  All steps of a search run inside one kernel launch, one workgroup per
+ * tree and one 64-lane wavefront per traversal.
+ *
+ * Selection.  Every decision of a traversal is the reference's (src/puct/puct_gpu_v3_cpp.cu:150-275): progressive
+ * widening from the node's visits plus claims in flight, capped by the node's number of empty cells; an expansion
+ * ticket if widening allows another child; otherwise the edge with the highest score q + cpuct * prior *
+ * sqrt(parent) / (n + in flight + 1), ties broken by the edge index rotated by the traversal's number; one unit of
+ * virtual loss on the chosen edge.  What this loop fixes, and the reference's kernel leaves to the timing of its
+ * atomics, is the order in which the traversals of a tree take their claims: they descend in lockstep, one level per
+ * round, and the traversals standing on the same node decide one after another, traversal number ascending, each
+ * seeing the claims and tickets of those before it.  That is one of the interleavings the reference's kernel allows; a
+ * claim taken in turn never loses, so the reference's winner-recalc retry and soft winner have nothing to do here, and a
+ * search is reproducible: the same configuration gives the same trees, bit for bit, on every run.  A traversal ends BUSY
+ * when it reaches a node that has no child yet and whose only allowed child is being created by a traversal before it;
+ * it keeps its claims until the step's backup gives them back (no traversal of the same step reads those edges again).
+ * With c_pw >= traversals a node without children admits one ticket per traversal and nothing ends BUSY.
+ *
+ * Storage is the loop's own, not the [trees, nodes, edges] arrays of the selection launcher (include/puct_select.h): one
+ * 16-byte record per edge (visits, value sum, prior, child and claims in flight), one per node, up to 2^20 nodes per
+ * tree; puct_gomoku_read() hands the fields out in the launcher's array shapes.
  *
  * All functions return 0 on success or a negative error code; puct_gomoku_last_error() describes the last failure
  * of the calling thread.  Host pointers only; the engine owns its device memory.
@@ -30,15 +47,23 @@ extern "C" {
 #define PUCT_GOMOKU_E_HIP (-2)
 #define PUCT_GOMOKU_E_ROOT (-3)
 
+#define PUCT_GOMOKU_MAX_NODES (1 << 20)
+#define PUCT_GOMOKU_MAX_PATH_DEPTH 256
+
+/* Selection word of a traversal (array PUCT_GOMOKU_ARR_OUT_SELECTED): kind << 28 | expansion slot << 20 | node, kinds
+ * as in include/puct_select.h (invalid 0, expand 1, terminal 2, depth limit 3, busy 4); node = all ones when the
+ * traversal reached no node. */
+#define PUCT_GOMOKU_SEL_NODE_MASK 0xFFFFF
+#define PUCT_GOMOKU_SEL_SLOT_SHIFT 20
+#define PUCT_GOMOKU_SEL_KIND_SHIFT 28
+
 typedef struct {
     int32_t board_m, board_n;  /* rows, columns; m * n <= 256 */
     int32_t trees;             /* independent trees on the same root, each with its own synthetic evaluator */
-    int32_t traversals;        /* concurrent selections per tree and step, 1..16 */
-    int32_t max_nodes;         /* node capacity per tree, 2..16384 */
-    int32_t path_depth;        /* longest path a selection may take, 1..1024 */
+    int32_t traversals;        /* selections per tree and step, 1..16 */
+    int32_t max_nodes;         /* node capacity per tree, 2..2^20 */
+    int32_t path_depth;        /* longest path a selection may take, 1..256 */
     float cpuct, c_pw, alpha_pw;
-    int32_t soft_winner;
-    int32_t recalc_attempts;   /* attempts of the winner-recalc claim per level, 1..64; 0 = 2 as in the reference's kernel */
     float dirichlet_alpha;     /* in (0, 1) */
     uint64_t seed;
     int32_t device;
@@ -55,8 +80,9 @@ typedef struct {
     int64_t nodes_total;             /* nodes over all trees after the search */
     int32_t max_nodes_in_tree;
     double time_total, time_device;  /* seconds */
-    int64_t levels_read;             /* tree levels the selections read (node word, ticket counter, edge rows) */
-    int64_t edges_examined;          /* expanded edges scored on those levels */
+    int64_t nodes_read;              /* node visits of the selections that loaded the node (its word and its expanded edges);
+                                        traversals standing on the same node in the same round share one */
+    int64_t edges_scored;            /* expanded edges loaded on those visits */
 } puct_gomoku_result;
 
 typedef struct puct_gomoku_engine puct_gomoku_engine;
@@ -65,28 +91,24 @@ int puct_gomoku_create(const puct_gomoku_config *config, puct_gomoku_engine **ou
 void puct_gomoku_destroy(puct_gomoku_engine *engine);
 
 /* Searches from `board` (int8 [m, n]: 0 empty, +1 / -1 stones) with `turn` (+1 / -1) to move for `steps` steps.
- * fused != 0: one kernel launch for the whole search; fused == 0: three launches per step (the selection of
- * puct_select_winner_recalc_launch, expansion / evaluation, the backup of puct_edge_backup_launch) — same results
- * whenever the selections of a step do not race (traversals == 1).  Selection differs from the plain launcher in one
- * point: progressive widening is capped by the node's number of empty cells instead of by the edge dimension, so a
- * fully expanded node is descended through rather than asked for another slot.
- * Edge slots: an expansion puts the child into the node's next free edge slot at the time it is committed (slots are
- * in descending prior order); the slot field of the selection word is the ticket that entitled the traversal to expand,
- * and the tickets of one step are not always contiguous, the expanded edges of a node always are.
- * Node limit: a tree holds at most max_nodes nodes (<= 16384, the node field of the packed selection word,
- * src/puct/puct_gpu_v3_cpp.cu:11-12).  The expansions a step selects in one tree are committed together or not at
- * all: once they no longer all fit, none of that step is committed in that tree, each of those traversals evaluates
- * the node it reached as a leaf instead (the evaluator's value of its position), backs that value up its path and
- * gives its expansion ticket back (a traversal that was asked to widen the root itself has an empty path and leaves
- * no visit).  The search then goes on over a tree that no longer grows: node_count stays within
+ * fused != 0: one kernel launch for the whole search; fused == 0: three launches per step (selection, expansion /
+ * evaluation, backup) — same results.
+ * Edge slots: an expansion puts the child into the node's next free edge slot, in traversal order (slots are in
+ * descending prior order); the slot field of the selection word is the ticket that entitled the traversal to expand.
+ * Node limit: a tree holds at most max_nodes nodes.  The expansions a step selects in one tree are committed together
+ * or not at all: once they no longer all fit, none of that step is committed in that tree, each of those traversals
+ * evaluates the node it reached as a leaf instead (the evaluator's value of its position), backs that value up its
+ * path and gives its expansion ticket back (a traversal that was asked to widen the root itself has an empty path and
+ * leaves no visit).  The search then goes on over a tree that no longer grows: node_count stays within
  * `traversals` of max_nodes and never exceeds it, nothing is left in flight, and result->expansions_committed stays
  * nodes_total - trees. */
 int puct_gomoku_run(puct_gomoku_engine *engine, const int8_t *board, int32_t turn, int32_t steps, int32_t fused,
                     puct_gomoku_result *result);
 
-/* Copies one device array of the last search to the host.  Shapes (T trees, N = max_nodes, E = 256, W traversals,
- * D = path_depth): see the ids below.  `bytes` must equal the array's size. */
-#define PUCT_GOMOKU_ARR_EDGE_CHILD 0       /* int32 [T, N, E] */
+/* Copies one array of the last search to the host (edge and node fields are gathered from their records on the device
+ * first).  Shapes (T trees, N = max_nodes, E = 256, W traversals, D = path_depth): see the ids below.  `bytes` must equal
+ * the array's size.  Rows of nodes that were never created hold no defined values. */
+#define PUCT_GOMOKU_ARR_EDGE_CHILD 0       /* int32 [T, N, E]: -1 = no child */
 #define PUCT_GOMOKU_ARR_EDGE_PRIOR 1       /* float32 [T, N, E] */
 #define PUCT_GOMOKU_ARR_EDGE_W 2           /* float32 [T, N, E] */
 #define PUCT_GOMOKU_ARR_EDGE_N 3           /* int32 [T, N, E] */
@@ -99,7 +121,7 @@ int puct_gomoku_run(puct_gomoku_engine *engine, const int8_t *board, int32_t tur
 #define PUCT_GOMOKU_ARR_NODE_TURN 10       /* int8 [T, N] */
 #define PUCT_GOMOKU_ARR_NODE_VALUE 11      /* float32 [T, N]: value of a terminal node for its player to move */
 #define PUCT_GOMOKU_ARR_OUT_SELECTED 12    /* int32 [T, W]: last step */
-#define PUCT_GOMOKU_ARR_OUT_PATH 13        /* int32 [T, W, D]: last step */
+#define PUCT_GOMOKU_ARR_OUT_PATH 13        /* int32 [T, W, D]: last step, node << 8 | edge slot per level, -1 beyond the path */
 #define PUCT_GOMOKU_ARR_OUT_LEN 14         /* int32 [T, W]: last step */
 #define PUCT_GOMOKU_ARR_PATH_VALUES 15     /* float32 [T, W, D]: last step */
 #define PUCT_GOMOKU_ARR_NODE_LEGAL 16      /* int32 [T, N]: empty cells of the node's position = most children it can have */

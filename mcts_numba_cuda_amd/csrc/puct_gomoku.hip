@@ -1,6 +1,8 @@
-// Gomoku PUCT search loop with virtual loss: the expansion / evaluation step between the selection and backup
-// kernels, a kernel that runs all steps of a search in one launch (one workgroup per tree, one wavefront per
-// traversal), and the host engine behind include/puct_gomoku.h.
+// Gomoku PUCT search loop with virtual loss behind include/puct_gomoku.h: selection, expansion / evaluation and backup of
+// all steps of a search in one launch, one workgroup per tree and one wavefront per traversal, on the loop's own tree
+// storage (one 16-byte record per edge, one per node), and the host engine.  A tree belongs to one workgroup for the
+// whole launch, so the traversals' claims are taken in a fixed order on registers instead of with atomics in memory,
+// which also makes a search reproducible.
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -18,30 +20,57 @@ using namespace puct;
 constexpr int kEdges = 256;       // edge slots per node (MAX_ACTION of src/puct/puct_gpu_v2.py:72)
 constexpr int kBoardWords = 16;   // 8 words per colour
 
-struct GomokuArgs {
-    SelectArgs sel;
-    BackupArgs bk;
-    int *node_expanded, *node_count, *node_expand_inflight, *node_legal;
-    uint32_t *node_board;
-    int8_t *node_turn;
-    float *node_value;
-    uint8_t *edge_action;
-    int *edge_child;
-    float *edge_prior;
-    float *edge_W;
-    int *edge_N;
-    int *edge_inflight;
-    float *path_values;
-    unsigned long long *tally;   // [trees][8]: selections by kind (0..4), children created (5)
-    int m, n, cells, max_nodes, steps;
+struct Edge {
+    int n;          // visits
+    float w;        // value sum, for the player who moves along the edge
+    float prior;
+    uint32_t link;  // child << 8 | claims in flight (virtual loss); child 0 = none (node 0 is the root)
+};
+static_assert(sizeof(Edge) == 16, "one edge is one 16-byte load");
+
+struct NodeInfo {
+    int expanded;    // edge slots with a child, or PUCT_NODE_EXPANDED_TERMINAL
+    int tickets;     // expansion tickets in flight
+    int legal_turn;  // empty cells of the position (most children the node can have) | 0x10000 if -1 is to move
+    float value;     // of the position for its player to move
+};
+static_assert(sizeof(NodeInfo) == 16, "one node word is one 16-byte load");
+constexpr int kTurnBit = 0x10000;
+
+constexpr int kTrav = kMaxWavesPerBlock;   // most traversals per tree: one wavefront each, one workgroup per tree
+constexpr int kSlices = kEdges / kWave;    // 64-edge slices of the widest node
+
+struct LoopArgs {
+    Edge *edges;       // [trees][max_nodes][256]
+    NodeInfo *info;    // [trees][max_nodes]
+    uint32_t *board;   // [trees][max_nodes][16]
+    uint8_t *action;   // [trees][max_nodes][256]: cell of every edge slot
+    int *node_count;   // [trees]
+    // what the traversals of the last step ended with, [trees][traversals] (paths: [trees][traversals][path_depth])
+    int *out_selected, *out_len, *out_claims, *out_path;
+    float *out_value;
+    unsigned long long *tally;   // [trees][8]: selections by kind (0..4), children created (5), nodes read (6), edges scored (7)
+    float cpuct, c_pw, alpha_pw;
+    int m, n, cells, max_nodes, traversals, path_depth, steps;
     uint64_t seed;
     double dirichlet_alpha;
 };
 
-struct Lds {
-    int want[kMaxWavesPerBlock];
-    uint32_t board[kMaxWavesPerBlock][kBoardWords];
+// What a step keeps per traversal between its phases.  The paths ([traversals][path_depth] words) follow in dynamic LDS.
+struct StepLds {
+    int cur[2][kTrav];   // node every traversal stands on, -1 once it has ended; double buffered by level parity
+    int sel[kTrav];      // selection word: kind << 28 | slot << 20 | node
+    int len[kTrav];      // path length as reported (nodes on the path; 0 for a traversal that reached no node)
+    int claims[kTrav];   // edges the traversal holds a claim on = path entries written
+    float value[kTrav];  // of the reached node, for the player who moved into it
+    int want[kTrav];     // node the traversal expands, -1 if none
+    int node_count;
+    uint32_t board[kTrav][kBoardWords];
 };
+
+__device__ __forceinline__ int pack_sel(int kind, int node, int slot) {
+    return (kind << PUCT_GOMOKU_SEL_KIND_SHIFT) | (slot << PUCT_GOMOKU_SEL_SLOT_SHIFT) | node;
+}
 
 __device__ __forceinline__ uint64_t wave_sum64(uint64_t v) {
     auto step = [](uint64_t x, auto ctrl) {
@@ -123,10 +152,24 @@ __device__ __forceinline__ void bitonic_sort(uint32_t (&v)[4], int lane) {
 }
 __device__ __forceinline__ void sort_keys_descending(uint32_t (&v)[4], int lane) { bitonic_sort<256>(v, lane); }
 
+__device__ __forceinline__ Edge load_edge(const Edge *p) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(p);
+    return Edge{(int)v.x, __uint_as_float(v.y), __uint_as_float(v.z), v.w};
+}
+__device__ __forceinline__ void store_edge(Edge *p, int n, float w, float prior, uint32_t link) {
+    *reinterpret_cast<uint4 *>(p) = make_uint4((uint32_t)n, __float_as_uint(w), __float_as_uint(prior), link);
+}
+__device__ __forceinline__ NodeInfo load_info(const NodeInfo *p) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(p);
+    return NodeInfo{(int)v.x, (int)v.y, (int)v.z, __uint_as_float(v.w)};
+}
+__device__ __forceinline__ uint64_t lanes_below(int lane) { return (1ull << lane) - 1ull; }
+
 // Priors of a new node: one Gamma weight per legal cell, prior = weight / sum, edge slots in descending weight order
-// (ties: smaller cell first), so that progressive widening opens the most promising moves first.  Initialises every
-// edge field of the node's legal slots.  All 64 lanes must call it together.
-__device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint32_t *board, int lane, uint64_t board_hash,
+// (ties: smaller cell first), so that progressive widening opens the most promising moves first.  Writes the whole
+// record of every legal slot (no visits, no child, nothing in flight) and the slot's cell.  All 64 lanes must call it
+// together.
+__device__ void write_priors(const LoopArgs &g, int tree, int node, const uint32_t *board, int lane, uint64_t board_hash,
                              int n_legal) {
     constexpr int kPer = kEdges / kWave;
     uint32_t mine[kPer];
@@ -164,73 +207,216 @@ __device__ void write_priors(const GomokuArgs &g, int tree, int node, const uint
     sum = wave_sum64(sum);
     // slot of a cell = rank of its key among the node's keys, largest first (0 = not a legal cell: last)
     sort_keys_descending(mine, lane);
-    const size_t erow = ((size_t)tree * g.sel.nodes + node) * kEdges + (size_t)kPer * lane;
+    const size_t erow = ((size_t)tree * g.max_nodes + node) * kEdges + (size_t)kPer * lane;
+    uint32_t cells_packed = 0;
 #pragma unroll
     for (int k = 0; k < kPer; ++k) {
-        if (mine[k] == 0u) continue;
-        const size_t e = erow + k;
-        g.edge_prior[e] = psyn_prior(psyn_key_weight(mine[k]), sum, n_legal);
-        g.edge_action[e] = (uint8_t)(255u - (mine[k] & 0xFFu));
-        g.edge_child[e] = -1;
-        g.edge_N[e] = 0;
-        g.edge_W[e] = 0.0f;
-        g.edge_inflight[e] = 0;
+        cells_packed |= (mine[k] ? 255u - (mine[k] & 0xFFu) : 0u) << (8 * k);
+        if (mine[k] != 0u) store_edge(g.edges + erow + k, 0, 0.0f, psyn_prior(psyn_key_weight(mine[k]), sum, n_legal), 0u);
+    }
+    if (mine[0] != 0u) *reinterpret_cast<uint32_t *>(g.action + erow) = cells_packed;   // keys descend: slot 4 * lane is the lane's first
+}
+
+// ---- selection ---------------------------------------------------------------------------------------------------
+// The traversals of a tree descend in lockstep, one level per round.  The traversals that stand on the same node are
+// served by one wavefront (that of the first of them), which loads the node's edges once and lets the traversals decide
+// one after another, wid ascending, on registers: every decision is the reference's (progressive widening, expansion
+// ticket, score, order on edges with the rotated tie-break: src/puct/puct_gpu_v3_cpp.cu:150-275) on the state that the
+// claims of the traversals before it have left.  Taking the claims in turn is one of the interleavings the reference's
+// atomics allow, needs no atomics itself, never loses a claim and makes a search reproducible.
+__device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *next, int tree, int node, uint64_t members,
+                             int depth, int lane, uint32_t &nodes_read, uint32_t &edges_scored) {
+    const size_t nrow = (size_t)tree * g.max_nodes + node;
+    Edge *row = g.edges + nrow * kEdges;
+    // the first 64 edges are requested together with the node's own word, before anything about the node is known
+    const Edge first = load_edge(row + lane);
+    const NodeInfo ni = load_info(g.info + nrow);
+    const int expanded = ni.expanded;
+    nodes_read += 1;
+    if (expanded == PUCT_NODE_EXPANDED_TERMINAL || depth >= g.path_depth) {
+        const int kind = expanded == PUCT_NODE_EXPANDED_TERMINAL ? PUCT_SELECT_TERMINAL : PUCT_SELECT_DEPTH_LIMIT;
+        if (lane < kTrav && ((members >> lane) & 1ull)) {
+            s.sel[lane] = pack_sel(kind, node, 0);
+            s.len[lane] = depth + 1;
+            s.claims[lane] = depth;
+            next[lane] = -1;
+        }
+        return;
+    }
+    edges_scored += (uint32_t)expanded;
+
+    float q[kSlices], cp[kSlices];
+    int den[kSlices];
+    uint32_t link[kSlices], link_loaded[kSlices];
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < kSlices; ++i) {
+        const int eid = lane + i * kWave;
+        Edge e = first;
+        if (i > 0) {
+            e = Edge{0, 0.0f, 0.0f, 0u};
+            if (i * kWave < expanded) e = load_edge(row + eid);
+        }
+        const bool valid = eid < expanded;
+        q[i] = valid && e.n > 0 ? e.w / (float)e.n : 0.0f;
+        cp[i] = g.cpuct * e.prior;
+        link[i] = link_loaded[i] = e.link;
+        den[i] = e.n + (int)(e.link & 0xFFu) + 1;
+        total += valid ? den[i] - 1 : 0;
+    }
+    total = wave_sum(total);
+    int tickets = ni.tickets;
+    const int legal = ni.legal_turn & 0xFFFF;
+
+    for (uint64_t rest = members; rest != 0; rest &= rest - 1) {
+        const int j = __builtin_ctzll(rest);   // the traversal deciding now
+        int parent_eff = 1, allowed = 1;
+        if (expanded != 1 || g.c_pw != 0.0f) {
+            parent_eff = total > 1 ? total : 1;
+            allowed = allowed_children(g.c_pw, g.alpha_pw, parent_eff, legal);
+        }
+        if (allowed > expanded) {
+            if (expanded + tickets < allowed) {   // expansion ticket
+                if (lane == 0) {
+                    s.sel[j] = pack_sel(PUCT_SELECT_EXPAND, node, expanded + tickets);
+                    s.len[j] = depth + 1;
+                    s.claims[j] = depth;
+                    next[j] = -1;
+                }
+                tickets += 1;
+                continue;
+            }
+            if (expanded == 0) {   // the node's only allowed child is being created by another traversal
+                if (lane == 0) {
+                    s.sel[j] = pack_sel(PUCT_SELECT_BUSY, node, 0);
+                    s.len[j] = 0;
+                    s.claims[j] = depth;
+                    next[j] = -1;
+                }
+                continue;
+            }
+        }
+        int best = 0;
+        if (expanded > 1) {
+            int tie_offset = j;
+            if (tie_offset >= expanded) tie_offset %= expanded;
+            const float sqrt_parent = sqrtf((float)parent_eff);
+            uint64_t key = 0;
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) {
+                const int eid = lane + i * kWave;
+                if (i * kWave < expanded && eid < expanded) {
+                    const float score = q[i] + cp[i] * sqrt_parent / (float)den[i];
+                    const uint64_t k = candidate_key(score, eid, tie_offset, expanded);
+                    key = k > key ? k : key;
+                }
+            }
+            const uint64_t top = wave_max(key);
+            best = top == 0 ? kNoEdge : (int)(top & 0xFFFFu);
+        }
+        const int best_lane = best & (kWave - 1), best_slice = best >> 6;
+        int child = 0;
+        if (best != kNoEdge) {
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i)
+                if (best_slice == i) child = (int)((uint32_t)__builtin_amdgcn_readlane((int)link[i], best_lane) >> 8);
+        }
+        if (child <= 0 || child >= g.max_nodes) {   // no edge with a comparable score, or a link that leads nowhere
+            if (lane == 0) {
+                s.sel[j] = pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
+                s.len[j] = 0;
+                s.claims[j] = depth;
+                next[j] = -1;
+            }
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < kSlices; ++i)
+            if (best_slice == i && lane == best_lane) {
+                den[i] += 1;
+                link[i] += 1u;
+            }
+        total += 1;
+        if (lane == 0) {
+            paths[j * g.path_depth + depth] = (node << 8) | best;
+            next[j] = child;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kSlices; ++i)
+        if (link[i] != link_loaded[i]) row[lane + i * kWave].link = link[i];
+    if (lane == 0 && tickets != ni.tickets) g.info[nrow].tickets = tickets;
+}
+
+// Selection of one step for the traversals of one tree; all wavefronts of the workgroup call it.  Ends behind a
+// workgroup barrier with every traversal's result in `s` and its path in `paths`.
+__device__ void select_phase(const LoopArgs &g, StepLds &s, int *paths, int tree, int wave, int lane, int n_waves,
+                             uint32_t &nodes_read, uint32_t &edges_scored) {
+    if (threadIdx.x < kTrav) {
+        const int t = threadIdx.x;
+        s.cur[0][t] = t < n_waves ? 0 : -1;
+        s.cur[1][t] = -1;
+        s.sel[t] = pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
+        s.len[t] = 0;
+        s.claims[t] = 0;
+        s.value[t] = 0.0f;
+    }
+    __syncthreads();
+    for (int depth = 0;; ++depth) {
+        const int *cur = s.cur[depth & 1];
+        int *next = s.cur[(depth & 1) ^ 1];
+        const int at = lane < kTrav ? cur[lane] : -1;
+        if (__ballot(at >= 0) == 0) break;   // every wavefront reads the same words: all leave together
+        const int mine = __builtin_amdgcn_readlane(at, wave);
+        const uint64_t members = __ballot(at >= 0 && at == mine);
+        if (mine < 0) {
+            if (lane == 0) next[wave] = -1;
+        } else if ((members & lanes_below(wave)) == 0) {
+            select_group(g, s, paths, next, tree, mine, members, depth, lane, nodes_read, edges_scored);
+        }
+        __syncthreads();
     }
 }
 
-// Expansion / evaluation of one step for the traversals of one tree; all wavefronts of the workgroup call it.
-// Children get consecutive node ids in traversal order; when the tree cannot take all expansions of a step none is
-// committed (those traversals evaluate the node they reached instead).
-__device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, int lane, int n_waves) {
-    const size_t out = (size_t)tree * g.sel.warps + wave;
-    const int raw = g.sel.out_selected_node[out];
-    const int kind = (raw >> PUCT_PACKED_KIND_SHIFT) & PUCT_PACKED_KIND_MASK;
-    const int node = raw & PUCT_PACKED_NODE_MASK, ticket_slot = (raw >> PUCT_PACKED_SLOT_SHIFT) & PUCT_PACKED_EDGE_MASK;
-    const int plen = g.sel.out_path_len[out];
-    const size_t trow = (size_t)tree * g.sel.nodes;
+// ---- expansion / evaluation -----------------------------------------------------------------------------------------
+// Every wavefront handles the leaf of its own traversal.  Children get consecutive node ids in traversal order and go
+// into the node's next free edge slots in traversal order (the expanded edges of a node stay contiguous whatever the
+// tickets say); when the tree cannot take all expansions of a step none is committed (those traversals evaluate the
+// node they reached instead).
+__device__ void expand_phase(const LoopArgs &g, StepLds &s, int tree, int wave, int lane, int n_waves, uint32_t &created) {
+    const int raw = s.sel[wave];
+    const int kind = (raw >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7;
+    const int node = raw & PUCT_GOMOKU_SEL_NODE_MASK, ticket_slot = (raw >> PUCT_GOMOKU_SEL_SLOT_SHIFT) & 0xFF;
+    const size_t trow = (size_t)tree * g.max_nodes;
     const uint64_t tree_seed = psyn_tree_seed(g.seed, tree);
     const bool has_node = kind == PUCT_SELECT_EXPAND || kind == PUCT_SELECT_TERMINAL || kind == PUCT_SELECT_DEPTH_LIMIT;
-    uint32_t *board = lds.board[wave];
-    int n_legal = 0, turn = 0;
+    uint32_t *board = s.board[wave];
+    NodeInfo ni{0, 0, 0, 0.0f};
     if (has_node) {
-        const uint32_t w = lane < kBoardWords ? g.node_board[(trow + node) * kBoardWords + lane] : 0u;
+        const uint32_t w = lane < kBoardWords ? g.board[(trow + node) * kBoardWords + lane] : 0u;
+        ni = load_info(g.info + trow + node);
         if (lane < kBoardWords) board[lane] = w;
-        n_legal = g.cells - wave_sum(__popc(w));
-        turn = g.node_turn[trow + node];
         wave_lds_fence();
     }
-    const int wants = (kind == PUCT_SELECT_EXPAND && ticket_slot < n_legal) ? 1 : 0;
-    if (lane == 0) {
-        lds.want[wave] = wants;
-        atomicAdd(&g.tally[(size_t)tree * 8 + kind], 1ull);
-    }
+    const int n_legal = ni.legal_turn & 0xFFFF, turn = (ni.legal_turn & kTurnBit) ? -1 : 1;
+    const bool wants = kind == PUCT_SELECT_EXPAND && ticket_slot < n_legal;
+    if (lane == 0) s.want[wave] = wants ? node : -1;
     __syncthreads();
-    int total = 0, before = 0;
-    for (int w = 0; w < n_waves; ++w) {
-        total += lds.want[w];
-        before += w < wave ? lds.want[w] : 0;
-    }
-    const int base = load_relaxed(g.node_count + tree);
+    const int other = lane < n_waves ? s.want[lane] : -1;
+    const uint64_t all = __ballot(other >= 0), here = __ballot(other >= 0 && other == node);
+    const int total = __popcll(all), before = __popcll(all & lanes_below(wave));
+    const int rank = __popcll(here & lanes_below(wave)), siblings = __popcll(here);
+    const int base = s.node_count;
     const bool fits = base + total <= g.max_nodes;
     __syncthreads();
-    if (wave == 0 && lane == 0 && fits && total > 0) {
-        g.node_count[tree] = base + total;
-        atomicAdd(&g.tally[(size_t)tree * 8 + 5], (unsigned long long)total);
-    }
+    if (wave == 0 && lane == 0 && fits) s.node_count = base + total;
+    if (wave == 0 && fits) created += (uint32_t)total;
 
-    float u = 0.0f;   // value of the reached node for its player to move
+    float u = 0.0f;   // value of the reached node for the player who moved into it
     if (wants && fits) {
-        const int child = base + before;
+        const int child = base + before, slot = ni.expanded + rank;
         const size_t erow = (trow + node) * kEdges;
-        // The edge slot the child goes into is the node's next free one, taken here, not the slot of the selection's
-        // ticket: tickets of one step can leave a hole (a traversal whose widening limit, computed from visit counts
-        // that include other traversals' virtual losses, is smaller gives its ticket back while one with a larger limit
-        // has already drawn the next), and the expanded edges of a node must stay contiguous.  With one traversal per
-        // tree the two are the same slot.
-        int slot_taken = 0;
-        if (lane == 0) slot_taken = atomicAdd(&g.node_expanded[trow + node], 1);
-        const int slot = __builtin_amdgcn_readfirstlane(slot_taken);
-        const int action = g.edge_action[erow + slot];
+        const int action = g.action[erow + slot];
         uint32_t *mine = board + (turn > 0 ? 0 : 8);
         if (lane == 0) mine[action >> 5] |= 1u << (action & 31);
         wave_lds_fence();
@@ -239,63 +425,133 @@ __device__ void expand_phase(const GomokuArgs &g, Lds &lds, int tree, int wave, 
         const bool terminal = win || child_legal == 0;
         const uint64_t bh = psyn_board_hash(tree_seed, board);
         const float v_child = win ? -1.0f : (terminal ? 0.0f : psyn_value(bh));
-        if (lane < kBoardWords) g.node_board[(trow + child) * kBoardWords + lane] = board[lane];
+        if (lane < kBoardWords) g.board[(trow + child) * kBoardWords + lane] = board[lane];
         if (lane == 0) {
-            g.node_turn[trow + child] = (int8_t)-turn;
-            g.node_value[trow + child] = v_child;
-            g.node_expanded[trow + child] = terminal ? PUCT_NODE_EXPANDED_TERMINAL : 0;
-            g.node_expand_inflight[trow + child] = 0;
-            g.node_legal[trow + child] = child_legal;
-            g.edge_child[erow + slot] = child;
-            g.edge_N[erow + slot] = 1;
-            g.edge_W[erow + slot] = -v_child;
+            *reinterpret_cast<uint4 *>(g.info + trow + child) =
+                make_uint4((uint32_t)(terminal ? PUCT_NODE_EXPANDED_TERMINAL : 0), 0u,
+                           (uint32_t)(child_legal | (turn > 0 ? kTurnBit : 0)), __float_as_uint(v_child));
+            Edge *e = g.edges + erow + slot;
+            e->n = 1;
+            e->w = -v_child;
+            e->link = (uint32_t)child << 8;
+            if (rank == 0) g.info[trow + node].expanded = ni.expanded + siblings;
         }
         if (!terminal) write_priors(g, tree, child, board, lane, bh, child_legal);
         u = -v_child;
     } else if (kind == PUCT_SELECT_TERMINAL) {
-        u = g.node_value[trow + node];
+        u = ni.value;
     } else if (has_node) {
         u = psyn_value(psyn_board_hash(tree_seed, board));
     }
-    if (has_node) {
-        // edge d was played by the player to move at depth d; the reached node sits at depth L
-        const int L = plen - 1;
-        for (int d = lane; d < L; d += kWave) g.path_values[out * g.sel.path_depth + d] = ((L - d) & 1) ? -u : u;
+    if (lane == 0) s.value[wave] = u;
+}
+
+// ---- backup ----------------------------------------------------------------------------------------------------------
+// Every traversal gives back the claims along its path; one that reached a node (expansion, terminal, depth limit) also
+// leaves a visit and the node's value, sign alternating, on every edge of the path (src/puct/puct_gpu_v2.py:847-927
+// moved to edge-level virtual loss), and an expansion returns its ticket.  Lane = (traversal, one of four depths): the
+// traversals whose paths share an edge at that depth meet inside a row of 16 lanes, and the last of them stores the
+// edge after adding the values in traversal order, so the float sums do not depend on timing.
+__device__ void backup_phase(const LoopArgs &g, StepLds &s, const int *paths, int tree, int wave, int lane, int n_waves) {
+    const size_t trow = (size_t)tree * g.max_nodes;
+    const int t = lane & (kTrav - 1), sub = lane >> 4;
+    const int raw = s.sel[t], my_claims = s.claims[t];
+    const int kind = (raw >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7;
+    const int counted = (kind == PUCT_SELECT_EXPAND || kind == PUCT_SELECT_TERMINAL || kind == PUCT_SELECT_DEPTH_LIMIT) ? 1 : 0;
+    const float u = s.value[t];
+    int deepest = 0;
+    for (int j = 0; j < n_waves; ++j) deepest = s.claims[j] > deepest ? s.claims[j] : deepest;
+    for (int d0 = 4 * wave; d0 < deepest; d0 += 4 * n_waves) {
+        const int d = d0 + sub;
+        const int enc = d < my_claims ? paths[t * g.path_depth + d] : -1;
+        const float val = ((my_claims - d) & 1) ? -u : u;   // a counted traversal's path has as many edges as claims
+        Edge *e = nullptr;
+        int n_old = 0;
+        float acc = 0.0f;
+        uint32_t link_old = 0;
+        if (enc >= 0) {
+            e = g.edges + (trow + (enc >> 8)) * kEdges + (enc & 0xFF);
+            n_old = e->n;
+            acc = e->w;
+            link_old = e->link;
+        }
+        int visits = 0, released = 0;
+        bool last = true;
+#pragma unroll
+        for (int j = 0; j < kTrav; ++j) {
+            const int src = ((lane & ~(kTrav - 1)) | j) << 2;
+            const int enc_j = __builtin_amdgcn_ds_bpermute(src, enc);
+            const float val_j = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(val)));
+            const int counted_j = __builtin_amdgcn_ds_bpermute(src, counted);
+            const bool same = enc >= 0 && enc_j == enc;
+            if (same && j <= t) {
+                released += 1;
+                if (counted_j) {
+                    acc += val_j;
+                    visits += 1;
+                }
+            }
+            if (same && j > t) last = false;
+        }
+        if (enc >= 0 && last) {
+            e->n = n_old + visits;
+            e->w = acc;
+            e->link = link_old - (uint32_t)released;
+        }
+    }
+    if (wave == 0) {   // expansion tickets back, once per node
+        const int sel_l = lane < n_waves ? s.sel[lane] : 0;
+        const bool is_exp = lane < n_waves && ((sel_l >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7) == PUCT_SELECT_EXPAND;
+        const int node_l = sel_l & PUCT_GOMOKU_SEL_NODE_MASK;
+        int returned = 0;
+        bool first = true;
+        for (int j = 0; j < n_waves; ++j) {
+            const int node_j = __builtin_amdgcn_readlane(node_l, j);
+            const bool exp_j = (__ballot(is_exp) >> j) & 1ull;
+            if (exp_j && node_j == node_l) {
+                returned += 1;
+                if (j < lane) first = false;
+            }
+        }
+        if (is_exp && first) g.info[trow + node_l].tickets -= returned;
     }
 }
 
 // Root of every tree: node 0 with the root position and its priors.
-__global__ __launch_bounds__(kWave) void init_kernel(const GomokuArgs g, const uint32_t *root_board, int root_turn) {
+__global__ __launch_bounds__(kWave) void init_kernel(const LoopArgs g, const uint32_t *root_board, int root_turn) {
     __shared__ uint32_t board[kBoardWords];
     const int tree = blockIdx.x, lane = threadIdx.x;
-    const size_t trow = (size_t)tree * g.sel.nodes;
+    const size_t trow = (size_t)tree * g.max_nodes;
     const uint32_t w = lane < kBoardWords ? root_board[lane] : 0u;
     if (lane < kBoardWords) {
         board[lane] = w;
-        g.node_board[trow * kBoardWords + lane] = w;
+        g.board[trow * kBoardWords + lane] = w;
     }
     const int n_legal = g.cells - wave_sum(__popc(w));
     wave_lds_fence();
     if (lane < 8) g.tally[(size_t)tree * 8 + lane] = 0ull;
+    if (lane < g.traversals) {
+        const size_t out = (size_t)tree * g.traversals + lane;
+        g.out_selected[out] = pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
+        g.out_len[out] = 0;
+        g.out_claims[out] = 0;
+        g.out_value[out] = 0.0f;
+    }
     if (lane == 0) {
-        g.node_turn[trow] = (int8_t)root_turn;
-        g.node_value[trow] = 0.0f;
-        g.node_expanded[trow] = n_legal == 0 ? PUCT_NODE_EXPANDED_TERMINAL : 0;
-        g.node_expand_inflight[trow] = 0;
-        g.node_legal[trow] = n_legal;
+        *reinterpret_cast<uint4 *>(g.info + trow) =
+            make_uint4((uint32_t)(n_legal == 0 ? PUCT_NODE_EXPANDED_TERMINAL : 0), 0u,
+                       (uint32_t)(n_legal | (root_turn > 0 ? 0 : kTurnBit)), 0u);
         g.node_count[tree] = 1;
     }
     if (n_legal > 0) write_priors(g, tree, 0, board, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
 }
 
-// Makes the writes of a phase (plain stores and atomics) visible to the loads of the next one.  All wavefronts of a
-// tree run on one CU and share its write-through L1 and the L2 behind it, so no L2 write-back is needed; what is needed
-// is (1) that every wavefront's stores and atomics of the phase have been acknowledged by the L2 before any wavefront
-// goes on -- a workgroup-scope release fence does not wait for that on one CU (it lowers to no vector-memory wait), and a
-// counter that another wavefront changed with a fire-and-forget atomic could otherwise still be read with its old value
-// after the barrier -- hence the explicit wait on the wavefront's own outstanding vector memory operations; and (2) that
-// the L1 drops the lines which device-scope atomics of other wavefronts have changed underneath it: the agent-scope
-// acquire.
+// Makes the stores of a phase visible to the loads of the next one.  All wavefronts of a tree run on one CU and share
+// its write-through L1 and the L2 behind it, so no L2 write-back is needed; what is needed is (1) that every
+// wavefront's stores of the phase have been acknowledged by the L2 before any wavefront goes on -- a workgroup-scope
+// release fence does not wait for that on one CU (it lowers to no vector-memory wait) -- hence the explicit wait on the
+// wavefront's own outstanding vector memory operations; and (2) that the L1 drops the lines which other wavefronts have
+// changed underneath it: the agent-scope acquire.
 __device__ __forceinline__ void phase_barrier() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -303,29 +559,142 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void search_kernel(const GomokuArgs g) {
-    __shared__ Lds lds;
-    const int tree = blockIdx.x, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-    const int n_waves = blockDim.x / kWave;
-    for (int step = 0; step < g.steps; ++step) {
-        select_traversal(g.sel, tree, wave, lane);
-        phase_barrier();
-        expand_phase(g, lds, tree, wave, lane, n_waves);
-        phase_barrier();
-        backup_traversal<false>(g.bk, tree, wave, lane);
-        phase_barrier();
+// What the traversals of a step ended with, between the launches of the stepwise mode and for the host to read.
+__device__ void state_to_memory(const LoopArgs &g, const StepLds &s, const int *paths, int tree, int n_waves) {
+    const size_t out = (size_t)tree * g.traversals;
+    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += blockDim.x) {
+        const int t = i / g.path_depth, d = i - t * g.path_depth;
+        g.out_path[out * g.path_depth + i] = d < s.claims[t] ? paths[i] : -1;
     }
+    if (threadIdx.x < n_waves) {
+        const int t = threadIdx.x;
+        g.out_selected[out + t] = s.sel[t];
+        g.out_len[out + t] = s.len[t];
+        g.out_claims[out + t] = s.claims[t];
+        g.out_value[out + t] = s.value[t];
+    }
+    if (threadIdx.x == 0) g.node_count[tree] = s.node_count;
+}
+__device__ void state_from_memory(const LoopArgs &g, StepLds &s, int *paths, int tree, int n_waves) {
+    const size_t out = (size_t)tree * g.traversals;
+    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += blockDim.x) paths[i] = g.out_path[out * g.path_depth + i];
+    if (threadIdx.x < kTrav) {
+        const int t = threadIdx.x;
+        const bool live = t < n_waves;
+        s.sel[t] = live ? g.out_selected[out + t] : pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
+        s.len[t] = live ? g.out_len[out + t] : 0;
+        s.claims[t] = live ? g.out_claims[out + t] : 0;
+        s.value[t] = live ? g.out_value[out + t] : 0.0f;
+    }
+    if (threadIdx.x == 0) s.node_count = g.node_count[tree];
+    __syncthreads();
 }
 
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_step_kernel(const GomokuArgs g) {
-    select_traversal(g.sel, blockIdx.x, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+struct Work {
+    uint32_t kinds[5] = {0, 0, 0, 0, 0}, created = 0, nodes_read = 0, edges_scored = 0;
+    __device__ void count_kind(const StepLds &s, int wave) {
+        const int kind = (s.sel[wave] >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7;
+#pragma unroll
+        for (int k = 0; k < 5; ++k) kinds[k] += kind == k ? 1u : 0u;
+    }
+    __device__ void to_memory(const LoopArgs &g, int tree, int lane) const {
+        if (lane != 0) return;
+        unsigned long long *row = g.tally + (size_t)tree * 8;
+#pragma unroll
+        for (int k = 0; k < 5; ++k)
+            if (kinds[k]) atomicAdd(row + k, (unsigned long long)kinds[k]);
+        if (created) atomicAdd(row + 5, (unsigned long long)created);
+        if (nodes_read) atomicAdd(row + 6, (unsigned long long)nodes_read);
+        if (edges_scored) atomicAdd(row + 7, (unsigned long long)edges_scored);
+    }
+};
+
+extern __shared__ int dynamic_lds[];
+
+// The whole search of one tree in one launch: one workgroup per tree, one wavefront per traversal.
+__global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g) {
+    __shared__ StepLds s;
+    int *paths = dynamic_lds;
+    const int tree = blockIdx.x, lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
+    Work work;
+    if (threadIdx.x == 0) s.node_count = g.node_count[tree];
+    __syncthreads();
+    for (int step = 0; step < g.steps; ++step) {
+        select_phase(g, s, paths, tree, wave, lane, n_waves, work.nodes_read, work.edges_scored);
+        work.count_kind(s, wave);
+        expand_phase(g, s, tree, wave, lane, n_waves, work.created);
+        phase_barrier();   // the claims of the selection and the new edges are in memory
+        backup_phase(g, s, paths, tree, wave, lane, n_waves);
+        phase_barrier();
+    }
+    state_to_memory(g, s, paths, tree, n_waves);
+    work.to_memory(g, tree, lane);
 }
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void expand_step_kernel(const GomokuArgs g) {
-    __shared__ Lds lds;
-    expand_phase(g, lds, blockIdx.x, threadIdx.x / kWave, threadIdx.x & (kWave - 1), blockDim.x / kWave);
+
+__global__ __launch_bounds__(kTrav *kWave) void select_step_kernel(const LoopArgs g) {
+    __shared__ StepLds s;
+    int *paths = dynamic_lds;
+    const int tree = blockIdx.x, lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
+    Work work;
+    if (threadIdx.x == 0) s.node_count = g.node_count[tree];
+    select_phase(g, s, paths, tree, wave, lane, n_waves, work.nodes_read, work.edges_scored);
+    work.count_kind(s, wave);
+    state_to_memory(g, s, paths, tree, n_waves);
+    work.to_memory(g, tree, lane);
 }
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_step_kernel(const GomokuArgs g) {
-    backup_traversal<false>(g.bk, blockIdx.x, threadIdx.x / kWave, threadIdx.x & (kWave - 1));
+__global__ __launch_bounds__(kTrav *kWave) void expand_step_kernel(const LoopArgs g) {
+    __shared__ StepLds s;
+    int *paths = dynamic_lds;
+    const int tree = blockIdx.x, lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
+    Work work;
+    state_from_memory(g, s, paths, tree, n_waves);
+    expand_phase(g, s, tree, wave, lane, n_waves, work.created);
+    __syncthreads();
+    state_to_memory(g, s, paths, tree, n_waves);
+    work.to_memory(g, tree, lane);
+}
+__global__ __launch_bounds__(kTrav *kWave) void backup_step_kernel(const LoopArgs g) {
+    __shared__ StepLds s;
+    int *paths = dynamic_lds;
+    const int tree = blockIdx.x, lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
+    state_from_memory(g, s, paths, tree, n_waves);
+    backup_phase(g, s, paths, tree, wave, lane, n_waves);
+}
+
+// ---- the arrays as the host reads them -------------------------------------------------------------------------------
+// One element of array `id` (include/puct_gomoku.h) per thread, written in the [trees, nodes, edges] / [trees, nodes]
+// shapes of the selection and backup launchers' arrays.
+__global__ void unpack_kernel(const LoopArgs g, int trees, int id, void *dst, size_t count) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    switch (id) {
+    case PUCT_GOMOKU_ARR_EDGE_CHILD: {
+        const int child = (int)(g.edges[i].link >> 8);
+        static_cast<int *>(dst)[i] = child > 0 ? child : -1;
+        break;
+    }
+    case PUCT_GOMOKU_ARR_EDGE_PRIOR: static_cast<float *>(dst)[i] = g.edges[i].prior; break;
+    case PUCT_GOMOKU_ARR_EDGE_W: static_cast<float *>(dst)[i] = g.edges[i].w; break;
+    case PUCT_GOMOKU_ARR_EDGE_N: static_cast<int *>(dst)[i] = g.edges[i].n; break;
+    case PUCT_GOMOKU_ARR_EDGE_INFLIGHT: static_cast<int *>(dst)[i] = (int)(g.edges[i].link & 0xFFu); break;
+    case PUCT_GOMOKU_ARR_NODE_EXPANDED: static_cast<int *>(dst)[i] = g.info[i].expanded; break;
+    case PUCT_GOMOKU_ARR_NODE_EXPAND_INFLIGHT: static_cast<int *>(dst)[i] = g.info[i].tickets; break;
+    case PUCT_GOMOKU_ARR_NODE_TURN: static_cast<int8_t *>(dst)[i] = (g.info[i].legal_turn & kTurnBit) ? -1 : 1; break;
+    case PUCT_GOMOKU_ARR_NODE_VALUE: static_cast<float *>(dst)[i] = g.info[i].value; break;
+    case PUCT_GOMOKU_ARR_NODE_LEGAL: static_cast<int *>(dst)[i] = g.info[i].legal_turn & 0xFFFF; break;
+    case PUCT_GOMOKU_ARR_PATH_VALUES: {
+        const size_t out = i / g.path_depth;
+        const int d = (int)(i - out * g.path_depth), edges_on_path = g.out_len[out] - 1;
+        const float u = g.out_value[out];
+        static_cast<float *>(dst)[i] = d < edges_on_path ? (((edges_on_path - d) & 1) ? -u : u) : 0.0f;
+        break;
+    }
+    default: break;
+    }
 }
 
 // ---- host engine -----------------------------------------------------------------------------------------------------
@@ -353,24 +722,39 @@ double now_s() { return std::chrono::duration<double>(std::chrono::steady_clock:
 
 struct puct_gomoku_engine {
     puct_gomoku_config cfg;
-    GomokuArgs args;
+    LoopArgs args;
     uint32_t *d_root = nullptr;
     std::vector<void *> allocations;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    struct Array { void *ptr; size_t bytes; };
-    Array arrays[17];
 };
 
 namespace {
 template <typename T>
-int alloc(puct_gomoku_engine *e, T **out, size_t count, int array_id) {
+int alloc(puct_gomoku_engine *e, T **out, size_t count) {
     void *p = nullptr;
     HIP_TRY(hipMalloc(&p, sizeof(T) * count));
     e->allocations.push_back(p);
     *out = static_cast<T *>(p);
-    if (array_id >= 0) e->arrays[array_id] = {p, sizeof(T) * count};
     return PUCT_GOMOKU_OK;
+}
+
+// Element size and count of array `id`, 0 if there is no such array.
+size_t array_shape(const puct_gomoku_config &c, int id, size_t *count) {
+    const size_t T = c.trees, N = c.max_nodes, W = c.traversals, D = c.path_depth;
+    switch (id) {
+    case PUCT_GOMOKU_ARR_EDGE_CHILD: case PUCT_GOMOKU_ARR_EDGE_PRIOR: case PUCT_GOMOKU_ARR_EDGE_W:
+    case PUCT_GOMOKU_ARR_EDGE_N: case PUCT_GOMOKU_ARR_EDGE_INFLIGHT: *count = T * N * kEdges; return 4;
+    case PUCT_GOMOKU_ARR_EDGE_ACTION: *count = T * N * kEdges; return 1;
+    case PUCT_GOMOKU_ARR_NODE_EXPANDED: case PUCT_GOMOKU_ARR_NODE_EXPAND_INFLIGHT: case PUCT_GOMOKU_ARR_NODE_VALUE:
+    case PUCT_GOMOKU_ARR_NODE_LEGAL: *count = T * N; return 4;
+    case PUCT_GOMOKU_ARR_NODE_TURN: *count = T * N; return 1;
+    case PUCT_GOMOKU_ARR_NODE_COUNT: *count = T; return 4;
+    case PUCT_GOMOKU_ARR_NODE_BOARD: *count = T * N * kBoardWords; return 4;
+    case PUCT_GOMOKU_ARR_OUT_SELECTED: case PUCT_GOMOKU_ARR_OUT_LEN: *count = T * W; return 4;
+    case PUCT_GOMOKU_ARR_OUT_PATH: case PUCT_GOMOKU_ARR_PATH_VALUES: *count = T * W * D; return 4;
+    default: *count = 0; return 0;
+    }
 }
 }  // namespace
 
@@ -392,51 +776,36 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     if (c->board_m < 1 || c->board_n < 1 || c->board_m * c->board_n > kEdges)
         return fail(PUCT_GOMOKU_E_INVALID, "board %dx%d: need 1 <= m * n <= %d", c->board_m, c->board_n, kEdges);
     if (c->trees < 1) return fail(PUCT_GOMOKU_E_INVALID, "trees = %d, need >= 1", c->trees);
-    if (c->traversals < 1 || c->traversals > kMaxWavesPerBlock)
-        return fail(PUCT_GOMOKU_E_INVALID, "traversals = %d, need 1..%d", c->traversals, kMaxWavesPerBlock);
-    if (c->max_nodes < 2 || c->max_nodes > PUCT_PACKED_NODE_LIMIT)
-        return fail(PUCT_GOMOKU_E_INVALID, "max_nodes = %d, need 2..%d", c->max_nodes, PUCT_PACKED_NODE_LIMIT);
-    if (c->path_depth < 1 || c->path_depth > 1024) return fail(PUCT_GOMOKU_E_INVALID, "path_depth = %d, need 1..1024", c->path_depth);
+    if (c->traversals < 1 || c->traversals > kTrav)
+        return fail(PUCT_GOMOKU_E_INVALID, "traversals = %d, need 1..%d", c->traversals, kTrav);
+    if (c->max_nodes < 2 || c->max_nodes > PUCT_GOMOKU_MAX_NODES)
+        return fail(PUCT_GOMOKU_E_INVALID, "max_nodes = %d, need 2..%d", c->max_nodes, PUCT_GOMOKU_MAX_NODES);
+    if (c->path_depth < 1 || c->path_depth > PUCT_GOMOKU_MAX_PATH_DEPTH)
+        return fail(PUCT_GOMOKU_E_INVALID, "path_depth = %d, need 1..%d", c->path_depth, PUCT_GOMOKU_MAX_PATH_DEPTH);
     if (!(c->dirichlet_alpha > 0.0f && c->dirichlet_alpha < 1.0f))
         return fail(PUCT_GOMOKU_E_INVALID, "dirichlet_alpha = %g, need 0 < alpha < 1", (double)c->dirichlet_alpha);
-    if (c->recalc_attempts < 0 || c->recalc_attempts > 64) return fail(PUCT_GOMOKU_E_INVALID, "recalc_attempts = %d, need 0..64", c->recalc_attempts);
     if (!(c->cpuct >= 0.0f) || !(c->c_pw >= 0.0f)) return fail(PUCT_GOMOKU_E_INVALID, "cpuct and c_pw must not be negative");
     HIP_TRY(hipSetDevice(c->device));
     auto *e = new puct_gomoku_engine();
     e->cfg = *c;
-    memset(e->arrays, 0, sizeof e->arrays);
-    const size_t T = c->trees, N = c->max_nodes, E = kEdges, W = c->traversals, D = c->path_depth;
-    GomokuArgs &g = e->args;
-    int *out_selected, *out_path, *out_len;
+    const size_t T = c->trees, N = c->max_nodes, W = c->traversals, D = c->path_depth;
+    LoopArgs &g = e->args;
     int rc = 0;
-    if ((rc = alloc(e, &g.edge_child, T * N * E, PUCT_GOMOKU_ARR_EDGE_CHILD)) || (rc = alloc(e, &g.edge_prior, T * N * E, PUCT_GOMOKU_ARR_EDGE_PRIOR)) ||
-        (rc = alloc(e, &g.edge_W, T * N * E, PUCT_GOMOKU_ARR_EDGE_W)) || (rc = alloc(e, &g.edge_N, T * N * E, PUCT_GOMOKU_ARR_EDGE_N)) ||
-        (rc = alloc(e, &g.edge_inflight, T * N * E, PUCT_GOMOKU_ARR_EDGE_INFLIGHT)) ||
-        (rc = alloc(e, &g.edge_action, T * N * E, PUCT_GOMOKU_ARR_EDGE_ACTION)) ||
-        (rc = alloc(e, &g.node_expanded, T * N, PUCT_GOMOKU_ARR_NODE_EXPANDED)) ||
-        (rc = alloc(e, &g.node_expand_inflight, T * N, PUCT_GOMOKU_ARR_NODE_EXPAND_INFLIGHT)) ||
-        (rc = alloc(e, &g.node_count, T, PUCT_GOMOKU_ARR_NODE_COUNT)) || (rc = alloc(e, &g.node_board, T * N * kBoardWords, PUCT_GOMOKU_ARR_NODE_BOARD)) ||
-        (rc = alloc(e, &g.node_turn, T * N, PUCT_GOMOKU_ARR_NODE_TURN)) || (rc = alloc(e, &g.node_value, T * N, PUCT_GOMOKU_ARR_NODE_VALUE)) ||
-        (rc = alloc(e, &out_selected, T * W, PUCT_GOMOKU_ARR_OUT_SELECTED)) || (rc = alloc(e, &out_path, T * W * D, PUCT_GOMOKU_ARR_OUT_PATH)) ||
-        (rc = alloc(e, &out_len, T * W, PUCT_GOMOKU_ARR_OUT_LEN)) || (rc = alloc(e, &g.path_values, T * W * D, PUCT_GOMOKU_ARR_PATH_VALUES)) ||
-        (rc = alloc(e, &g.node_legal, T * N, PUCT_GOMOKU_ARR_NODE_LEGAL)) || (rc = alloc(e, &g.tally, T * 8, -1)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords, -1))) {
+    if ((rc = alloc(e, &g.edges, T * N * kEdges)) || (rc = alloc(e, &g.info, T * N)) || (rc = alloc(e, &g.board, T * N * kBoardWords)) ||
+        (rc = alloc(e, &g.action, T * N * kEdges)) || (rc = alloc(e, &g.node_count, T)) || (rc = alloc(e, &g.out_selected, T * W)) ||
+        (rc = alloc(e, &g.out_len, T * W)) || (rc = alloc(e, &g.out_claims, T * W)) || (rc = alloc(e, &g.out_path, T * W * D)) ||
+        (rc = alloc(e, &g.out_value, T * W)) || (rc = alloc(e, &g.tally, T * 8)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords))) {
         puct_gomoku_destroy(e);
         return rc;
     }
-    g.sel = SelectArgs{c->cpuct, c->c_pw, c->alpha_pw, c->soft_winner, g.edge_child, g.edge_prior, g.edge_W, g.edge_N, g.edge_inflight,
-                       g.node_expand_inflight, g.node_expanded, g.node_count, out_selected, out_path, out_len,
-                       c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth, g.node_legal,
-                       c->recalc_attempts > 0 ? c->recalc_attempts : kRecalcAttempts, g.tally};
-    g.bk = BackupArgs{1, nullptr, g.edge_W, g.edge_N, g.edge_inflight, nullptr, g.node_expand_inflight, g.node_count,
-                      out_selected, out_path, out_len, g.path_values, c->trees, c->max_nodes, kEdges, c->traversals, c->path_depth};
-    g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes; g.steps = 0;
+    g.cpuct = c->cpuct; g.c_pw = c->c_pw; g.alpha_pw = c->alpha_pw;
+    g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes;
+    g.traversals = c->traversals; g.path_depth = c->path_depth; g.steps = 0;
     g.seed = c->seed; g.dirichlet_alpha = (double)c->dirichlet_alpha;
     hipError_t err = hipStreamCreate(&e->stream);
     if (err == hipSuccess) err = hipEventCreate(&e->ev0);
     if (err == hipSuccess) err = hipEventCreate(&e->ev1);
-    // the paths and values of slots a step does not write must still be readable
-    if (err == hipSuccess) err = hipMemset(out_path, 0xFF, sizeof(int) * T * W * D);
-    if (err == hipSuccess) err = hipMemset(g.path_values, 0, sizeof(float) * T * W * D);
+    if (err == hipSuccess) err = hipMemset(g.out_path, 0xFF, sizeof(int) * T * W * D);
     if (err != hipSuccess) {
         puct_gomoku_destroy(e);
         return fail(PUCT_GOMOKU_E_HIP, "engine set-up failed: %s", hipGetErrorString(err));
@@ -463,24 +832,25 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
     if (empty == 0) return fail(PUCT_GOMOKU_E_ROOT, "the root position has no empty cell");
     const double t0 = now_s();
     HIP_TRY(hipSetDevice(c.device));
-    GomokuArgs g = e->args;
+    LoopArgs g = e->args;
     g.steps = steps;
     hipStream_t s = e->stream;
     HIP_TRY(hipMemcpyAsync(e->d_root, words, sizeof words, hipMemcpyHostToDevice, s));
     hipLaunchKernelGGL(init_kernel, dim3(c.trees), dim3(kWave), 0, s, g, e->d_root, (int)turn);
     HIP_TRY(hipGetLastError());
     const dim3 grid(c.trees), block(c.traversals * kWave);
+    const size_t lds = sizeof(int) * (size_t)c.traversals * c.path_depth;
     HIP_TRY(hipEventRecord(e->ev0, s));
     if (fused) {
         if (steps > 0) {
-            hipLaunchKernelGGL(search_kernel, grid, block, 0, s, g);
+            hipLaunchKernelGGL(search_kernel, grid, block, lds, s, g);
             HIP_TRY(hipGetLastError());
         }
     } else {
         for (int i = 0; i < steps; ++i) {
-            hipLaunchKernelGGL(select_step_kernel, grid, block, 0, s, g);
-            hipLaunchKernelGGL(expand_step_kernel, grid, block, 0, s, g);
-            hipLaunchKernelGGL(backup_step_kernel, grid, block, 0, s, g);
+            hipLaunchKernelGGL(select_step_kernel, grid, block, lds, s, g);
+            hipLaunchKernelGGL(expand_step_kernel, grid, block, lds, s, g);
+            hipLaunchKernelGGL(backup_step_kernel, grid, block, lds, s, g);
         }
         HIP_TRY(hipGetLastError());
     }
@@ -491,30 +861,28 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
 
     // root tables of all trees
     const size_t T = c.trees, N = c.max_nodes;
-    std::vector<int> n_root(T * kEdges), expanded(T), counts(T);
-    std::vector<float> w_root(T * kEdges);
+    std::vector<Edge> root_edges(T * kEdges);
+    std::vector<NodeInfo> root_info(T);
     std::vector<uint8_t> a_root(T * kEdges);
+    std::vector<int> counts(T);
     std::vector<unsigned long long> tally(T * 8);
-    for (size_t t = 0; t < T; ++t) {
-        HIP_TRY(hipMemcpy(n_root.data() + t * kEdges, g.edge_N + t * N * kEdges, sizeof(int) * kEdges, hipMemcpyDeviceToHost));
-        HIP_TRY(hipMemcpy(w_root.data() + t * kEdges, g.edge_W + t * N * kEdges, sizeof(float) * kEdges, hipMemcpyDeviceToHost));
-        HIP_TRY(hipMemcpy(a_root.data() + t * kEdges, g.edge_action + t * N * kEdges, kEdges, hipMemcpyDeviceToHost));
-        HIP_TRY(hipMemcpy(&expanded[t], g.node_expanded + t * N, sizeof(int), hipMemcpyDeviceToHost));
-    }
+    HIP_TRY(hipMemcpy2D(root_edges.data(), sizeof(Edge) * kEdges, g.edges, sizeof(Edge) * kEdges * N, sizeof(Edge) * kEdges, T, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy2D(root_info.data(), sizeof(NodeInfo), g.info, sizeof(NodeInfo) * N, sizeof(NodeInfo), T, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy2D(a_root.data(), kEdges, g.action, (size_t)kEdges * N, kEdges, T, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(counts.data(), g.node_count, sizeof(int) * T, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(tally.data(), g.tally, sizeof(unsigned long long) * T * 8, hipMemcpyDeviceToHost));
     memset(res, 0, sizeof *res);
     res->steps = steps;
     for (size_t t = 0; t < T; ++t) {
-        for (int sl = 0; sl < expanded[t] && sl < kEdges; ++sl) {
+        for (int sl = 0; sl < root_info[t].expanded && sl < kEdges; ++sl) {
             const int a = a_root[t * kEdges + sl];
-            res->root_n[a] += n_root[t * kEdges + sl];
-            res->root_w[a] += (double)w_root[t * kEdges + sl];
+            res->root_n[a] += root_edges[t * kEdges + sl].n;
+            res->root_w[a] += (double)root_edges[t * kEdges + sl].w;
         }
         for (int k = 0; k < 5; ++k) res->selections[k] += (int64_t)tally[t * 8 + k];
         res->expansions_committed += (int64_t)tally[t * 8 + 5];
-        res->levels_read += (int64_t)tally[t * 8 + 6];
-        res->edges_examined += (int64_t)tally[t * 8 + 7];
+        res->nodes_read += (int64_t)tally[t * 8 + 6];
+        res->edges_scored += (int64_t)tally[t * 8 + 7];
         res->nodes_total += counts[t];
         if (counts[t] > res->max_nodes_in_tree) res->max_nodes_in_tree = counts[t];
     }
@@ -527,14 +895,43 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
 }
 
 extern "C" int64_t puct_gomoku_array_bytes(puct_gomoku_engine *e, int32_t id) {
-    if (!e || id < 0 || id > PUCT_GOMOKU_ARR_NODE_LEGAL || !e->arrays[id].ptr) return fail(PUCT_GOMOKU_E_INVALID, "unknown array id %d", id);
-    return (int64_t)e->arrays[id].bytes;
+    size_t count = 0;
+    const size_t elem = e ? array_shape(e->cfg, id, &count) : 0;
+    if (elem == 0) return fail(PUCT_GOMOKU_E_INVALID, "unknown array id %d", id);
+    return (int64_t)(elem * count);
 }
 
 extern "C" int puct_gomoku_read(puct_gomoku_engine *e, int32_t id, void *dst, size_t bytes) {
-    if (!e || !dst || id < 0 || id > PUCT_GOMOKU_ARR_NODE_LEGAL || !e->arrays[id].ptr) return fail(PUCT_GOMOKU_E_INVALID, "unknown array id %d", id);
-    if (bytes != e->arrays[id].bytes) return fail(PUCT_GOMOKU_E_INVALID, "array %d has %zu bytes, buffer has %zu", id, e->arrays[id].bytes, bytes);
+    size_t count = 0;
+    const size_t elem = (e && dst) ? array_shape(e->cfg, id, &count) : 0;
+    if (elem == 0) return fail(PUCT_GOMOKU_E_INVALID, "unknown array id %d", id);
+    if (bytes != elem * count) return fail(PUCT_GOMOKU_E_INVALID, "array %d has %zu bytes, buffer has %zu", id, elem * count, bytes);
     HIP_TRY(hipSetDevice(e->cfg.device));
-    HIP_TRY(hipMemcpy(dst, e->arrays[id].ptr, bytes, hipMemcpyDeviceToHost));
+    const LoopArgs &g = e->args;
+    const void *direct = nullptr;   // arrays the engine keeps in the shape the host reads
+    switch (id) {
+    case PUCT_GOMOKU_ARR_EDGE_ACTION: direct = g.action; break;
+    case PUCT_GOMOKU_ARR_NODE_COUNT: direct = g.node_count; break;
+    case PUCT_GOMOKU_ARR_NODE_BOARD: direct = g.board; break;
+    case PUCT_GOMOKU_ARR_OUT_SELECTED: direct = g.out_selected; break;
+    case PUCT_GOMOKU_ARR_OUT_LEN: direct = g.out_len; break;
+    case PUCT_GOMOKU_ARR_OUT_PATH: direct = g.out_path; break;
+    default: break;
+    }
+    if (direct) {
+        HIP_TRY(hipMemcpy(dst, direct, bytes, hipMemcpyDeviceToHost));
+        return PUCT_GOMOKU_OK;
+    }
+    // the others are fields of the edge and node records: gathered on the device, then copied
+    void *staging = nullptr;
+    HIP_TRY(hipMalloc(&staging, bytes));
+    const unsigned threads = 256;
+    hipLaunchKernelGGL(unpack_kernel, dim3((unsigned)((count + threads - 1) / threads)), dim3(threads), 0, e->stream, g, e->cfg.trees,
+                       (int)id, staging, count);
+    hipError_t err = hipGetLastError();
+    if (err == hipSuccess) err = hipStreamSynchronize(e->stream);
+    if (err == hipSuccess) err = hipMemcpy(dst, staging, bytes, hipMemcpyDeviceToHost);
+    (void)hipFree(staging);
+    if (err != hipSuccess) return fail(PUCT_GOMOKU_E_HIP, "reading array %d failed: %s", id, hipGetErrorString(err));
     return PUCT_GOMOKU_OK;
 }

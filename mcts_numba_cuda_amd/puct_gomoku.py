@@ -24,7 +24,7 @@ class Config(ctypes.Structure):
     _fields_ = [("board_m", ctypes.c_int32), ("board_n", ctypes.c_int32), ("trees", ctypes.c_int32),
                 ("traversals", ctypes.c_int32), ("max_nodes", ctypes.c_int32), ("path_depth", ctypes.c_int32),
                 ("cpuct", ctypes.c_float), ("c_pw", ctypes.c_float), ("alpha_pw", ctypes.c_float),
-                ("soft_winner", ctypes.c_int32), ("recalc_attempts", ctypes.c_int32), ("dirichlet_alpha", ctypes.c_float), ("seed", ctypes.c_uint64),
+                ("dirichlet_alpha", ctypes.c_float), ("seed", ctypes.c_uint64),
                 ("device", ctypes.c_int32)]
 
 
@@ -33,7 +33,7 @@ class Result(ctypes.Structure):
                 ("root_n", ctypes.c_int64 * 256), ("root_w", ctypes.c_double * 256), ("selections", ctypes.c_int64 * 5),
                 ("expansions_committed", ctypes.c_int64), ("nodes_total", ctypes.c_int64),
                 ("max_nodes_in_tree", ctypes.c_int32), ("time_total", ctypes.c_double), ("time_device", ctypes.c_double),
-                ("levels_read", ctypes.c_int64), ("edges_examined", ctypes.c_int64)]
+                ("nodes_read", ctypes.c_int64), ("edges_scored", ctypes.c_int64)]
 
 
 class EngineError(RuntimeError):
@@ -71,16 +71,16 @@ def _check(rc):
 
 
 class PUCTGomoku:
-    """PUCT search on Gomoku with virtual loss: `trees` independent trees on one root, `traversals` concurrent
-    selections per tree and step, a synthetic evaluator (Dirichlet(dirichlet_alpha) priors over the legal cells and a
+    """PUCT search on Gomoku with virtual loss: `trees` independent trees on one root, `traversals` selections per
+    tree and step (claims taken in a fixed order, so a search is reproducible), a synthetic evaluator (Dirichlet(dirichlet_alpha) priors over the legal cells and a
     value in [-1, 1), both pure functions of the position and the seed).  `run` returns the cell with the most root
     visits; `root_n`, `root_q`, `selections`, `performance_info` describe the last search."""
 
     def __init__(self, board_shape=(15, 15), trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5,
-                 c_pw=1.0, alpha_pw=0.5, soft_winner=False, recalc_attempts=0, dirichlet_alpha=0.3, seed=0, device=0):
+                 c_pw=1.0, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, device=0):
         self.cfg = Config(int(board_shape[0]), int(board_shape[1]), int(trees), int(traversals), int(max_nodes),
-                          int(path_depth), float(cpuct), float(c_pw), float(alpha_pw), int(bool(soft_winner)),
-                          int(recalc_attempts), float(dirichlet_alpha), int(seed), int(device))
+                          int(path_depth), float(cpuct), float(c_pw), float(alpha_pw), float(dirichlet_alpha), int(seed),
+                          int(device))
         self._engine = ctypes.c_void_p()
         _check(_lib().puct_gomoku_create(ctypes.byref(self.cfg), ctypes.byref(self._engine)))
         self.result = None
@@ -117,11 +117,14 @@ class PUCTGomoku:
             self.root_q = np.where(self.root_n > 0, root_w / self.root_n, np.nan)
         self.selections = dict(zip(("invalid", "expand", "terminal", "depth_limit", "busy"), res.selections))
         total = sum(res.selections)
+        leaves = total - res.selections[0] - res.selections[4]    # selections that reached a node to evaluate
         self.performance_info = {
             "steps": int(res.steps), "selections": int(total), "selections_per_second": total / max(res.time_device, 1e-12),
+            "leaves": int(leaves), "leaves_per_second": leaves / max(res.time_device, 1e-12),
+            "leaves_per_step": leaves / max(res.steps, 1), "busy_share": res.selections[4] / max(total, 1),
             "steps_per_second": res.steps / max(res.time_device, 1e-12), "expansions": int(res.expansions_committed),
             "nodes_total": int(res.nodes_total), "max_nodes_in_tree": int(res.max_nodes_in_tree),
-            "levels_read": int(res.levels_read), "edges_examined": int(res.edges_examined),
+            "nodes_read": int(res.nodes_read), "edges_scored": int(res.edges_scored),
             "times_[ms]": {"total": 1e3 * res.time_total, "device": 1e3 * res.time_device}}
         self.best_action = int(res.best_action)
         return self.best_action

@@ -245,23 +245,39 @@ void po_backup(int node_level, int virtual_loss, const int *edge_child_id, float
 
 /* ---------------------------------------------------------------------------------------------------------------------
  * Gomoku PUCT loop (selection -> expansion / evaluation -> backup per step).  The reference has no such loop; this
- * restates the library's own definition (include/puct_gomoku.h) sequentially, so it is a second implementation of
- * the same specification rather than a restatement of reference code: PARITY UNPINNED against the reference.  The
- * synthetic evaluator (hash, value, Gamma weights) is shared with the library through its header, because it is
- * the definition of the workload's inputs; what is restated here is the tree logic.  Pins: tests/test_puct_oracle.py
- * checks the rules (five in a row exactly) against the brute-force outcome routine of the MCTS-NC oracle, the priors
- * against the Dirichlet moments, and structural invariants of the trees.
+ * restates the library's own definition (include/puct_gomoku.h) as plain scalar code, so it is a second
+ * implementation of the same specification rather than a restatement of reference code: PARITY UNPINNED against the
+ * reference.  The synthetic evaluator (hash, value, Gamma weights) is shared with the library through its header,
+ * because it is the definition of the workload's inputs; what is restated here is the tree logic.  Pins:
+ * tests/test_puct_oracle.py checks the rules (five in a row exactly) against the brute-force outcome routine of the
+ * MCTS-NC oracle, the priors against the Dirichlet moments, and structural invariants of the trees.
+ *
+ * The order in which the traversals of one step take their claims is part of that definition (it makes a search
+ * reproducible): the traversals of a tree descend in lockstep, one level per round; within a round the traversals
+ * standing on the same node decide one after another, wid ascending, each seeing the claims and expansion tickets of
+ * those before it.  Every single decision is the reference's (src/puct/puct_gpu_v3_cpp.cu:150-275: progressive
+ * widening, expansion ticket, score, order on edges with the rotated tie-break); a claim that is taken in turn never
+ * loses, so the winner-recalc retry and the soft winner have nothing to do.  A traversal that ends BUSY keeps its
+ * claims until the step's backup releases them (the reference's kernel rolls them back at once; no traversal of the
+ * same step reads those edges again, so the difference cannot be observed).
  * ------------------------------------------------------------------------------------------------------------------ */
 #include "../mcts_numba_cuda_amd/csrc/puct_synthetic.h"
 
 #define G_EDGES 256
 #define G_WORDS 16
+#define G_MAX_WARPS 16
+/* selection word of the loop: kind << 28 | slot << 20 | node (include/puct_gomoku.h) */
+#define G_NODE_MASK 0xFFFFF
+#define G_SLOT_SHIFT 20
+#define G_KIND_SHIFT 28
 
 typedef struct {
     int *edge_child; float *edge_prior; float *edge_w; int *edge_n; int *edge_inflight; uint8_t *edge_action;
     int *node_expanded; int *node_expand_inflight; int *node_count; uint32_t *node_board; int8_t *node_turn;
     float *node_value; int *out_selected; int *out_path; int *out_len; float *path_values; int *node_legal;
 } po_gomoku_arrays;
+
+static int g_pack(int kind, int node, int slot) { return (kind << G_KIND_SHIFT) | (slot << G_SLOT_SHIFT) | node; }
 
 static int g_stone(const uint32_t *colour, int cell) { return (colour[cell >> 5] >> (cell & 31)) & 1u; }
 
@@ -315,95 +331,217 @@ static void g_write_priors(const po_gomoku_arrays *A, size_t node_row, const uin
     }
 }
 
-void po_gomoku_search(const po_gomoku_arrays *A, const int8_t *root, int root_turn, int m, int n, int trees, int nodes,
-                      int warps, int path_depth, int steps, float cpuct, float c_pw, float alpha_pw, int soft_winner,
-                      float dirichlet_alpha, uint64_t seed, int64_t *tally /* [trees][8] */) {
+/* Selection of one step in one tree: lockstep descent, claims in wid order within a node.  claims[w] = number of
+ * path entries (claimed edges) traversal w holds when it ends, whatever its kind. */
+static void g_select_step(const po_gomoku_arrays *A, int t, int nodes, int warps, int path_depth, float cpuct,
+                          float c_pw, float alpha_pw, int *claims, int64_t *work) {
+    const size_t trow = (size_t)t * nodes;
+    int cur[G_MAX_WARPS], active[G_MAX_WARPS];
+    for (int w = 0; w < warps; ++w) {
+        cur[w] = 0;
+        active[w] = 1;
+        claims[w] = 0;
+        A->out_selected[(size_t)t * warps + w] = g_pack(K_INVALID, G_NODE_MASK, 0);
+        A->out_len[(size_t)t * warps + w] = 0;
+    }
+    for (int depth = 0;; ++depth) {
+        int any = 0;
+        for (int w = 0; w < warps; ++w) any |= active[w];
+        if (!any) break;
+        int next[G_MAX_WARPS], standing[G_MAX_WARPS];   /* standing: active when the round began */
+        for (int w = 0; w < warps; ++w) next[w] = cur[w], standing[w] = active[w];
+        for (int lead = 0; lead < warps; ++lead) {
+            if (!standing[lead]) continue;
+            int is_leader = 1;
+            for (int w = 0; w < lead; ++w) is_leader &= !(standing[w] && cur[w] == cur[lead]);
+            if (!is_leader) continue;
+            const int node = cur[lead];
+            const size_t nrow = trow + node, erow = nrow * G_EDGES;
+            const int info = A->node_expanded[nrow];
+            work[6] += 1;
+            if (info >= 0 && depth < path_depth) work[7] += info;
+            for (int w = lead; w < warps; ++w) {
+                if (!standing[w] || cur[w] != node) continue;
+                const size_t out = (size_t)t * warps + w;
+                int *path = A->out_path + out * path_depth;
+                claims[w] = depth;
+                if (info == TERMINAL) {
+                    A->out_selected[out] = g_pack(K_TERMINAL, node, 0);
+                    A->out_len[out] = depth + 1;
+                    active[w] = 0;
+                    continue;
+                }
+                if (depth >= path_depth) {
+                    A->out_selected[out] = g_pack(K_DEPTH_LIMIT, node, 0);
+                    A->out_len[out] = depth + 1;
+                    active[w] = 0;
+                    continue;
+                }
+                const int expanded = info;
+                int parent_eff = 1, allowed = 1;
+                if (expanded != 1 || c_pw != 0.0f) {
+                    int total = 0;
+                    for (int e = 0; e < expanded; ++e) total += A->edge_n[erow + e] + A->edge_inflight[erow + e];
+                    parent_eff = total > 1 ? total : 1;
+                    allowed = allowed_children(c_pw, alpha_pw, parent_eff, A->node_legal[nrow]);
+                }
+                if (allowed > expanded) {
+                    if (expanded + A->node_expand_inflight[nrow] < allowed) {
+                        const int slot = expanded + A->node_expand_inflight[nrow]++;
+                        A->out_selected[out] = g_pack(K_EXPAND, node, slot);
+                        A->out_len[out] = depth + 1;
+                        active[w] = 0;
+                        continue;
+                    }
+                    if (expanded == 0) {
+                        A->out_selected[out] = g_pack(K_BUSY, node, 0);
+                        active[w] = 0;
+                        continue;
+                    }
+                }
+                int tie_offset = w;
+                if (tie_offset >= expanded) tie_offset %= expanded;
+                int best = 0;
+                if (expanded > 1) {
+                    const float sqrt_parent = sqrtf((float)parent_eff);
+                    float best_score = -FLT_MAX;
+                    best = INT32_MAX;
+                    for (int e = 0; e < expanded; ++e) {
+                        const int n = A->edge_n[erow + e];
+                        const float q = n > 0 ? A->edge_w[erow + e] / (float)n : 0.0f;
+                        const float u = cpuct * A->edge_prior[erow + e] * sqrt_parent / (float)(n + A->edge_inflight[erow + e] + 1);
+                        const float score = q + u;
+                        if (ahead(score, e, best_score, best, tie_offset, expanded)) {
+                            best_score = score;
+                            best = e;
+                        }
+                    }
+                }
+                if (best == INT32_MAX) {   /* no edge with a comparable score */
+                    A->out_selected[out] = g_pack(K_INVALID, G_NODE_MASK, 0);
+                    active[w] = 0;
+                    continue;
+                }
+                A->edge_inflight[erow + best] += 1;
+                path[depth] = (node << 8) | best;
+                next[w] = A->edge_child[erow + best];
+            }
+        }
+        for (int w = 0; w < warps; ++w) cur[w] = next[w];
+    }
+}
+
+static void g_search_tree(const po_gomoku_arrays *A, int t, const uint32_t *root_words, int root_turn, int m, int n,
+                          int nodes, int warps, int path_depth, int steps, float cpuct, float c_pw, float alpha_pw,
+                          double alpha, uint64_t seed, int64_t *tally) {
     const int cells = m * n;
-    const double alpha = (double)dirichlet_alpha;
+    const size_t trow = (size_t)t * nodes;
+    const uint64_t tree_seed = psyn_tree_seed(seed, t);
+    for (int i = 0; i < G_WORDS; ++i) A->node_board[trow * G_WORDS + i] = root_words[i];
+    const int root_legal = cells - g_popcount(root_words);
+    A->node_turn[trow] = (int8_t)root_turn;
+    A->node_value[trow] = 0.0f;
+    A->node_expanded[trow] = root_legal == 0 ? TERMINAL : 0;
+    A->node_expand_inflight[trow] = 0;
+    A->node_legal[trow] = root_legal;
+    A->node_count[t] = 1;
+    for (int k = 0; k < 8; ++k) tally[k] = 0;
+    if (root_legal > 0) g_write_priors(A, trow, root_words, psyn_board_hash(tree_seed, root_words), cells, alpha);
+    for (int step = 0; step < steps; ++step) {
+        int claims[G_MAX_WARPS];
+        g_select_step(A, t, nodes, warps, path_depth, cpuct, c_pw, alpha_pw, claims, tally);
+        /* which traversals want a child, and does the tree have room for all of them? */
+        int total = 0;
+        for (int w = 0; w < warps; ++w) {
+            const int raw = A->out_selected[(size_t)t * warps + w];
+            const int kind = (raw >> G_KIND_SHIFT) & KIND_MASK, node = raw & G_NODE_MASK, slot = (raw >> G_SLOT_SHIFT) & EDGE_MASK;
+            tally[kind] += 1;
+            if (kind == K_EXPAND && slot < A->node_legal[trow + node]) ++total;
+        }
+        const int base = A->node_count[t];
+        const int fits = base + total <= nodes;
+        int next = base;
+        if (fits) {
+            A->node_count[t] = base + total;
+            tally[5] += total;
+        }
+        for (int w = 0; w < warps; ++w) {
+            const size_t out = (size_t)t * warps + w;
+            const int raw = A->out_selected[out];
+            const int kind = (raw >> G_KIND_SHIFT) & KIND_MASK, node = raw & G_NODE_MASK, slot = (raw >> G_SLOT_SHIFT) & EDGE_MASK;
+            if (kind != K_EXPAND && kind != K_TERMINAL && kind != K_DEPTH_LIMIT) continue;
+            uint32_t board[G_WORDS];
+            for (int i = 0; i < G_WORDS; ++i) board[i] = A->node_board[(trow + node) * G_WORDS + i];
+            const int n_legal = A->node_legal[trow + node];
+            const int turn = A->node_turn[trow + node];
+            float u;
+            if (kind == K_EXPAND && slot < n_legal && fits) {
+                /* the child goes into the node's next free edge slot (the expanded edges of a node stay contiguous
+                 * whatever the tickets say), children numbered in traversal order */
+                const int child = next++;
+                const int taken = A->node_expanded[trow + node]++;
+                const size_t e = (trow + node) * G_EDGES + taken;
+                const int action = A->edge_action[e];
+                uint32_t *mine = board + (turn > 0 ? 0 : 8);
+                mine[action >> 5] |= 1u << (action & 31);
+                const int win = g_makes_five(mine, action, m, n);
+                const int terminal = win || n_legal - 1 == 0;
+                const uint64_t bh = psyn_board_hash(tree_seed, board);
+                const float v_child = win ? -1.0f : (terminal ? 0.0f : psyn_value(bh));
+                for (int i = 0; i < G_WORDS; ++i) A->node_board[(trow + child) * G_WORDS + i] = board[i];
+                A->node_turn[trow + child] = (int8_t)-turn;
+                A->node_value[trow + child] = v_child;
+                A->node_expanded[trow + child] = terminal ? TERMINAL : 0;
+                A->node_expand_inflight[trow + child] = 0;
+                A->node_legal[trow + child] = n_legal - 1;
+                A->edge_child[e] = child;
+                A->edge_n[e] = 1;
+                A->edge_w[e] = -v_child;
+                if (!terminal) g_write_priors(A, trow + child, board, bh, cells, alpha);
+                u = -v_child;
+            } else if (kind == K_TERMINAL) {
+                u = A->node_value[trow + node];
+            } else {
+                u = psyn_value(psyn_board_hash(tree_seed, board));
+            }
+            const int L = A->out_len[out] - 1;
+            for (int d = 0; d < L; ++d) A->path_values[out * path_depth + d] = ((L - d) & 1) ? -u : u;
+        }
+        /* backup: every traversal releases its claims; those that reached a node also leave a visit and a value */
+        for (int w = 0; w < warps; ++w) {
+            const size_t out = (size_t)t * warps + w;
+            const int raw = A->out_selected[out];
+            const int kind = (raw >> G_KIND_SHIFT) & KIND_MASK;
+            const int counted = kind == K_EXPAND || kind == K_TERMINAL || kind == K_DEPTH_LIMIT;
+            for (int d = 0; d < claims[w]; ++d) {
+                const int enc = A->out_path[out * path_depth + d];
+                const size_t e = (trow + (enc >> 8)) * G_EDGES + (enc & 0xFF);
+                A->edge_inflight[e] -= 1;
+                if (counted) {
+                    A->edge_n[e] += 1;
+                    A->edge_w[e] += A->path_values[out * path_depth + d];
+                }
+            }
+            if (kind == K_EXPAND) A->node_expand_inflight[trow + (raw & G_NODE_MASK)] -= 1;
+        }
+    }
+}
+
+void po_gomoku_search(const po_gomoku_arrays *A, const int8_t *root, int root_turn, int m, int n, int trees, int nodes,
+                      int warps, int path_depth, int steps, float cpuct, float c_pw, float alpha_pw,
+                      float dirichlet_alpha, uint64_t seed, int threads, int64_t *tally /* [trees][8] */) {
+    const int cells = m * n;
     uint32_t words[G_WORDS] = {0};
     for (int i = 0; i < cells; ++i) {
         if (root[i] == 1) words[i >> 5] |= 1u << (i & 31);
         if (root[i] == -1) words[8 + (i >> 5)] |= 1u << (i & 31);
     }
-    for (int t = 0; t < trees; ++t) {
-        const size_t trow = (size_t)t * nodes;
-        for (int i = 0; i < G_WORDS; ++i) A->node_board[trow * G_WORDS + i] = words[i];
-        const int n_legal = cells - g_popcount(words);
-        A->node_turn[trow] = (int8_t)root_turn;
-        A->node_value[trow] = 0.0f;
-        A->node_expanded[trow] = n_legal == 0 ? TERMINAL : 0;
-        A->node_expand_inflight[trow] = 0;
-        A->node_legal[trow] = n_legal;
-        A->node_count[t] = 1;
-        for (int k = 0; k < 8; ++k) tally[t * 8 + k] = 0;
-        if (n_legal > 0) g_write_priors(A, trow, words, psyn_board_hash(psyn_tree_seed(seed, t), words), cells, alpha);
-    }
-    for (int step = 0; step < steps; ++step) {
-        select_all(cpuct, c_pw, alpha_pw, soft_winner, A->edge_child, A->edge_prior, A->edge_w, A->edge_n, A->edge_inflight,
-                   A->node_expand_inflight, A->node_expanded, A->node_count, A->out_selected, A->out_path, A->out_len, trees,
-                   nodes, G_EDGES, warps, path_depth, A->node_legal);
-        for (int t = 0; t < trees; ++t) {
-            const size_t trow = (size_t)t * nodes;
-            const uint64_t tree_seed = psyn_tree_seed(seed, t);
-            /* which traversals want a child, and does the tree have room for all of them? */
-            int total = 0;
-            for (int w = 0; w < warps; ++w) {
-                const int raw = A->out_selected[(size_t)t * warps + w];
-                const int kind = (raw >> KIND_SHIFT) & KIND_MASK, node = raw & NODE_MASK, slot = (raw >> SLOT_SHIFT) & EDGE_MASK;
-                tally[t * 8 + kind] += 1;
-                if (kind == K_EXPAND && slot < cells - g_popcount(A->node_board + (trow + node) * G_WORDS)) ++total;
-            }
-            const int base = A->node_count[t];
-            const int fits = base + total <= nodes;
-            int next = base;
-            if (fits) {
-                A->node_count[t] = base + total;
-                tally[t * 8 + 5] += total;
-            }
-            for (int w = 0; w < warps; ++w) {
-                const size_t out = (size_t)t * warps + w;
-                const int raw = A->out_selected[out];
-                const int kind = (raw >> KIND_SHIFT) & KIND_MASK, node = raw & NODE_MASK, slot = (raw >> SLOT_SHIFT) & EDGE_MASK;
-                if (kind != K_EXPAND && kind != K_TERMINAL && kind != K_DEPTH_LIMIT) continue;
-                uint32_t board[G_WORDS];
-                for (int i = 0; i < G_WORDS; ++i) board[i] = A->node_board[(trow + node) * G_WORDS + i];
-                const int n_legal = cells - g_popcount(board);
-                const int turn = A->node_turn[trow + node];
-                float u;
-                if (kind == K_EXPAND && slot < n_legal && fits) {
-                    const int child = next++;
-                    const size_t e = (trow + node) * G_EDGES + slot;
-                    const int action = A->edge_action[e];
-                    uint32_t *mine = board + (turn > 0 ? 0 : 8);
-                    mine[action >> 5] |= 1u << (action & 31);
-                    const int win = g_makes_five(mine, action, m, n);
-                    const int terminal = win || n_legal - 1 == 0;
-                    const uint64_t bh = psyn_board_hash(tree_seed, board);
-                    const float v_child = win ? -1.0f : (terminal ? 0.0f : psyn_value(bh));
-                    for (int i = 0; i < G_WORDS; ++i) A->node_board[(trow + child) * G_WORDS + i] = board[i];
-                    A->node_turn[trow + child] = (int8_t)-turn;
-                    A->node_value[trow + child] = v_child;
-                    A->node_expanded[trow + child] = terminal ? TERMINAL : 0;
-                    A->node_expand_inflight[trow + child] = 0;
-                    A->node_legal[trow + child] = n_legal - 1;
-                    A->edge_child[e] = child;
-                    A->edge_n[e] = 1;
-                    A->edge_w[e] = -v_child;
-                    A->node_expanded[trow + node] += 1;
-                    if (!terminal) g_write_priors(A, trow + child, board, bh, cells, alpha);
-                    u = -v_child;
-                } else if (kind == K_TERMINAL) {
-                    u = A->node_value[trow + node];
-                } else {
-                    u = psyn_value(psyn_board_hash(tree_seed, board));
-                }
-                const int L = A->out_len[out] - 1;
-                for (int d = 0; d < L; ++d) A->path_values[out * path_depth + d] = ((L - d) & 1) ? -u : u;
-            }
-        }
-        po_backup(0, 1, NULL, A->edge_w, A->edge_n, A->edge_inflight, NULL, A->node_expand_inflight, A->node_count,
-                  A->out_selected, A->out_path, A->out_len, A->path_values, trees, nodes, G_EDGES, warps, path_depth);
-    }
+    if (warps > G_MAX_WARPS) warps = G_MAX_WARPS;
+    /* trees are independent searches */
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads > 0 ? threads : 1)
+    for (int t = 0; t < trees; ++t)
+        g_search_tree(A, t, words, root_turn, m, n, nodes, warps, path_depth, steps, cpuct, c_pw, alpha_pw,
+                      (double)dirichlet_alpha, seed, tally + (size_t)t * 8);
 }
 
 /* helpers the tests use to pin the evaluator and the rule check */

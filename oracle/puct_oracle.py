@@ -68,13 +68,14 @@ class _GomokuArrays(ctypes.Structure):
 
 
 def gomoku_search(board, turn, steps, trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0,
-                  alpha_pw=0.5, soft_winner=0, dirichlet_alpha=0.3, seed=0):
-    """Sequential Gomoku PUCT search (oracle/puct_oracle.c: po_gomoku_search); returns every array plus the tallies."""
+                  alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, threads=8):
+    """Gomoku PUCT search on the host (oracle/puct_oracle.c: po_gomoku_search), `threads` trees at a time; returns
+    every array plus the tallies."""
     board = np.ascontiguousarray(board, dtype=np.int8)
     m, n = board.shape
     T, N, E, W, D = trees, max_nodes, 256, traversals, path_depth
     h = {
-        "edge_child": np.full((T, N, E), -1, np.int32), "edge_prior": np.zeros((T, N, E), np.float32),
+        "edge_child": np.zeros((T, N, E), np.int32), "edge_prior": np.zeros((T, N, E), np.float32),
         "edge_w": np.zeros((T, N, E), np.float32), "edge_n": np.zeros((T, N, E), np.int32),
         "edge_inflight": np.zeros((T, N, E), np.int32), "edge_action": np.zeros((T, N, E), np.uint8),
         "node_expanded": np.zeros((T, N), np.int32), "node_expand_inflight": np.zeros((T, N), np.int32),
@@ -89,9 +90,9 @@ def gomoku_search(board, turn, steps, trees=16, traversals=16, max_nodes=16384, 
     L = lib()
     L.po_gomoku_search.restype = None
     L.po_gomoku_search.argtypes = [ctypes.POINTER(_GomokuArrays), ctypes.c_void_p] + [ctypes.c_int] * 8 + \
-        [ctypes.c_float] * 3 + [ctypes.c_int, ctypes.c_float, ctypes.c_uint64, ctypes.c_void_p]
+        [ctypes.c_float] * 4 + [ctypes.c_uint64, ctypes.c_int, ctypes.c_void_p]
     L.po_gomoku_search(ctypes.byref(arrays), board.ctypes.data, int(turn), m, n, T, N, W, D, int(steps), cpuct, c_pw,
-                       alpha_pw, int(soft_winner), dirichlet_alpha, int(seed), tally.ctypes.data)
+                       alpha_pw, dirichlet_alpha, int(seed), int(threads), tally.ctypes.data)
     h["tally"] = tally
     return h
 
