@@ -83,6 +83,8 @@ typedef struct {
     int64_t nodes_read;              /* node visits of the selections that loaded the node (its word and its expanded edges);
                                         traversals standing on the same node in the same round share one */
     int64_t edges_scored;            /* expanded edges loaded on those visits */
+    double time_select, time_expand, time_backup; /* seconds of time_device per phase (fused search only; mean over the
+                                        trees of what the first wavefront of each tree's workgroup measured) */
 } puct_gomoku_result;
 
 typedef struct puct_gomoku_engine puct_gomoku_engine;

@@ -1,10 +1,10 @@
 /*
- * Natural logarithm and exponential built only from IEEE-754 double basic operations (no fused multiply-add when
- * compiled with -ffp-contract=off, no library call), so that every compiler and both host and device evaluate
- * bit-identical results.  Plain C99 / C++ / HIP.  Both follow the classic table-free argument reductions:
+ * Natural logarithm and exponential built only from IEEE-754 basic operations (no fused multiply-add when compiled
+ * with -ffp-contract=off, no library call), so that every compiler and both host and device evaluate bit-identical
+ * results.  Plain C99 / C++ / HIP.  They follow the classic table-free argument reductions:
  *   log: x = 2^k (1 + f), s = f / (2 + f), log(1 + f) = f - hfsq + s (hfsq + R(s^2));
  *   exp: x = k ln2 + r, |r| <= ln2 / 2, exp(r) = 1 + r + r c / (2 - c) with c = r - r^2 P(r^2).
- * Errors stay below 1 ulp.
+ * The double precision logarithm stays below 1 ulp.
  */
 #ifndef MCTSNC_DET_MATH_H
 #define MCTSNC_DET_MATH_H
@@ -60,48 +60,45 @@ DETM_FN double detm_log(double x) {
     return dk * ln2_hi - ((s * (f - R) - dk * ln2_lo) - f);
 }
 
-/* Any finite x; overflows to +inf above 709.78, returns 0 below -745.13 (no subnormal results are needed by the
- * callers, which only use arguments <= 0 and a few small positive ones). */
-DETM_FN double detm_exp(double x) {
-    const double ln2_hi = 6.93147180369123816490e-01, ln2_lo = 1.90821492927058770002e-10,
-                 inv_ln2 = 1.44269504088896338700e+00;
-    const double P1 = 1.66666666666666019037e-01, P2 = -2.77777777770155933842e-03, P3 = 6.61375632143793436117e-05,
-                 P4 = -1.65339022054652515390e-06, P5 = 4.13813679705723846039e-08;
-    if (x != x) return x;
-    if (x > 7.09782712893383973096e+02) {
-        union { uint64_t u; double d; } inf;
-        inf.u = 0x7ff0000000000000ull;
-        return inf.d;
-    }
-    if (x < -7.45133219101941108420e+02) return 0.0;
-    const double ax = x < 0.0 ? -x : x;
-    double hi = x, lo = 0.0;
-    int32_t k = 0;
-    if (ax > 0.34657359027997264) { /* |x| > ln2 / 2 */
-        if (ax < 1.0397207708399179) {
-            k = x < 0.0 ? -1 : 1;
-        } else {
-            k = (int32_t)(inv_ln2 * x + (x < 0.0 ? -0.5 : 0.5));
-        }
-        const double t = (double)k;
-        hi = x - t * ln2_hi;
-        lo = t * ln2_lo;
-        x = hi - lo;
-    } else if (ax < 3.725290298461914e-09) { /* 2^-28 */
-        return 1.0 + x;
-    }
-    const double t = x * x;
-    const double c = x - t * (P1 + t * (P2 + t * (P3 + t * (P4 + t * P5))));
-    if (k == 0) return 1.0 - ((x * c) / (c - 2.0) - x);
-    double y = 1.0 - ((lo - (x * c) / (2.0 - c)) - hi);
-    union { double d; uint64_t u; } v;
-    v.d = y;
-    if (k >= -1021) {
-        v.u += (uint64_t)(int64_t)k << 52;
-        return v.d;
-    }
-    v.u += (uint64_t)(int64_t)(k + 1000) << 52;
-    return v.d * 9.33263618503218878990e-302; /* 2^-1000 */
+/* Single precision, branch-free: natural logarithm of a positive normal x and exponential of x <= 0 (0 below -86,
+ * where the result would near the end of the normal range).  Same reductions as above with shorter polynomials; errors stay
+ * below 2 ulp.  Every lane of a wavefront runs the same instructions whatever its argument. */
+DETM_FN float detm_logf(float x) {
+    const float ln2_hi = 6.9313812256e-01f, ln2_lo = 9.0580006145e-06f;
+    const float Lg1 = 0.66666662693f, Lg2 = 0.40000972152f, Lg3 = 0.28498786688f, Lg4 = 0.24279078841f;
+    union { float f; uint32_t u; } v;
+    v.f = x;
+    uint32_t ix = v.u + (0x3f800000u - 0x3f3504f3u);
+    const int32_t k = (int32_t)(ix >> 23) - 0x7f;
+    v.u = (ix & 0x007fffffu) + 0x3f3504f3u; /* x / 2^k in [sqrt(1/2), sqrt(2)) */
+    const float f = v.f - 1.0f;
+    const float s = f / (2.0f + f);
+    const float z = s * s;
+    const float w = z * z;
+    const float t1 = w * (Lg2 + w * Lg4);
+    const float t2 = z * (Lg1 + w * Lg3);
+    const float R = t2 + t1;
+    const float hfsq = 0.5f * f * f;
+    const float dk = (float)k;
+    return s * (hfsq + R) + dk * ln2_lo - hfsq + f + dk * ln2_hi;
+}
+
+DETM_FN float detm_expf(float x) {
+    const float ln2_hi = 6.9314575195e-01f, ln2_lo = 1.4286067653e-06f, inv_ln2 = 1.4426950216e+00f;
+    const float P1 = 1.6666625440e-1f, P2 = -2.7667332906e-3f;
+    const float xc = x < -86.0f ? -86.0f : x;
+    const int32_t k = (int32_t)(inv_ln2 * xc - 0.5f);
+    const float t = (float)k;
+    const float hi = xc - t * ln2_hi;
+    const float lo = t * ln2_lo;
+    const float r = hi - lo;
+    const float rr = r * r;
+    const float c = r - rr * (P1 + rr * P2);
+    const float y = 1.0f + (r * c / (2.0f - c) - lo + hi);
+    union { float f; uint32_t u; } v;
+    v.f = y;
+    v.u += (uint32_t)k << 23; /* k in [-125, 0]: the result stays normal */
+    return x < -86.0f ? 0.0f : v.f;
 }
 
 #endif

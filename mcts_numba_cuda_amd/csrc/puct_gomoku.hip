@@ -39,6 +39,7 @@ constexpr int kTurnBit = 0x10000;
 
 constexpr int kTrav = kMaxWavesPerBlock;   // most traversals per tree: one wavefront each, one workgroup per tree
 constexpr int kSlices = kEdges / kWave;    // 64-edge slices of the widest node
+constexpr int kTally = 12;
 
 struct LoopArgs {
     Edge *edges;       // [trees][max_nodes][256]
@@ -49,11 +50,12 @@ struct LoopArgs {
     // what the traversals of the last step ended with, [trees][traversals] (paths: [trees][traversals][path_depth])
     int *out_selected, *out_len, *out_claims, *out_path;
     float *out_value;
-    unsigned long long *tally;   // [trees][8]: selections by kind (0..4), children created (5), nodes read (6), edges scored (7)
+    unsigned long long *tally;   // [trees][12]: selections by kind (0..4), children created (5), nodes read (6), edges scored (7),
+                                 // ticks of the 100 MHz clock that wavefront 0 spent selecting (8), expanding (9), backing up (10)
     float cpuct, c_pw, alpha_pw;
     int m, n, cells, max_nodes, traversals, path_depth, steps;
     uint64_t seed;
-    double dirichlet_alpha;
+    float dirichlet_alpha;
 };
 
 // What a step keeps per traversal between its phases.  The paths ([traversals][path_depth] words) follow in dynamic LDS.
@@ -183,19 +185,20 @@ __device__ void write_priors(const LoopArgs &g, int tree, int node, const uint32
         return c < g.cells && !stone_at(board, c) && !stone_at(board + 8, c);
     };
     while (i < kPer && !legal_cell(i)) ++i;
+    uint64_t key = i < kPer ? psyn_cell_key(board_hash, lane + i * kWave) : 0;
     while (__ballot(i < kPer) != 0) {
+        float x;
+        const int ok = psyn_gamma_round(g.dirichlet_alpha, key, round, &x);
         if (i < kPer) {
-            const int c = lane + i * kWave;
-            double x;
-            const int ok = psyn_gamma_round(g.dirichlet_alpha, psyn_cell_key(board_hash, c), round, &x);
             if (ok || round == PSYN_GAMMA_ROUNDS - 1) {
-                const uint32_t key = psyn_weight_key(x, c);
+                const uint32_t weight = psyn_weight_key(x, lane + i * kWave);
 #pragma unroll
                 for (int k = 0; k < kPer; ++k)
-                    if (k == i) mine[k] = key;
+                    if (k == i) mine[k] = weight;
                 ++i;
                 round = 0;
                 while (i < kPer && !legal_cell(i)) ++i;
+                if (i < kPer) key = psyn_cell_key(board_hash, lane + i * kWave);
             } else {
                 ++round;
             }
@@ -215,6 +218,38 @@ __device__ void write_priors(const LoopArgs &g, int tree, int node, const uint32
         if (mine[k] != 0u) store_edge(g.edges + erow + k, 0, 0.0f, psyn_prior(psyn_key_weight(mine[k]), sum, n_legal), 0u);
     }
     if (mine[0] != 0u) *reinterpret_cast<uint32_t *>(g.action + erow) = cells_packed;   // keys descend: slot 4 * lane is the lane's first
+}
+
+// Order-preserving integer image of a score that can win: the reference starts from (-FLT_MAX, no edge) and accepts
+// a score that is greater than or equal to it, so NaN and -inf never win and get 0 (src/puct/puct_gpu_v3_cpp.cu:51-71);
+// -0.0f counts as +0.0f because the reference compares floats.  The upper word of candidate_key().
+__device__ __forceinline__ uint32_t score_image(float score) {
+    if (!(score >= -FLT_MAX)) return 0u;
+    const uint32_t b = __float_as_uint(score + 0.0f);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    auto step = [](uint32_t x, auto ctrl) {
+        const uint32_t o = (uint32_t)dpp<decltype(ctrl)::value>((int)x);
+        return o > x ? o : x;
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});
+    v = step(v, std::integral_constant<int, 0x4E>{});
+    v = step(v, std::integral_constant<int, 0x141>{});
+    v = step(v, std::integral_constant<int, 0x140>{});
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
+// Progressive widening, src/puct/puct_gpu_v3_cpp.cu:150-157; sqrt_n = sqrtf((float)n_node), which the score needs too.
+__device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int n_node, float sqrt_n, int edges) {
+    const float val = (alpha_pw == 0.5f) ? c_pw * sqrt_n : c_pw * powf((float)n_node, alpha_pw);
+    if (val >= (float)edges) return edges;
+    const int allowed = (int)ceilf(val);
+    return allowed > 1 ? allowed : 1;
 }
 
 // ---- selection ---------------------------------------------------------------------------------------------------
@@ -271,9 +306,11 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
     for (uint64_t rest = members; rest != 0; rest &= rest - 1) {
         const int j = __builtin_ctzll(rest);   // the traversal deciding now
         int parent_eff = 1, allowed = 1;
+        float sqrt_parent = 1.0f;
         if (expanded != 1 || g.c_pw != 0.0f) {
             parent_eff = total > 1 ? total : 1;
-            allowed = allowed_children(g.c_pw, g.alpha_pw, parent_eff, legal);
+            sqrt_parent = sqrtf((float)parent_eff);
+            allowed = allowed_children(g.c_pw, g.alpha_pw, parent_eff, sqrt_parent, legal);
         }
         if (allowed > expanded) {
             if (expanded + tickets < allowed) {   // expansion ticket
@@ -298,21 +335,38 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
         }
         int best = 0;
         if (expanded > 1) {
-            int tie_offset = j;
-            if (tie_offset >= expanded) tie_offset %= expanded;
-            const float sqrt_parent = sqrtf((float)parent_eff);
-            uint64_t key = 0;
+            // The highest score first: its order-preserving integer image, reduced over the wavefront.  Only if more
+            // than one edge attains it does the rotated edge index decide, through the full keys.
+            float score[kSlices];
+            uint32_t image[kSlices], lane_top = 0;
 #pragma unroll
             for (int i = 0; i < kSlices; ++i) {
-                const int eid = lane + i * kWave;
-                if (i * kWave < expanded && eid < expanded) {
-                    const float score = q[i] + cp[i] * sqrt_parent / (float)den[i];
-                    const uint64_t k = candidate_key(score, eid, tie_offset, expanded);
+                score[i] = q[i] + cp[i] * sqrt_parent / (float)den[i];
+                image[i] = (i * kWave < expanded && lane + i * kWave < expanded) ? score_image(score[i]) : 0u;
+                lane_top = image[i] > lane_top ? image[i] : lane_top;
+            }
+            const uint32_t top = wave_max_u32(lane_top);
+            int hits = 0;
+            best = kNoEdge;
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) {
+                const uint64_t at = __ballot(image[i] == top);
+                hits += __popcll(at);
+                if (at != 0) best = i * kWave + __builtin_ctzll(at);
+            }
+            if (top == 0) {
+                best = kNoEdge;
+            } else if (hits > 1) {
+                int tie_offset = j;
+                if (tie_offset >= expanded) tie_offset %= expanded;
+                uint64_t key = 0;
+#pragma unroll
+                for (int i = 0; i < kSlices; ++i) {
+                    const uint64_t k = image[i] == top ? candidate_key(score[i], lane + i * kWave, tie_offset, expanded) : 0;
                     key = k > key ? k : key;
                 }
+                best = (int)(wave_max(key) & 0xFFFFu);
             }
-            const uint64_t top = wave_max(key);
-            best = top == 0 ? kNoEdge : (int)(top & 0xFFFFu);
         }
         const int best_lane = best & (kWave - 1), best_slice = best >> 6;
         int child = 0;
@@ -529,7 +583,7 @@ __global__ __launch_bounds__(kWave) void init_kernel(const LoopArgs g, const uin
     }
     const int n_legal = g.cells - wave_sum(__popc(w));
     wave_lds_fence();
-    if (lane < 8) g.tally[(size_t)tree * 8 + lane] = 0ull;
+    if (lane < kTally) g.tally[(size_t)tree * kTally + lane] = 0ull;
     if (lane < g.traversals) {
         const size_t out = (size_t)tree * g.traversals + lane;
         g.out_selected[out] = pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
@@ -592,6 +646,7 @@ __device__ void state_from_memory(const LoopArgs &g, StepLds &s, int *paths, int
 
 struct Work {
     uint32_t kinds[5] = {0, 0, 0, 0, 0}, created = 0, nodes_read = 0, edges_scored = 0;
+    uint64_t ticks[3] = {0, 0, 0};   // selection, expansion, backup, on wavefront 0
     __device__ void count_kind(const StepLds &s, int wave) {
         const int kind = (s.sel[wave] >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7;
 #pragma unroll
@@ -599,13 +654,16 @@ struct Work {
     }
     __device__ void to_memory(const LoopArgs &g, int tree, int lane) const {
         if (lane != 0) return;
-        unsigned long long *row = g.tally + (size_t)tree * 8;
+        unsigned long long *row = g.tally + (size_t)tree * kTally;
 #pragma unroll
         for (int k = 0; k < 5; ++k)
             if (kinds[k]) atomicAdd(row + k, (unsigned long long)kinds[k]);
         if (created) atomicAdd(row + 5, (unsigned long long)created);
         if (nodes_read) atomicAdd(row + 6, (unsigned long long)nodes_read);
         if (edges_scored) atomicAdd(row + 7, (unsigned long long)edges_scored);
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+            if (ticks[k]) atomicAdd(row + 8 + k, (unsigned long long)ticks[k]);
     }
 };
 
@@ -620,13 +678,24 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g) 
     Work work;
     if (threadIdx.x == 0) s.node_count = g.node_count[tree];
     __syncthreads();
+    uint64_t t0 = wave == 0 ? wall_clock64() : 0;
     for (int step = 0; step < g.steps; ++step) {
         select_phase(g, s, paths, tree, wave, lane, n_waves, work.nodes_read, work.edges_scored);
         work.count_kind(s, wave);
+        uint64_t t1 = 0, t2 = 0;
+        if (wave == 0) t1 = wall_clock64();
         expand_phase(g, s, tree, wave, lane, n_waves, work.created);
         phase_barrier();   // the claims of the selection and the new edges are in memory
+        if (wave == 0) t2 = wall_clock64();
         backup_phase(g, s, paths, tree, wave, lane, n_waves);
         phase_barrier();
+        if (wave == 0) {
+            const uint64_t t3 = wall_clock64();
+            work.ticks[0] += t1 - t0;
+            work.ticks[1] += t2 - t1;
+            work.ticks[2] += t3 - t2;
+            t0 = t3;
+        }
     }
     state_to_memory(g, s, paths, tree, n_waves);
     work.to_memory(g, tree, lane);
@@ -794,14 +863,14 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     if ((rc = alloc(e, &g.edges, T * N * kEdges)) || (rc = alloc(e, &g.info, T * N)) || (rc = alloc(e, &g.board, T * N * kBoardWords)) ||
         (rc = alloc(e, &g.action, T * N * kEdges)) || (rc = alloc(e, &g.node_count, T)) || (rc = alloc(e, &g.out_selected, T * W)) ||
         (rc = alloc(e, &g.out_len, T * W)) || (rc = alloc(e, &g.out_claims, T * W)) || (rc = alloc(e, &g.out_path, T * W * D)) ||
-        (rc = alloc(e, &g.out_value, T * W)) || (rc = alloc(e, &g.tally, T * 8)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords))) {
+        (rc = alloc(e, &g.out_value, T * W)) || (rc = alloc(e, &g.tally, T * kTally)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords))) {
         puct_gomoku_destroy(e);
         return rc;
     }
     g.cpuct = c->cpuct; g.c_pw = c->c_pw; g.alpha_pw = c->alpha_pw;
     g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes;
     g.traversals = c->traversals; g.path_depth = c->path_depth; g.steps = 0;
-    g.seed = c->seed; g.dirichlet_alpha = (double)c->dirichlet_alpha;
+    g.seed = c->seed; g.dirichlet_alpha = c->dirichlet_alpha;
     hipError_t err = hipStreamCreate(&e->stream);
     if (err == hipSuccess) err = hipEventCreate(&e->ev0);
     if (err == hipSuccess) err = hipEventCreate(&e->ev1);
@@ -865,12 +934,12 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
     std::vector<NodeInfo> root_info(T);
     std::vector<uint8_t> a_root(T * kEdges);
     std::vector<int> counts(T);
-    std::vector<unsigned long long> tally(T * 8);
+    std::vector<unsigned long long> tally(T * kTally);
     HIP_TRY(hipMemcpy2D(root_edges.data(), sizeof(Edge) * kEdges, g.edges, sizeof(Edge) * kEdges * N, sizeof(Edge) * kEdges, T, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy2D(root_info.data(), sizeof(NodeInfo), g.info, sizeof(NodeInfo) * N, sizeof(NodeInfo), T, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy2D(a_root.data(), kEdges, g.action, (size_t)kEdges * N, kEdges, T, hipMemcpyDeviceToHost));
     HIP_TRY(hipMemcpy(counts.data(), g.node_count, sizeof(int) * T, hipMemcpyDeviceToHost));
-    HIP_TRY(hipMemcpy(tally.data(), g.tally, sizeof(unsigned long long) * T * 8, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(tally.data(), g.tally, sizeof(unsigned long long) * T * kTally, hipMemcpyDeviceToHost));
     memset(res, 0, sizeof *res);
     res->steps = steps;
     for (size_t t = 0; t < T; ++t) {
@@ -879,10 +948,13 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
             res->root_n[a] += root_edges[t * kEdges + sl].n;
             res->root_w[a] += (double)root_edges[t * kEdges + sl].w;
         }
-        for (int k = 0; k < 5; ++k) res->selections[k] += (int64_t)tally[t * 8 + k];
-        res->expansions_committed += (int64_t)tally[t * 8 + 5];
-        res->nodes_read += (int64_t)tally[t * 8 + 6];
-        res->edges_scored += (int64_t)tally[t * 8 + 7];
+        for (int k = 0; k < 5; ++k) res->selections[k] += (int64_t)tally[t * kTally + k];
+        res->expansions_committed += (int64_t)tally[t * kTally + 5];
+        res->nodes_read += (int64_t)tally[t * kTally + 6];
+        res->edges_scored += (int64_t)tally[t * kTally + 7];
+        res->time_select += 1e-8 * (double)tally[t * kTally + 8] / (double)T;
+        res->time_expand += 1e-8 * (double)tally[t * kTally + 9] / (double)T;
+        res->time_backup += 1e-8 * (double)tally[t * kTally + 10] / (double)T;
         res->nodes_total += counts[t];
         if (counts[t] > res->max_nodes_in_tree) res->max_nodes_in_tree = counts[t];
     }

@@ -1,8 +1,8 @@
 /*
  * Synthetic evaluator of the Gomoku PUCT loop: stands in for a policy/value network with a pure function of the
  * position, so that a search is reproducible and the host can recompute every prior and value.  Plain C99 / C++ / HIP;
- * all arithmetic is 64-bit integer mixing plus IEEE double basic operations and the deterministic log / exp of
- * det_math.h, so host and device agree bit for bit.
+ * all arithmetic is 64-bit integer mixing plus IEEE basic operations and the deterministic log / exp of det_math.h, so
+ * host and device agree bit for bit.
  *
  *   value(position)      uniform in [-1, 1) from a hash of the position (for the player to move)
  *   prior over the legal cells:  Dirichlet(alpha): one Gamma(alpha, 1) variate per legal cell from a hash of
@@ -48,33 +48,36 @@ PSYN_FN float psyn_value(uint64_t board_hash) {
     return (float)((int32_t)(h >> 40) - 8388608) * (1.0f / 8388608.0f);
 }
 
-/* Uniform double in (0, 1), never 0 or 1. */
-PSYN_FN double psyn_unit(uint64_t h) { return ((double)(h >> 11) + 0.5) * (1.0 / 9007199254740992.0); }
+/* Uniform float in (0, 1), never 0 or 1, from 23 bits. */
+PSYN_FN float psyn_unit(uint32_t h) { return ((float)(h >> 9) + 0.5f) * (1.0f / 8388608.0f); }
 
-/* One round of the Ahrens-Dieter rejection sampler "GS" for Gamma(alpha, 1), 0 < alpha < 1, driven by the uniforms
- * number 2 * round and 2 * round + 1 of the counter-based stream of `key`.  Writes the candidate to *x and returns
- * whether it is accepted.  The acceptance tests are taken in the log domain (log u2 <= -x, resp.
- * log u2 <= (alpha - 1) log x), which lets both branches share two of their three logarithms. */
-PSYN_FN int psyn_gamma_round(double alpha, uint64_t key, int round, double *x) {
-    const double b = 1.0 + alpha * 0.36787944117144233; /* 1 + alpha / e */
-    const double inv_alpha = 1.0 / alpha;
-    const double u1 = psyn_unit(psyn_mix64(key + 2u * (uint64_t)round));
-    const double log_u2 = detm_log(psyn_unit(psyn_mix64(key + 2u * (uint64_t)round + 1u)));
-    const double p = b * u1;
-    const int small = p <= 1.0;
-    const double log_t = detm_log(small ? p : (b - p) * inv_alpha);
-    if (small) {
-        *x = detm_exp(log_t * inv_alpha);
-        return log_u2 <= -*x;
-    }
-    *x = -log_t;
-    return log_u2 <= (alpha - 1.0) * detm_log(*x);
+/* One round of the Ahrens-Dieter rejection sampler "GS" for Gamma(alpha, 1), 0 < alpha < 1, driven by the two halves
+ * of word number `round` of the counter-based stream of `key`.  Writes the candidate to *x and returns whether it is
+ * accepted.  The acceptance tests are taken in the log domain (log u2 <= -x, resp. log u2 <= (alpha - 1) log x).
+ * Single precision throughout (a weight keeps 15 mantissa bits) and without a branch: a wavefront whose lanes take
+ * different sides of the sampler runs the same instructions. */
+PSYN_FN int psyn_gamma_round(float alpha, uint64_t key, int round, float *x) {
+    const float b = 1.0f + alpha * 0.36787944117f; /* 1 + alpha / e */
+    const float inv_alpha = 1.0f / alpha;
+    const uint64_t h = psyn_mix64(key + (uint64_t)round);
+    const float u1 = psyn_unit((uint32_t)(h >> 32));
+    const float log_u2 = detm_logf(psyn_unit((uint32_t)h));
+    const float p = b * u1;
+    const int small = p <= 1.0f;
+    float t = small ? p : (b - p) * inv_alpha;
+    t = t < 1.17549435e-38f ? 1.17549435e-38f : t;
+    const float log_t = detm_logf(t);
+    const float x_small = detm_expf(log_t * inv_alpha);
+    const float x_large = -log_t; /* > 1 on this side: b - p < alpha / e */
+    const float bound = small ? -x_small : (alpha - 1.0f) * detm_logf(small ? 2.0f : x_large);
+    *x = small ? x_small : x_large;
+    return log_u2 <= bound;
 }
 
 #define PSYN_GAMMA_ROUNDS 16 /* the chance of needing more is below 1e-9; the last candidate is taken then */
 
-PSYN_FN double psyn_gamma(double alpha, uint64_t key) {
-    double x = 0.0;
+PSYN_FN float psyn_gamma(float alpha, uint64_t key) {
+    float x = 0.0f;
     for (int round = 0; round < PSYN_GAMMA_ROUNDS; ++round)
         if (psyn_gamma_round(alpha, key, round, &x)) break;
     return x;
@@ -89,9 +92,9 @@ PSYN_FN uint64_t psyn_cell_key(uint64_t board_hash, int cell) {
  * views of the same number: a 32-bit sort key whose unsigned order is "larger weight first, then smaller cell" (0 is
  * reserved for cells that are not legal), and the weight in 2^-32 fixed point for the exact, order-independent sum
  * (a sum over 256 cells stays below 2^48). */
-PSYN_FN uint32_t psyn_weight_key(double gamma, int cell) {
+PSYN_FN uint32_t psyn_weight_key(float gamma, int cell) {
     union { float f; uint32_t u; } v;
-    v.f = (float)(gamma > 255.0 ? 255.0 : gamma);
+    v.f = gamma > 255.0f ? 255.0f : gamma;
     return 0x80000000u | (v.u & 0xFFFFFF00u) | (uint32_t)(255 - cell);
 }
 PSYN_FN uint64_t psyn_key_weight(uint32_t key) {

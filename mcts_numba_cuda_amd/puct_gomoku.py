@@ -33,7 +33,8 @@ class Result(ctypes.Structure):
                 ("root_n", ctypes.c_int64 * 256), ("root_w", ctypes.c_double * 256), ("selections", ctypes.c_int64 * 5),
                 ("expansions_committed", ctypes.c_int64), ("nodes_total", ctypes.c_int64),
                 ("max_nodes_in_tree", ctypes.c_int32), ("time_total", ctypes.c_double), ("time_device", ctypes.c_double),
-                ("nodes_read", ctypes.c_int64), ("edges_scored", ctypes.c_int64)]
+                ("nodes_read", ctypes.c_int64), ("edges_scored", ctypes.c_int64), ("time_select", ctypes.c_double),
+                ("time_expand", ctypes.c_double), ("time_backup", ctypes.c_double)]
 
 
 class EngineError(RuntimeError):
@@ -125,7 +126,8 @@ class PUCTGomoku:
             "steps_per_second": res.steps / max(res.time_device, 1e-12), "expansions": int(res.expansions_committed),
             "nodes_total": int(res.nodes_total), "max_nodes_in_tree": int(res.max_nodes_in_tree),
             "nodes_read": int(res.nodes_read), "edges_scored": int(res.edges_scored),
-            "times_[ms]": {"total": 1e3 * res.time_total, "device": 1e3 * res.time_device}}
+            "times_[ms]": {"total": 1e3 * res.time_total, "device": 1e3 * res.time_device, "select": 1e3 * res.time_select,
+                           "expand": 1e3 * res.time_expand, "backup": 1e3 * res.time_backup}}
         self.best_action = int(res.best_action)
         return self.best_action
 

@@ -305,7 +305,7 @@ static int g_makes_five(const uint32_t *mine, int cell, int m, int n) {
 }
 
 static void g_write_priors(const po_gomoku_arrays *A, size_t node_row, const uint32_t *board, uint64_t bh, int cells,
-                           double alpha) {
+                           float alpha) {
     uint32_t key[G_EDGES];
     uint64_t sum = 0;
     int n_legal = 0;
@@ -433,7 +433,7 @@ static void g_select_step(const po_gomoku_arrays *A, int t, int nodes, int warps
 
 static void g_search_tree(const po_gomoku_arrays *A, int t, const uint32_t *root_words, int root_turn, int m, int n,
                           int nodes, int warps, int path_depth, int steps, float cpuct, float c_pw, float alpha_pw,
-                          double alpha, uint64_t seed, int64_t *tally) {
+                          float alpha, uint64_t seed, int64_t *tally) {
     const int cells = m * n;
     const size_t trow = (size_t)t * nodes;
     const uint64_t tree_seed = psyn_tree_seed(seed, t);
@@ -541,13 +541,14 @@ void po_gomoku_search(const po_gomoku_arrays *A, const int8_t *root, int root_tu
 #pragma omp parallel for schedule(dynamic, 1) num_threads(threads > 0 ? threads : 1)
     for (int t = 0; t < trees; ++t)
         g_search_tree(A, t, words, root_turn, m, n, nodes, warps, path_depth, steps, cpuct, c_pw, alpha_pw,
-                      (double)dirichlet_alpha, seed, tally + (size_t)t * 8);
+                      dirichlet_alpha, seed, tally + (size_t)t * 8);
 }
 
 /* helpers the tests use to pin the evaluator and the rule check */
-double po_det_exp(double x) { return detm_exp(x); }
-double po_gamma(double alpha, uint64_t key) { return psyn_gamma(alpha, key); }
-uint32_t po_cell_key(double alpha, uint64_t board_hash, int cell) { return psyn_weight_key(psyn_gamma(alpha, psyn_cell_key(board_hash, cell)), cell); }
+float po_det_expf(float x) { return detm_expf(x); }
+float po_det_logf(float x) { return detm_logf(x); }
+float po_gamma(float alpha, uint64_t key) { return psyn_gamma(alpha, key); }
+uint32_t po_cell_key(float alpha, uint64_t board_hash, int cell) { return psyn_weight_key(psyn_gamma(alpha, psyn_cell_key(board_hash, cell)), cell); }
 float po_value(uint64_t board_hash) { return psyn_value(board_hash); }
 uint64_t po_board_hash(uint64_t seed, int tree, const uint32_t *words) { return psyn_board_hash(psyn_tree_seed(seed, tree), words); }
 int po_makes_five(const uint32_t *mine, int cell, int m, int n) { return g_makes_five(mine, cell, m, n); }

@@ -100,12 +100,13 @@ def gomoku_search(board, turn, steps, trees=16, traversals=16, max_nodes=16384, 
 def evaluator():
     """The synthetic evaluator's primitives, for the tests that pin them."""
     L = lib()
-    L.po_det_exp.restype = ctypes.c_double
-    L.po_det_exp.argtypes = [ctypes.c_double]
-    L.po_gamma.restype = ctypes.c_double
-    L.po_gamma.argtypes = [ctypes.c_double, ctypes.c_uint64]
+    for name in ("po_det_expf", "po_det_logf"):
+        getattr(L, name).restype = ctypes.c_float
+        getattr(L, name).argtypes = [ctypes.c_float]
+    L.po_gamma.restype = ctypes.c_float
+    L.po_gamma.argtypes = [ctypes.c_float, ctypes.c_uint64]
     L.po_cell_key.restype = ctypes.c_uint32
-    L.po_cell_key.argtypes = [ctypes.c_double, ctypes.c_uint64, ctypes.c_int]
+    L.po_cell_key.argtypes = [ctypes.c_float, ctypes.c_uint64, ctypes.c_int]
     L.po_value.restype = ctypes.c_float
     L.po_value.argtypes = [ctypes.c_uint64]
     L.po_board_hash.restype = ctypes.c_uint64

@@ -69,14 +69,22 @@ import math
 import puct_gomoku_checks as gc
 
 
-def test_det_exp_within_one_ulp_of_libm():
+def test_single_precision_log_and_exp_within_two_ulp_of_libm():
+    """The evaluator's branch-free float32 log (positive normal arguments) and exp (arguments <= 0, zero below -86)
+    against numpy's, which are correctly rounded to well below an ulp."""
     ev = po.evaluator()
     rng = np.random.default_rng(0)
-    xs = np.concatenate([rng.uniform(-700, 700, 20000), rng.uniform(-2, 2, 20000), [0.0, -0.0, 1e-10, -1e-10, 0.3465735, 1.0397]])
+    xs = np.concatenate([rng.uniform(0, 1, 20000), np.exp(rng.uniform(-87, 88, 20000)), [1.0, 0.5, 2.0, 1.17549435e-38, 3.4e38,
+                         0.70710677, 0.70710683, 1.4142135, 1.4142137]]).astype(np.float32)
     for x in xs:
-        got, want = ev.po_det_exp(float(x)), math.exp(float(x))
-        assert abs(got - want) <= math.ulp(want), x
-    assert ev.po_det_exp(-800.0) == 0.0 and ev.po_det_exp(800.0) == math.inf
+        got, want = np.float32(ev.po_det_logf(float(x))), np.log(np.float64(x))
+        assert abs(np.float64(got) - want) <= 2 * np.spacing(np.float32(abs(want))), x
+    assert ev.po_det_logf(1.0) == 0.0
+    xs = np.concatenate([-rng.uniform(0, 86, 20000), -rng.uniform(0, 2, 20000), [0.0, -0.0, -1e-10, -0.3465735, -0.3465737, -1.0397, -86.0]]).astype(np.float32)
+    for x in xs:
+        got, want = np.float32(ev.po_det_expf(float(x))), np.exp(np.float64(x))
+        assert abs(np.float64(got) - want) <= 2 * np.spacing(np.float32(want)), x
+    assert ev.po_det_expf(0.0) == 1.0 and ev.po_det_expf(-86.5) == 0.0 and ev.po_det_expf(-1000.0) == 0.0
 
 
 def test_gamma_variates_have_gamma_moments():
