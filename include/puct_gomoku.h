@@ -46,6 +46,7 @@ extern "C" {
 #define PUCT_GOMOKU_E_INVALID (-1)
 #define PUCT_GOMOKU_E_HIP (-2)
 #define PUCT_GOMOKU_E_ROOT (-3)
+#define PUCT_GOMOKU_E_SYNC (-4)   /* workgroups of the search launch waited for each other in vain; the search was abandoned */
 
 #define PUCT_GOMOKU_MAX_NODES (1 << 20)
 #define PUCT_GOMOKU_MAX_PATH_DEPTH 256
@@ -67,6 +68,10 @@ typedef struct {
     float dirichlet_alpha;     /* in (0, 1) */
     uint64_t seed;
     int32_t device;
+    int32_t evaluators;        /* 0..8: workgroups per tree that work out the priors of the step's new nodes on other
+                                  compute units while the tree's own workgroup backs the step up (fused search only; fewer
+                                  are used when the device cannot keep trees * (1 + evaluators) workgroups resident);
+                                  0 = the tree's workgroup does it itself.  The trees are the same either way. */
 } puct_gomoku_config;
 
 typedef struct {

@@ -56,7 +56,21 @@ struct LoopArgs {
     int m, n, cells, max_nodes, traversals, path_depth, steps;
     uint64_t seed;
     float dirichlet_alpha;
+    struct EvalRequests *requests;   // [trees]
+    int evaluators;                  // workgroups per tree that work out the priors of new nodes (fused search), 0 = none
 };
+
+// What a tree's workgroup hands to its evaluator workgroups, step by step: the non-terminal children the step created.
+struct EvalRequests {
+    int tag;     // step + 1 once the step's entries are complete; -1 when the search is over
+    int done;    // entries the evaluators have worked off since the search began
+    int abort;   // a bounded wait gave up: everybody leaves
+    int n;       // entries of the step
+    int child[kMaxWavesPerBlock];       // node to evaluate, -1 = nothing to do for this entry
+    uint64_t hash[kMaxWavesPerBlock];   // its position's hash
+};
+constexpr int kMaxEvaluators = 8;
+constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s of the 100 MHz clock: a partner that is not there
 
 // What a step keeps per traversal between its phases.  The paths ([traversals][path_depth] words) follow in dynamic LDS.
 struct StepLds {
@@ -67,6 +81,9 @@ struct StepLds {
     float value[kTrav];  // of the reached node, for the player who moved into it
     int want[kTrav];     // node the traversal expands, -1 if none
     int node_count;
+    int requests;        // evaluation requests of this step
+    int requested;       // ... and of all steps so far
+    int gave_up;
     uint32_t board[kTrav][kBoardWords];
 };
 
@@ -437,6 +454,7 @@ __device__ void select_phase(const LoopArgs &g, StepLds &s, int *paths, int tree
 // into the node's next free edge slots in traversal order (the expanded edges of a node stay contiguous whatever the
 // tickets say); when the tree cannot take all expansions of a step none is committed (those traversals evaluate the
 // node they reached instead).
+template <bool FARM>
 __device__ void expand_phase(const LoopArgs &g, StepLds &s, int tree, int wave, int lane, int n_waves, uint32_t &created) {
     const int raw = s.sel[wave];
     const int kind = (raw >> PUCT_GOMOKU_SEL_KIND_SHIFT) & 7;
@@ -463,7 +481,10 @@ __device__ void expand_phase(const LoopArgs &g, StepLds &s, int tree, int wave, 
     const int base = s.node_count;
     const bool fits = base + total <= g.max_nodes;
     __syncthreads();
-    if (wave == 0 && lane == 0 && fits) s.node_count = base + total;
+    if (wave == 0 && lane == 0) {
+        if (fits) s.node_count = base + total;
+        s.requests = fits ? total : 0;
+    }
     if (wave == 0 && fits) created += (uint32_t)total;
 
     float u = 0.0f;   // value of the reached node for the player who moved into it
@@ -490,7 +511,14 @@ __device__ void expand_phase(const LoopArgs &g, StepLds &s, int tree, int wave, 
             e->link = (uint32_t)child << 8;
             if (rank == 0) g.info[trow + node].expanded = ni.expanded + siblings;
         }
-        if (!terminal) write_priors(g, tree, child, board, lane, bh, child_legal);
+        if (FARM) {   // the child's priors are an evaluator workgroup's work
+            if (lane == 0) {
+                g.requests[tree].child[before] = terminal ? -1 : child;
+                g.requests[tree].hash[before] = bh;
+            }
+        } else if (!terminal) {
+            write_priors(g, tree, child, board, lane, bh, child_legal);
+        }
         u = -v_child;
     } else if (kind == PUCT_SELECT_TERMINAL) {
         u = ni.value;
@@ -596,6 +624,11 @@ __global__ __launch_bounds__(kWave) void init_kernel(const LoopArgs g, const uin
             make_uint4((uint32_t)(n_legal == 0 ? PUCT_NODE_EXPANDED_TERMINAL : 0), 0u,
                        (uint32_t)(n_legal | (root_turn > 0 ? 0 : kTurnBit)), 0u);
         g.node_count[tree] = 1;
+        EvalRequests &rq = g.requests[tree];
+        rq.tag = 0;
+        rq.done = 0;
+        rq.abort = 0;
+        rq.n = 0;
     }
     if (n_legal > 0) write_priors(g, tree, 0, board, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
 }
@@ -616,7 +649,7 @@ __device__ __forceinline__ void phase_barrier() {
 // What the traversals of a step ended with, between the launches of the stepwise mode and for the host to read.
 __device__ void state_to_memory(const LoopArgs &g, const StepLds &s, const int *paths, int tree, int n_waves) {
     const size_t out = (size_t)tree * g.traversals;
-    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += blockDim.x) {
+    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += n_waves * kWave) {   // the workgroup's live threads
         const int t = i / g.path_depth, d = i - t * g.path_depth;
         g.out_path[out * g.path_depth + i] = d < s.claims[t] ? paths[i] : -1;
     }
@@ -631,7 +664,7 @@ __device__ void state_to_memory(const LoopArgs &g, const StepLds &s, const int *
 }
 __device__ void state_from_memory(const LoopArgs &g, StepLds &s, int *paths, int tree, int n_waves) {
     const size_t out = (size_t)tree * g.traversals;
-    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += blockDim.x) paths[i] = g.out_path[out * g.path_depth + i];
+    for (int i = threadIdx.x; i < n_waves * g.path_depth; i += n_waves * kWave) paths[i] = g.out_path[out * g.path_depth + i];
     if (threadIdx.x < kTrav) {
         const int t = threadIdx.x;
         const bool live = t < n_waves;
@@ -669,14 +702,143 @@ struct Work {
 
 extern __shared__ int dynamic_lds[];
 
-// The whole search of one tree in one launch: one workgroup per tree, one wavefront per traversal.
-__global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g) {
+// ---- evaluator workgroups --------------------------------------------------------------------------------------------
+// The priors of a new node are a pure function of its position, and nothing reads them before the next step's
+// selection, so they need not be worked out on the compute unit that owns the tree: the tree's workgroup posts the
+// step's new nodes, goes on with its backup, and picks the results up before the next step.  An evaluator workgroup
+// takes two nodes at a time, four wavefronts and one cell per lane each; the slot of a cell is the number of larger keys
+// among the node's 256, counted from LDS.  Same priors, bit for bit, as write_priors().
+struct EvalLds {
+    uint32_t keys[2][kEdges];
+    unsigned long long weight[2][4];
+    int legal[2][4];
+    int tag;
+};
+
+__device__ __forceinline__ int poll_word(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// Entries `first` and `first + 1` of the step, by wavefronts 0..3 and 4..7 of the workgroup; all eight must call it.
+__device__ void evaluate_pair(const LoopArgs &g, EvalLds &L, int tree, int first, int n, int wave, int lane) {
+    const EvalRequests &rq = g.requests[tree];
+    const int group = wave >> 2, part = wave & 3, index = first + group;
+    const int child = index < n ? rq.child[index] : -1;
+    const bool active = child > 0;
+    const size_t trow = (size_t)tree * g.max_nodes;
+    const int cell = part * kWave + lane;
+    uint32_t weight_key = 0;
+    bool legal = false;
+    if (active) {
+        const uint32_t w = lane < kBoardWords ? g.board[(trow + child) * kBoardWords + lane] : 0u;
+        // words of the lane's cell: the same for each half of the wavefront
+        uint32_t plus = (uint32_t)__builtin_amdgcn_readlane((int)w, 2 * part), minus = (uint32_t)__builtin_amdgcn_readlane((int)w, 8 + 2 * part);
+        const uint32_t plus_hi = (uint32_t)__builtin_amdgcn_readlane((int)w, 2 * part + 1);
+        const uint32_t minus_hi = (uint32_t)__builtin_amdgcn_readlane((int)w, 8 + 2 * part + 1);
+        if (lane >= 32) plus = plus_hi, minus = minus_hi;
+        legal = cell < g.cells && !(((plus | minus) >> (lane & 31)) & 1u);
+        const uint64_t key = psyn_cell_key(rq.hash[index], cell);
+        bool pending = legal;
+        for (int round = 0; __ballot(pending) != 0; ++round) {
+            float x;
+            const int ok = psyn_gamma_round(g.dirichlet_alpha, key, round, &x);
+            if (pending && (ok || round == PSYN_GAMMA_ROUNDS - 1)) {
+                weight_key = psyn_weight_key(x, cell);
+                pending = false;
+            }
+        }
+    }
+    L.keys[group][cell] = weight_key;
+    const uint64_t part_sum = wave_sum64(weight_key ? psyn_key_weight(weight_key) : 0);
+    const int part_legal = __popcll(__ballot(legal));
+    if (lane == 0) {
+        L.weight[group][part] = part_sum;
+        L.legal[group][part] = part_legal;
+    }
+    __syncthreads();
+    if (legal) {
+        const uint64_t sum = L.weight[group][0] + L.weight[group][1] + L.weight[group][2] + L.weight[group][3];
+        const int n_legal = L.legal[group][0] + L.legal[group][1] + L.legal[group][2] + L.legal[group][3];
+        int slot = 0;
+        const uint4 *keys = reinterpret_cast<const uint4 *>(L.keys[group]);
+#pragma unroll 8
+        for (int c = 0; c < kEdges / 4; ++c) {
+            const uint4 k = keys[c];
+            slot += (k.x > weight_key) + (k.y > weight_key) + (k.z > weight_key) + (k.w > weight_key);
+        }
+        const size_t e = (trow + child) * kEdges + slot;
+        store_edge(g.edges + e, 0, 0.0f, psyn_prior(psyn_key_weight(weight_key), sum, n_legal), 0u);
+        g.action[e] = (uint8_t)cell;
+    }
+    __syncthreads();   // the keys are free again
+}
+
+__device__ void evaluator_loop(const LoopArgs &g, EvalLds &L, int tree, int helper, int wave, int lane) {
+    EvalRequests &rq = g.requests[tree];
+    for (int step = 0;; ++step) {
+        if (threadIdx.x == 0) {
+            const uint64_t start = wall_clock64();
+            int tag;
+            while ((tag = poll_word(&rq.tag)) >= 0 && tag <= step) {
+                if (poll_word(&rq.abort) != 0 || wall_clock64() - start > kWaitTicks) {
+                    __hip_atomic_store(&rq.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    tag = -1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            L.tag = tag;
+        }
+        __syncthreads();
+        const int tag = L.tag;
+        __syncthreads();
+        if (tag < 0) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const int n = rq.n;
+        int worked_off = 0;
+        for (int first = 2 * helper; first < n; first += 2 * g.evaluators) {
+            evaluate_pair(g, L, tree, first, n, wave, lane);
+            worked_off += n - first >= 2 ? 2 : 1;
+        }
+        // every wavefront's stores have reached the L2 before one of them reports; the release pushes them on
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (threadIdx.x == 0 && worked_off > 0) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_fetch_add(&rq.done, worked_off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+// The whole search in one launch.  evaluators == 0: one workgroup per tree (grid = trees).  Otherwise every tree has
+// 1 + evaluators workgroups; those of one tree have the same blockIdx.x % 8, which is how workgroups are dealt to the
+// eight XCDs, so a tree's requests and results meet in one L2.
+__global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, int trees) {
     __shared__ StepLds s;
+    __shared__ EvalLds eval_lds;
     int *paths = dynamic_lds;
-    const int tree = blockIdx.x, lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = g.traversals;
+    int tree = blockIdx.x, role = 0;
+    if (g.evaluators > 0) {
+        const int per_tree = 1 + g.evaluators, nth = blockIdx.x / 8;
+        tree = (int)(blockIdx.x % 8) + 8 * (nth / per_tree);
+        role = nth % per_tree;
+    }
+    if (tree >= trees) return;
+    if (role > 0) {
+        if (wave >= 8) return;   // an evaluator workgroup works with eight wavefronts
+        evaluator_loop(g, eval_lds, tree, role - 1, wave, lane);
+        return;
+    }
+    if (wave >= n_waves) return;   // the launch's workgroups are as large as the larger of the two kinds needs
+    const bool farm = g.evaluators > 0;
+    EvalRequests &rq = g.requests[tree];
     Work work;
-    if (threadIdx.x == 0) s.node_count = g.node_count[tree];
+    if (threadIdx.x == 0) {
+        s.node_count = g.node_count[tree];
+        s.requested = 0;
+        s.gave_up = 0;
+    }
     __syncthreads();
     uint64_t t0 = wave == 0 ? wall_clock64() : 0;
     for (int step = 0; step < g.steps; ++step) {
@@ -684,11 +846,32 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g) 
         work.count_kind(s, wave);
         uint64_t t1 = 0, t2 = 0;
         if (wave == 0) t1 = wall_clock64();
-        expand_phase(g, s, tree, wave, lane, n_waves, work.created);
-        phase_barrier();   // the claims of the selection and the new edges are in memory
+        if (farm)
+            expand_phase<true>(g, s, tree, wave, lane, n_waves, work.created);
+        else
+            expand_phase<false>(g, s, tree, wave, lane, n_waves, work.created);
+        phase_barrier();   // the claims of the selection and the new nodes are in memory
+        if (farm && threadIdx.x == 0) {   // ... and the evaluators may start on this step's nodes
+            rq.n = s.requests;
+            s.requested += s.requests;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_store(&rq.tag, step + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         if (wave == 0) t2 = wall_clock64();
         backup_phase(g, s, paths, tree, wave, lane, n_waves);
+        if (farm && threadIdx.x == 0) {   // the next selection may descend into the new nodes: their priors must be there
+            const uint64_t start = wall_clock64();
+            while (poll_word(&rq.done) < s.requested) {
+                if (poll_word(&rq.abort) != 0 || wall_clock64() - start > kWaitTicks) {
+                    __hip_atomic_store(&rq.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s.gave_up = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
         phase_barrier();
+        if (s.gave_up) break;
         if (wave == 0) {
             const uint64_t t3 = wall_clock64();
             work.ticks[0] += t1 - t0;
@@ -697,6 +880,7 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g) 
             t0 = t3;
         }
     }
+    if (farm && threadIdx.x == 0) __hip_atomic_store(&rq.tag, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     state_to_memory(g, s, paths, tree, n_waves);
     work.to_memory(g, tree, lane);
 }
@@ -720,7 +904,7 @@ __global__ __launch_bounds__(kTrav *kWave) void expand_step_kernel(const LoopArg
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), n_waves = blockDim.x / kWave;
     Work work;
     state_from_memory(g, s, paths, tree, n_waves);
-    expand_phase(g, s, tree, wave, lane, n_waves, work.created);
+    expand_phase<false>(g, s, tree, wave, lane, n_waves, work.created);
     __syncthreads();
     state_to_memory(g, s, paths, tree, n_waves);
     work.to_memory(g, tree, lane);
@@ -854,6 +1038,8 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     if (!(c->dirichlet_alpha > 0.0f && c->dirichlet_alpha < 1.0f))
         return fail(PUCT_GOMOKU_E_INVALID, "dirichlet_alpha = %g, need 0 < alpha < 1", (double)c->dirichlet_alpha);
     if (!(c->cpuct >= 0.0f) || !(c->c_pw >= 0.0f)) return fail(PUCT_GOMOKU_E_INVALID, "cpuct and c_pw must not be negative");
+    if (c->evaluators < 0 || c->evaluators > kMaxEvaluators)
+        return fail(PUCT_GOMOKU_E_INVALID, "evaluators = %d, need 0..%d", c->evaluators, kMaxEvaluators);
     HIP_TRY(hipSetDevice(c->device));
     auto *e = new puct_gomoku_engine();
     e->cfg = *c;
@@ -863,14 +1049,14 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     if ((rc = alloc(e, &g.edges, T * N * kEdges)) || (rc = alloc(e, &g.info, T * N)) || (rc = alloc(e, &g.board, T * N * kBoardWords)) ||
         (rc = alloc(e, &g.action, T * N * kEdges)) || (rc = alloc(e, &g.node_count, T)) || (rc = alloc(e, &g.out_selected, T * W)) ||
         (rc = alloc(e, &g.out_len, T * W)) || (rc = alloc(e, &g.out_claims, T * W)) || (rc = alloc(e, &g.out_path, T * W * D)) ||
-        (rc = alloc(e, &g.out_value, T * W)) || (rc = alloc(e, &g.tally, T * kTally)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords))) {
+        (rc = alloc(e, &g.out_value, T * W)) || (rc = alloc(e, &g.tally, T * kTally)) || (rc = alloc(e, &g.requests, T)) || (rc = alloc(e, &e->d_root, (size_t)kBoardWords))) {
         puct_gomoku_destroy(e);
         return rc;
     }
     g.cpuct = c->cpuct; g.c_pw = c->c_pw; g.alpha_pw = c->alpha_pw;
     g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes;
     g.traversals = c->traversals; g.path_depth = c->path_depth; g.steps = 0;
-    g.seed = c->seed; g.dirichlet_alpha = c->dirichlet_alpha;
+    g.seed = c->seed; g.dirichlet_alpha = c->dirichlet_alpha; g.evaluators = c->evaluators;
     hipError_t err = hipStreamCreate(&e->stream);
     if (err == hipSuccess) err = hipEventCreate(&e->ev0);
     if (err == hipSuccess) err = hipEventCreate(&e->ev1);
@@ -912,7 +1098,18 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
     HIP_TRY(hipEventRecord(e->ev0, s));
     if (fused) {
         if (steps > 0) {
-            hipLaunchKernelGGL(search_kernel, grid, block, lds, s, g);
+            // The tree workgroups and their evaluators wait for each other, so every workgroup of the launch must be
+            // resident: as many evaluators per tree as the device takes at once, none if it comes to that.
+            int waves = c.traversals, per_cu = 0;
+            if (g.evaluators > 0 && waves < 8) waves = 8;
+            hipDeviceProp_t prop;
+            HIP_TRY(hipGetDeviceProperties(&prop, c.device));
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, search_kernel, waves * kWave, lds));
+            const long resident = (long)per_cu * prop.multiProcessorCount, groups = 8L * ((c.trees + 7) / 8);
+            while (g.evaluators > 0 && groups * (1 + g.evaluators) > resident) g.evaluators -= 1;
+            if (g.evaluators == 0) waves = c.traversals;
+            const dim3 all(g.evaluators > 0 ? (unsigned)(groups * (1 + g.evaluators)) : (unsigned)c.trees);
+            hipLaunchKernelGGL(search_kernel, all, dim3(waves * kWave), lds, s, g, (int)c.trees);
             HIP_TRY(hipGetLastError());
         }
     } else {
@@ -927,6 +1124,14 @@ extern "C" int puct_gomoku_run(puct_gomoku_engine *e, const int8_t *board, int32
     HIP_TRY(hipStreamSynchronize(s));
     float ms = 0.0f;
     HIP_TRY(hipEventElapsedTime(&ms, e->ev0, e->ev1));
+    if (fused && g.evaluators > 0 && steps > 0) {
+        std::vector<EvalRequests> rq(c.trees);
+        HIP_TRY(hipMemcpy(rq.data(), g.requests, sizeof(EvalRequests) * c.trees, hipMemcpyDeviceToHost));
+        for (int t = 0; t < c.trees; ++t)
+            if (rq[t].abort)
+                return fail(PUCT_GOMOKU_E_SYNC, "tree %d: a workgroup waited for more than 3 s for its partners (are all %d workgroups of "
+                            "the launch resident?); the search was abandoned", t, (int)(8 * ((c.trees + 7) / 8) * (1 + g.evaluators)));
+    }
 
     // root tables of all trees
     const size_t T = c.trees, N = c.max_nodes;
