@@ -85,6 +85,7 @@ struct StepLds {
     int requested;       // ... and of all steps so far
     int gave_up;
     uint32_t board[kTrav][kBoardWords];
+    int stage[kTrav][kWave];   // per wavefront: edges on their way from four per lane to one per lane
 };
 
 __device__ __forceinline__ int pack_sel(int kind, int node, int slot) {
@@ -270,56 +271,26 @@ __device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int 
 }
 
 // ---- selection ---------------------------------------------------------------------------------------------------
-// The traversals of a tree descend in lockstep, one level per round.  The traversals that stand on the same node are
-// served by one wavefront (that of the first of them), which loads the node's edges once and lets the traversals decide
-// one after another, wid ascending, on registers: every decision is the reference's (progressive widening, expansion
-// ticket, score, order on edges with the rotated tie-break: src/puct/puct_gpu_v3_cpp.cu:150-275) on the state that the
-// claims of the traversals before it have left.  Taking the claims in turn is one of the interleavings the reference's
-// atomics allow, needs no atomics itself, never loses a claim and makes a search reproducible.
-__device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *next, int tree, int node, uint64_t members,
-                             int depth, int lane, uint32_t &nodes_read, uint32_t &edges_scored) {
-    const size_t nrow = (size_t)tree * g.max_nodes + node;
-    Edge *row = g.edges + nrow * kEdges;
-    // the first 64 edges are requested together with the node's own word, before anything about the node is known
-    const Edge first = load_edge(row + lane);
-    const NodeInfo ni = load_info(g.info + nrow);
-    const int expanded = ni.expanded;
-    nodes_read += 1;
-    if (expanded == PUCT_NODE_EXPANDED_TERMINAL || depth >= g.path_depth) {
-        const int kind = expanded == PUCT_NODE_EXPANDED_TERMINAL ? PUCT_SELECT_TERMINAL : PUCT_SELECT_DEPTH_LIMIT;
-        if (lane < kTrav && ((members >> lane) & 1ull)) {
-            s.sel[lane] = pack_sel(kind, node, 0);
-            s.len[lane] = depth + 1;
-            s.claims[lane] = depth;
-            next[lane] = -1;
-        }
-        return;
-    }
-    edges_scored += (uint32_t)expanded;
+// The edges of one node as the deciding traversals see them: up to NS per lane.
+template <int NS>
+struct EdgeSet {
+    float q[NS], cp[NS];   // mean value, cpuct * prior
+    int den[NS];           // visits + claims in flight + 1
+    uint32_t link[NS], link_loaded[NS];
+    int eid[NS];           // edge slot, -1 = none
+};
 
-    float q[kSlices], cp[kSlices];
-    int den[kSlices];
-    uint32_t link[kSlices], link_loaded[kSlices];
-    int total = 0;
-#pragma unroll
-    for (int i = 0; i < kSlices; ++i) {
-        const int eid = lane + i * kWave;
-        Edge e = first;
-        if (i > 0) {
-            e = Edge{0, 0.0f, 0.0f, 0u};
-            if (i * kWave < expanded) e = load_edge(row + eid);
-        }
-        const bool valid = eid < expanded;
-        q[i] = valid && e.n > 0 ? e.w / (float)e.n : 0.0f;
-        cp[i] = g.cpuct * e.prior;
-        link[i] = link_loaded[i] = e.link;
-        den[i] = e.n + (int)(e.link & 0xFFu) + 1;
-        total += valid ? den[i] - 1 : 0;
-    }
-    total = wave_sum(total);
-    int tickets = ni.tickets;
-    const int legal = ni.legal_turn & 0xFFFF;
+template <int NS>
+__device__ __forceinline__ float edge_score(const EdgeSet<NS> &e, int i, float sqrt_parent, int more_claims) {
+    return e.q[i] + e.cp[i] * sqrt_parent / (float)(e.den[i] + more_claims);
+}
 
+// The traversals `members` decide one after another on the edges in `e` (which must include every edge that can come
+// first for any of them); `total` = visits + claims over all expanded edges of the node, `tickets` = expansion tickets out.
+template <int NS>
+__device__ __forceinline__ void decide_in_turn(const LoopArgs &g, StepLds &s, int *paths, int *next, EdgeSet<NS> &e, int node,
+                                               uint64_t members, int depth, int lane, int expanded, int legal, int &total,
+                                               int &tickets) {
     for (uint64_t rest = members; rest != 0; rest &= rest - 1) {
         const int j = __builtin_ctzll(rest);   // the traversal deciding now
         int parent_eff = 1, allowed = 1;
@@ -350,47 +321,52 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
                 continue;
             }
         }
-        int best = 0;
+        // The highest score first: its order-preserving integer image, reduced over the wavefront.  Only if more than
+        // one edge attains it does the rotated edge index decide, through the full keys.  (A node's only edge is taken
+        // whatever its score, as in the reference.)
+        int best_lane = 0, best_slot = 0, hits = 1;
         if (expanded > 1) {
-            // The highest score first: its order-preserving integer image, reduced over the wavefront.  Only if more
-            // than one edge attains it does the rotated edge index decide, through the full keys.
-            float score[kSlices];
-            uint32_t image[kSlices], lane_top = 0;
+            float score[NS];
+            uint32_t image[NS], lane_top = 0;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) {
-                score[i] = q[i] + cp[i] * sqrt_parent / (float)den[i];
-                image[i] = (i * kWave < expanded && lane + i * kWave < expanded) ? score_image(score[i]) : 0u;
+            for (int i = 0; i < NS; ++i) {
+                score[i] = edge_score(e, i, sqrt_parent, 0);
+                image[i] = e.eid[i] >= 0 ? score_image(score[i]) : 0u;
                 lane_top = image[i] > lane_top ? image[i] : lane_top;
             }
             const uint32_t top = wave_max_u32(lane_top);
-            int hits = 0;
-            best = kNoEdge;
+            hits = 0;
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i) {
+            for (int i = 0; i < NS; ++i) {
                 const uint64_t at = __ballot(image[i] == top);
                 hits += __popcll(at);
-                if (at != 0) best = i * kWave + __builtin_ctzll(at);
+                if (at != 0) best_lane = __builtin_ctzll(at), best_slot = i;
             }
             if (top == 0) {
-                best = kNoEdge;
+                hits = 0;
             } else if (hits > 1) {
                 int tie_offset = j;
                 if (tie_offset >= expanded) tie_offset %= expanded;
                 uint64_t key = 0;
+                int key_slot = 0;
 #pragma unroll
-                for (int i = 0; i < kSlices; ++i) {
-                    const uint64_t k = image[i] == top ? candidate_key(score[i], lane + i * kWave, tie_offset, expanded) : 0;
-                    key = k > key ? k : key;
+                for (int i = 0; i < NS; ++i) {
+                    const uint64_t k = image[i] == top ? candidate_key(score[i], e.eid[i], tie_offset, expanded) : 0;
+                    if (k > key) key = k, key_slot = i;
                 }
-                best = (int)(wave_max(key) & 0xFFFFu);
+                const uint64_t first = wave_max(key);
+                best_lane = __builtin_ctzll(__ballot(key == first));
+                best_slot = __builtin_amdgcn_readlane(key_slot, best_lane);
             }
         }
-        const int best_lane = best & (kWave - 1), best_slice = best >> 6;
-        int child = 0;
-        if (best != kNoEdge) {
+        int child = 0, best = 0;
+        if (hits > 0) {
 #pragma unroll
-            for (int i = 0; i < kSlices; ++i)
-                if (best_slice == i) child = (int)((uint32_t)__builtin_amdgcn_readlane((int)link[i], best_lane) >> 8);
+            for (int i = 0; i < NS; ++i)
+                if (best_slot == i) {
+                    child = (int)((uint32_t)__builtin_amdgcn_readlane((int)e.link[i], best_lane) >> 8);
+                    best = __builtin_amdgcn_readlane(e.eid[i], best_lane);
+                }
         }
         if (child <= 0 || child >= g.max_nodes) {   // no edge with a comparable score, or a link that leads nowhere
             if (lane == 0) {
@@ -402,10 +378,10 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
             continue;
         }
 #pragma unroll
-        for (int i = 0; i < kSlices; ++i)
-            if (best_slice == i && lane == best_lane) {
-                den[i] += 1;
-                link[i] += 1u;
+        for (int i = 0; i < NS; ++i)
+            if (best_slot == i && lane == best_lane) {
+                e.den[i] += 1;
+                e.link[i] += 1u;
             }
         total += 1;
         if (lane == 0) {
@@ -413,9 +389,118 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
             next[j] = child;
         }
     }
+}
+
+// The traversals of a tree descend in lockstep, one level per round.  The traversals that stand on the same node are
+// served by one wavefront (that of the first of them), which loads the node's edges once and lets the traversals decide
+// one after another, wid ascending, on registers: every decision is the reference's (progressive widening, expansion
+// ticket, score, order on edges with the rotated tie-break: src/puct/puct_gpu_v3_cpp.cu:150-275) on the state that the
+// claims of the traversals before it have left.  Taking the claims in turn is one of the interleavings the reference's
+// atomics allow, needs no atomics itself, never loses a claim and makes a search reproducible.
+__device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *next, int tree, int node, uint64_t members,
+                             int depth, int wave, int lane, uint32_t &nodes_read, uint32_t &edges_scored) {
+    const size_t nrow = (size_t)tree * g.max_nodes + node;
+    Edge *row = g.edges + nrow * kEdges;
+    // all 256 edge slots are requested together with the node's own word, before anything about the node is known: one
+    // round trip per level, whatever the node's width
+    Edge loaded[kSlices];
 #pragma unroll
-    for (int i = 0; i < kSlices; ++i)
-        if (link[i] != link_loaded[i]) row[lane + i * kWave].link = link[i];
+    for (int i = 0; i < kSlices; ++i) loaded[i] = load_edge(row + lane + i * kWave);
+    const NodeInfo ni = load_info(g.info + nrow);
+    const int expanded = ni.expanded;
+    nodes_read += 1;
+    if (expanded == PUCT_NODE_EXPANDED_TERMINAL || depth >= g.path_depth) {
+        const int kind = expanded == PUCT_NODE_EXPANDED_TERMINAL ? PUCT_SELECT_TERMINAL : PUCT_SELECT_DEPTH_LIMIT;
+        if (lane < kTrav && ((members >> lane) & 1ull)) {
+            s.sel[lane] = pack_sel(kind, node, 0);
+            s.len[lane] = depth + 1;
+            s.claims[lane] = depth;
+            next[lane] = -1;
+        }
+        return;
+    }
+    edges_scored += (uint32_t)expanded;
+
+    EdgeSet<kSlices> all;
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < kSlices; ++i) {
+        const Edge e = loaded[i];
+        const bool valid = lane + i * kWave < expanded;
+        all.q[i] = valid && e.n > 0 ? e.w / (float)e.n : 0.0f;
+        all.cp[i] = g.cpuct * e.prior;
+        all.link[i] = all.link_loaded[i] = e.link;
+        all.den[i] = e.n + (int)(e.link & 0xFFu) + 1;
+        all.eid[i] = valid ? lane + i * kWave : -1;
+        total += valid ? all.den[i] - 1 : 0;
+    }
+    total = wave_sum(total);
+    int tickets = ni.tickets;
+    const int legal = ni.legal_turn & 0xFFFF, n_members = __popcll(members);
+
+    if (expanded <= kWave) {
+        EdgeSet<1> one{{all.q[0]}, {all.cp[0]}, {all.den[0]}, {all.link[0]}, {all.link_loaded[0]}, {all.eid[0]}};
+        decide_in_turn<1>(g, s, paths, next, one, node, members, depth, lane, expanded, legal, total, tickets);
+        if (one.link[0] != one.link_loaded[0]) row[lane].link = one.link[0];
+    } else {
+        // A wide node with several traversals on it: most edges cannot come first for any of them.  While these
+        // traversals decide, sqrt(parent) only grows (by their own claims) and an edge's claims only grow, and every
+        // operation of the score is monotonic, so an edge's score stays below its score at the largest sqrt(parent) and
+        // its present claims, and the best edge's score stays above the largest score at the present sqrt(parent) with
+        // all of these traversals' claims on it.  Edges whose upper bound is below that lower bound are out; when at
+        // most 64 remain they move to one edge per lane and a decision costs one division instead of four.
+        bool pruned = false;
+        if (n_members >= 3) {
+            const int now = total > 1 ? total : 1, then = total + n_members > 1 ? total + n_members : 1;
+            const float sqrt_now = sqrtf((float)now), sqrt_then = sqrtf((float)then);
+            uint32_t low = 0, high[kSlices];
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) {
+                const uint32_t l = all.eid[i] >= 0 ? score_image(edge_score(all, i, sqrt_now, n_members)) : 0u;
+                high[i] = all.eid[i] >= 0 ? score_image(edge_score(all, i, sqrt_then, 0)) : 0u;
+                low = l > low ? l : low;
+            }
+            low = wave_max_u32(low);
+            int kept = 0, place[kSlices];
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i) {
+                const bool in = low != 0 && high[i] >= low && high[i] != 0;
+                const uint64_t mask = __ballot(in);
+                place[i] = in ? kept + __popcll(mask & lanes_below(lane)) : -1;
+                kept += __popcll(mask);
+            }
+            if (kept >= 1 && kept <= kWave && low != 0) {
+                pruned = true;
+                // through LDS into one edge per lane
+                EdgeSet<1> few{{0.0f}, {0.0f}, {1}, {0u}, {0u}, {-1}};
+                int *stage = s.stage[wave];
+#pragma unroll
+                for (int f = 0; f < 5; ++f) {
+#pragma unroll
+                    for (int i = 0; i < kSlices; ++i)
+                        if (place[i] >= 0)
+                            stage[place[i]] = f == 0 ? __float_as_int(all.q[i]) : f == 1 ? __float_as_int(all.cp[i]) : f == 2 ? all.den[i]
+                                            : f == 3 ? (int)all.link[i] : all.eid[i];
+                    wave_lds_fence();
+                    const int v = lane < kept ? stage[lane] : 0;
+                    wave_lds_fence();
+                    if (f == 0) few.q[0] = __int_as_float(v);
+                    if (f == 1) few.cp[0] = __int_as_float(v);
+                    if (f == 2) few.den[0] = lane < kept ? v : 1;
+                    if (f == 3) few.link[0] = few.link_loaded[0] = (uint32_t)v;
+                    if (f == 4) few.eid[0] = lane < kept ? v : -1;
+                }
+                decide_in_turn<1>(g, s, paths, next, few, node, members, depth, lane, expanded, legal, total, tickets);
+                if (few.eid[0] >= 0 && few.link[0] != few.link_loaded[0]) row[few.eid[0]].link = few.link[0];
+            }
+        }
+        if (!pruned) {
+            decide_in_turn<kSlices>(g, s, paths, next, all, node, members, depth, lane, expanded, legal, total, tickets);
+#pragma unroll
+            for (int i = 0; i < kSlices; ++i)
+                if (all.link[i] != all.link_loaded[i]) row[lane + i * kWave].link = all.link[i];
+        }
+    }
     if (lane == 0 && tickets != ni.tickets) g.info[nrow].tickets = tickets;
 }
 
@@ -443,7 +528,7 @@ __device__ void select_phase(const LoopArgs &g, StepLds &s, int *paths, int tree
         if (mine < 0) {
             if (lane == 0) next[wave] = -1;
         } else if ((members & lanes_below(wave)) == 0) {
-            select_group(g, s, paths, next, tree, mine, members, depth, lane, nodes_read, edges_scored);
+            select_group(g, s, paths, next, tree, mine, members, depth, wave, lane, nodes_read, edges_scored);
         }
         __syncthreads();
     }
