@@ -559,6 +559,7 @@ __device__ void expand_phase(const LoopArgs &g, StepLds &s, int tree, int wave, 
     const bool wants = kind == PUCT_SELECT_EXPAND && ticket_slot < n_legal;
     if (lane == 0) s.want[wave] = wants ? node : -1;
     __syncthreads();
+    if (FARM) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the evaluators' priors of the step before (see search_kernel)
     const int other = lane < n_waves ? s.want[lane] : -1;
     const uint64_t all = __ballot(other >= 0), here = __ballot(other >= 0 && other == node);
     const int total = __popcll(all), before = __popcll(all & lanes_below(wave));
@@ -894,6 +895,19 @@ __device__ void evaluator_loop(const LoopArgs &g, EvalLds &L, int tree, int help
     }
 }
 
+// Until the evaluators have worked off everything handed to them so far; gives up after a bounded wait.
+__device__ void wait_for_evaluators(EvalRequests &rq, StepLds &s) {
+    const uint64_t start = wall_clock64();
+    while (poll_word(&rq.done) < s.requested) {
+        if (poll_word(&rq.abort) != 0 || wall_clock64() - start > kWaitTicks) {
+            __hip_atomic_store(&rq.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s.gave_up = 1;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
+
 // The whole search in one launch.  evaluators == 0: one workgroup per tree (grid = trees).  Otherwise every tree has
 // 1 + evaluators workgroups; those of one tree have the same blockIdx.x % 8, which is how workgroups are dealt to the
 // eight XCDs, so a tree's requests and results meet in one L2.
@@ -931,11 +945,16 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, 
         work.count_kind(s, wave);
         uint64_t t1 = 0, t2 = 0;
         if (wave == 0) t1 = wall_clock64();
-        if (farm)
+        if (farm) {
+            // A node created in the step before can be expanded now at the earliest (selection hands out tickets without
+            // looking at a node's priors), so this is where its priors must be there, not a step's length earlier.
+            if (threadIdx.x == 0) wait_for_evaluators(rq, s);
             expand_phase<true>(g, s, tree, wave, lane, n_waves, work.created);
-        else
+        } else {
             expand_phase<false>(g, s, tree, wave, lane, n_waves, work.created);
+        }
         phase_barrier();   // the claims of the selection and the new nodes are in memory
+        if (s.gave_up) break;
         if (farm && threadIdx.x == 0) {   // ... and the evaluators may start on this step's nodes
             rq.n = s.requests;
             s.requested += s.requests;
@@ -944,19 +963,7 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, 
         }
         if (wave == 0) t2 = wall_clock64();
         backup_phase(g, s, paths, tree, wave, lane, n_waves);
-        if (farm && threadIdx.x == 0) {   // the next selection may descend into the new nodes: their priors must be there
-            const uint64_t start = wall_clock64();
-            while (poll_word(&rq.done) < s.requested) {
-                if (poll_word(&rq.abort) != 0 || wall_clock64() - start > kWaitTicks) {
-                    __hip_atomic_store(&rq.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    s.gave_up = 1;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-        }
         phase_barrier();
-        if (s.gave_up) break;
         if (wave == 0) {
             const uint64_t t3 = wall_clock64();
             work.ticks[0] += t1 - t0;
@@ -964,6 +971,10 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, 
             work.ticks[2] += t3 - t2;
             t0 = t3;
         }
+    }
+    if (farm) {   // the last step's nodes
+        if (threadIdx.x == 0) wait_for_evaluators(rq, s);
+        __syncthreads();
     }
     if (farm && threadIdx.x == 0) __hip_atomic_store(&rq.tag, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     state_to_memory(g, s, paths, tree, n_waves);

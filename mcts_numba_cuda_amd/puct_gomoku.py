@@ -79,7 +79,7 @@ class PUCTGomoku:
     visits; `root_n`, `root_q`, `selections`, `performance_info` describe the last search."""
 
     def __init__(self, board_shape=(15, 15), trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5,
-                 c_pw=1.0, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, device=0, evaluators=8):
+                 c_pw=1.0, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, device=0, evaluators=4):
         self.cfg = Config(int(board_shape[0]), int(board_shape[1]), int(trees), int(traversals), int(max_nodes),
                           int(path_depth), float(cpuct), float(c_pw), float(alpha_pw), float(dirichlet_alpha), int(seed),
                           int(device), int(evaluators))
