@@ -290,16 +290,19 @@ __device__ __forceinline__ float edge_score(const EdgeSet<NS> &e, int i, float s
 template <int NS>
 __device__ __forceinline__ void decide_in_turn(const LoopArgs &g, StepLds &s, int *paths, int *next, EdgeSet<NS> &e, int node,
                                                uint64_t members, int depth, int lane, int expanded, int legal, int &total,
-                                               int &tickets) {
+                                               int &tickets, bool only_one = false) {
+    // sqrt(parent) and the widening limit after 0, 1, 2 ... more claims, worked out side by side in lanes 0..15 (fewer
+    // than 64 traversals decide here, and every claim adds one to the node's total)
+    const bool widening = expanded != 1 || g.c_pw != 0.0f;
+    const int claims_base = total;
+    const int eff_lane = widening ? (total + lane > 1 ? total + lane : 1) : 1;
+    const float sqrt_lane = widening ? sqrtf((float)eff_lane) : 1.0f;
+    const int allowed_lane = widening ? allowed_children(g.c_pw, g.alpha_pw, eff_lane, sqrt_lane, legal) : 1;
     for (uint64_t rest = members; rest != 0; rest &= rest - 1) {
         const int j = __builtin_ctzll(rest);   // the traversal deciding now
-        int parent_eff = 1, allowed = 1;
-        float sqrt_parent = 1.0f;
-        if (expanded != 1 || g.c_pw != 0.0f) {
-            parent_eff = total > 1 ? total : 1;
-            sqrt_parent = sqrtf((float)parent_eff);
-            allowed = allowed_children(g.c_pw, g.alpha_pw, parent_eff, sqrt_parent, legal);
-        }
+        const int claimed = total - claims_base;
+        const float sqrt_parent = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sqrt_lane), claimed));
+        const int allowed = __builtin_amdgcn_readlane(allowed_lane, claimed);
         if (allowed > expanded) {
             if (expanded + tickets < allowed) {   // expansion ticket
                 if (lane == 0) {
@@ -325,7 +328,7 @@ __device__ __forceinline__ void decide_in_turn(const LoopArgs &g, StepLds &s, in
         // one edge attains it does the rotated edge index decide, through the full keys.  (A node's only edge is taken
         // whatever its score, as in the reference.)
         int best_lane = 0, best_slot = 0, hits = 1;
-        if (expanded > 1) {
+        if (expanded > 1 && !only_one) {
             float score[NS];
             uint32_t image[NS], lane_top = 0;
 #pragma unroll
@@ -490,7 +493,7 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
                     if (f == 3) few.link[0] = few.link_loaded[0] = (uint32_t)v;
                     if (f == 4) few.eid[0] = lane < kept ? v : -1;
                 }
-                decide_in_turn<1>(g, s, paths, next, few, node, members, depth, lane, expanded, legal, total, tickets);
+                decide_in_turn<1>(g, s, paths, next, few, node, members, depth, lane, expanded, legal, total, tickets, kept == 1);
                 if (few.eid[0] >= 0 && few.link[0] != few.link_loaded[0]) row[few.eid[0]].link = few.link[0];
             }
         }
