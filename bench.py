@@ -54,7 +54,20 @@ def profile_json(name):
     except ValueError:
         return None
     d["file"] = "profiles/" + name
+    # A summary that records the hashes of its kernel's source files can say whether they have changed since the counters
+    # were taken (None: the summary holds no hashes).
+    d["stale"] = None
+    if isinstance(d.get("kernel_sources"), dict):
+        d["stale"] = any(source_hash(path) != h for path, h in d["kernel_sources"].items())
     return d
+
+
+def source_hash(path):
+    import hashlib
+    try:
+        return hashlib.sha256(open(os.path.join(ROOT, path), "rb").read()).hexdigest()[:16]
+    except OSError:
+        return None
 
 
 def valu_roofline(insts, seconds, source, what):
@@ -65,7 +78,10 @@ def valu_roofline(insts, seconds, source, what):
     achieved = insts / seconds / 1e9
     return {"bound": "valu", "achieved": achieved, "peak": VALU_PEAK_G, "unit": "G wavefront instructions/s", "frac": achieved / VALU_PEAK_G,
             "formula": "SQ_INSTS_VALU x 4 / (1024 SIMDs x kernel time x 2.4 GHz)", "what": what,
-            "counter_file": source.get("file"), "counter_commit": source.get("commit")}
+            "counter_file": source.get("file"), "counter_commit": source.get("commit"),
+            # the instruction count comes from the counter summary, the time from this run: true if the kernel's sources
+            # have changed since the counters were taken, None if the summary does not record their hashes
+            "stale": source.get("stale")}
 
 
 def has_four(board, token):
@@ -341,78 +357,111 @@ def bench_gomoku(args):
     print(json.dumps(out))
 
 
-def bench_puct_gomoku(args):
-    """PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step,
-    Dirichlet(0.3) priors and hashed values, c_puct = 1.5, 4000 steps; one bench step = one whole search."""
+def puct_gomoku_search(board, steps, search_steps, warmup, **kw):
+    """`steps` timed searches of `search_steps` steps each; returns totals and the algorithmic bytes by phase."""
     from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
-    steps = args.steps if args.steps != N_ROOTS else 5
-    search_steps = 4000
-    prof = profile_json("search_kernel_puct_gomoku_16_trees_x16.md")
-    board = np.zeros((15, 15), np.int8)
-    e = PUCTGomoku(trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0, alpha_pw=0.5,
-                   recalc_attempts=16, dirichlet_alpha=0.3, seed=0)
-    for _ in range(max(args.warmup, 1)):
+    e = PUCTGomoku(**kw)
+    for _ in range(max(warmup, 1)):
         e.run(board, 1, 200)
-    sel = useful = nodes = 0
-    dev = 0.0
-    alg = dict(select=0, expand=0, backup=0, total=0)
-    # legal cells of the nodes a search creates (priors are written for each): the trees are the same in every timed
-    # search but for races, so one look at the warm-up's arrays serves all
+    # legal cells of the nodes a search creates (a 16-byte record and a cell byte are written for each): the trees are the
+    # same in every search, so one look at one search's arrays serves all
     e.run(board, 1, search_steps)
     counts, legal_arr, expanded_arr = e.read_array("node_count"), e.read_array("node_legal"), e.read_array("node_expanded")
     created = sum(int(c) - 1 for c in counts)
     legal_per_created = sum(int(legal_arr[t, 1:c][expanded_arr[t, 1:c] != -1].sum()) for t, c in enumerate(counts)) / max(created, 1)
+    tot = dict(selections=0, leaves=0, busy=0, nodes=0, dev=0.0, select=0.0, expand=0.0, backup=0.0)
+    alg = dict(select=0, expand=0, backup=0, total=0)
     t0 = time.perf_counter()
     for _ in range(steps):
         e.run(board, 1, search_steps)
-        sel += e.performance_info["selections"]
-        useful += e.performance_info["selections"] - e.selections["busy"]
-        nodes += e.performance_info["nodes_total"]
-        dev += e.result.time_device
-        # Algorithmic bytes with the element sizes of the reference's arrays (src/puct/puct_gpu_v2.py:69-103): a level read
-        # costs the node word, the ticket counter and five 4-byte fields per expanded edge; a selection writes its word,
-        # its length and 4 bytes per path entry; an expansion reads the parent's position and action, writes the child's
-        # position (128 B), turn, value, counters (17 B), links it (12 B) and writes 21 bytes per legal cell of the child
-        # (prior, action, child, N, W, in-flight); the backup reads 8 bytes and updates three 4-byte words per path edge.
-        r = e.result
-        path_edges = r.levels_read - sum(r.selections)          # every selection read one level more than it descended edges
+        p, r = e.performance_info, e.result
+        tot["selections"] += p["selections"]
+        tot["leaves"] += p["leaves"]
+        tot["busy"] += e.selections["busy"]
+        tot["nodes"] += p["nodes_total"]
+        tot["dev"] += r.time_device
+        for k in ("select", "expand", "backup"):
+            tot[k] += getattr(r, "time_" + k)
+        # Algorithmic bytes of the loop's own layout.  Selection: a node that a group of traversals stands on is read once
+        # (16-byte node word + one 16-byte record per expanded edge), a claim rewrites the edge's 4-byte link word and
+        # adds a 4-byte path entry, every traversal leaves 12 bytes (selection word, length, claims).  Expansion: parent
+        # position and node word in (64 + 16), the slot's cell in (1), child position, node word and link out (64 + 16 +
+        # 12), one 16-byte record and one cell byte per legal cell of the child.  Backup: three 4-byte words of every
+        # path edge in and out (24).
         legal_cells = legal_per_created * r.expansions_committed
-        b_sel = 8 * r.levels_read + 20 * r.edges_examined + 8 * sum(r.selections) + 4 * path_edges
-        b_exp = r.expansions_committed * (128 + 1 + 128 + 17 + 12) + 21 * legal_cells
-        b_bak = 32 * path_edges
-        for key, v in (("select", b_sel), ("expand", b_exp), ("backup", b_bak), ("total", b_sel + b_exp + b_bak)):
-            alg[key] += v
+        b_sel = 16 * r.nodes_read + 16 * r.edges_scored + 12 * p["selections"]
+        b_exp = r.expansions_committed * (64 + 16 + 1 + 64 + 16 + 12) + 17 * legal_cells
+        alg["select"] += b_sel
+        alg["expand"] += b_exp
     wall = time.perf_counter() - t0
+    # path edges: every visit of an edge was a path entry of a traversal that reached a node; visits = sum over all
+    # edges of n minus the visit each child got at its creation.  Claims of busy traversals are not counted (few bytes).
+    edge_n = e.read_array("edge_n")
+    visits = 0
+    for t, c in enumerate(counts):
+        rows = edge_n[t, :c]
+        ne = np.maximum(expanded_arr[t, :c], 0)
+        visits += int(rows[np.arange(256)[None, :] < ne[:, None]].sum()) - (int(c) - 1)
+    del edge_n
+    alg["select"] += 8 * visits * steps
+    alg["backup"] = 24 * visits * steps
+    alg["total"] = alg["select"] + alg["expand"] + alg["backup"]
+    e.close()
+    return tot, alg, wall
+
+
+def bench_puct_gomoku(args):
+    """PUCT on Gomoku 15x15 with virtual loss, 16 trees x 16 traversals = 256 leaves per step, Dirichlet(0.3) priors and
+    hashed values, c_puct = 1.5, 4000 steps; one bench step = one whole search.  c_pw = 16: a node without children
+    admits a ticket per traversal, so every selection reaches a leaf; the reference's default c_pw = 1 is timed beside it
+    (most traversals of a step then end busy behind the first to reach a new node: that follows from the widening rule,
+    the host oracle shows the same share)."""
+    steps = args.steps if args.steps != N_ROOTS else 5
+    search_steps = 4000
+    prof = profile_json("search_kernel_puct_gomoku_16_trees_x16.md")
+    board = np.zeros((15, 15), np.int8)
+    kw = dict(trees=16, traversals=16, path_depth=64, cpuct=1.5, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0)
+    tot, alg, wall = puct_gomoku_search(board, steps, search_steps, args.warmup, c_pw=16.0, max_nodes=65536, **kw)
+    ref, _, ref_wall = puct_gomoku_search(board, max(steps // 2, 1), search_steps, 1, c_pw=1.0, max_nodes=16384, **kw)
+    dev, n_steps = tot["dev"], steps * search_steps
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import puct_oracle as po
         t1 = time.perf_counter()
-        h = po.gomoku_search(board, 1, 250, trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5, c_pw=1.0,
-                             dirichlet_alpha=0.3, seed=0)
+        h = po.gomoku_search(board, 1, 1000, c_pw=16.0, max_nodes=16384, threads=1, **kw)
         dt = time.perf_counter() - t1
-        cpu = {"value": 250 * 256 / dt, "unit": "selections/s", "cores": 1, "kind": "port",
-               "sample": "the same search for 250 steps (64000 selections), sequential CPU oracle",
-               "selections_not_busy_per_s": int(h["tally"][:, 1:4].sum()) / dt}
-    out = {"metric": "PUCT selections/s, Gomoku 15x15 search loop with virtual loss (16 trees x 16 traversals)",
-           "value": sel / wall, "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+        cpu = {"value": int(h["tally"][:, 1:4].sum()) / dt, "unit": "leaves/s", "cores": 1, "kind": "port",
+               "sample": "the same search for 1000 steps (256000 selections, all of them leaves), host oracle on one core"}
+    out = {"metric": "PUCT leaves/s (selections that reach a node and are evaluated and backed up), Gomoku 15x15 search loop "
+                     "with virtual loss (16 trees x 16 traversals)",
+           "value": tot["leaves"] / wall, "unit": "leaves/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
            "ms_per_step": wall / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-           "dtype": "f32 scores + int32 atomics", "data": "synthetic",
+           "dtype": "f32 scores, int32 counters, claims in a fixed order (no atomics)", "data": "synthetic",
            "config": {"workload": "Gomoku 15x15 empty board, 16 trees x 16 traversals per step, Dirichlet(0.3) priors and hashed "
-                                  "values, c_puct=1.5, c_pw=1.0, alpha_pw=0.5, 16 claim attempts, 4000 steps per search, "
-                                  "node limit 16384 per tree"},
-           "search_steps_per_s": steps * search_steps / wall, "selections_not_busy_per_s": useful / wall,
-           "nodes_created_per_search": nodes / steps, "device_share": dev / wall,
+                                  "values, c_puct=1.5, c_pw=16, alpha_pw=0.5, 4000 steps per search, room for 65536 nodes per "
+                                  "tree (64001 used), 4 evaluator workgroups per tree"},
+           "selections_per_s": tot["selections"] / wall, "busy_share": tot["busy"] / tot["selections"],
+           "leaves_per_step": tot["leaves"] / n_steps, "search_steps_per_s": n_steps / wall,
+           "nodes_created_per_search": tot["nodes"] / steps, "device_share": dev / wall,
+           "us_per_search_step": {"total": dev / n_steps * 1e6, "select": tot["select"] / n_steps * 1e6,
+                                  "expand": tot["expand"] / n_steps * 1e6, "backup": tot["backup"] / n_steps * 1e6},
+           "stage_achieved_gbs": {k: alg[k] / max(tot[k], 1e-12) / 1e9 for k in ("select", "expand", "backup")},
+           "reference_default_widening": {
+               "config": "c_pw=1 (src/puct/puct_gpu_v3_cpp.py:121), room for 16384 nodes per tree, otherwise the same",
+               "leaves_per_s": ref["leaves"] / ref_wall, "selections_per_s": ref["selections"] / ref_wall,
+               "busy_share": ref["busy"] / ref["selections"], "leaves_per_step": ref["leaves"] / (max(steps // 2, 1) * search_steps),
+               "search_steps_per_s": max(steps // 2, 1) * search_steps / ref_wall},
            "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
-                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit")} if prof else None,
+                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
                         "kernel": "puct::search_kernel (select, expand, backup of all 4000 steps in one launch)",
                         "algorithmic_bytes_per_launch": alg["total"] / steps, "avg_launch_ms": dev / steps * 1e3,
                         "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
-                        "note": "16 workgroups of 16 wavefronts: bound by the dependent L2 round trips of a level (edge rows, claim, "
-                                "recalculation) and the fp64 Gamma sampling of an expansion, not by memory"},
+                        "note": "16 tree workgroups of 16 wavefronts and 64 evaluator workgroups of 8: a step is a chain of dependent "
+                                "decisions (the traversals on one node decide in turn) and one round trip per tree level, "
+                                "not a stream"},
            "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_launch"), dev / steps, prof or {}, "one search of 4000 steps"),
            "cpu_baseline": cpu}
-    e.close()
     print(json.dumps(out))
 
 
