@@ -62,6 +62,16 @@ def profile_json(name):
     return d
 
 
+PLAIN_LAUNCH = False
+
+
+def apply_launch_options(engine):
+    """--plain-launch: the all-children kernels as ordinary launches (profilers and the runtime's cooperative queue do not
+    get along: a rocprofv3 process that has made a cooperative launch ends with SIGSEGV in the runtime's exit handler)."""
+    if PLAIN_LAUNCH:
+        engine.set_option("plain_launch", 1)
+
+
 def source_hash(path):
     import hashlib
     try:
@@ -278,6 +288,7 @@ def bench_gomoku(args):
         e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=2000, n_trees=4, n_playouts=128,
                    variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
         e.init_device_side_arrays()
+        apply_launch_options(e)
         for w in range(max(args.warmup, 1)):
             e.reseed()
             e.run(roots[w][0], None, roots[w][1])
@@ -305,6 +316,7 @@ def bench_gomoku(args):
                 x = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=2000, n_trees=4, n_playouts=128,
                            variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
                 x.init_device_side_arrays()
+                apply_launch_options(x)
                 engines.append(x)
             for rep in range(2):    # first pass warms the pools up
                 for x in engines:
@@ -481,6 +493,7 @@ def bench_c4_many(args):
             e = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=T, n_playouts=P,
                        variant="acp_prodigal", device_memory=0.06, ucb_c=2.0, seed=0, verbose_info=False)
             e.init_device_side_arrays()
+            apply_launch_options(e)
             engines.append(e)
         chunk = [roots[i % len(roots)] for i in range(n)]
         times = []
@@ -522,6 +535,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-batched", action="store_true")
+    ap.add_argument("--plain-launch", action="store_true",
+                    help="launch the kernels whose workgroups wait for each other as ordinary kernels (for profilers)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by) and exit")
@@ -531,6 +546,8 @@ def main():
     ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
     ap.add_argument("--searches", type=int, default=768, help="c4_many: concurrent searches in the pass")
     args = ap.parse_args()
+    global PLAIN_LAUNCH
+    PLAIN_LAUNCH = args.plain_launch
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (trees are independent and would shard over GPUs with one "
                  "final all-reduce of the root table, but no multi-GPU path is part of it); run with --gpus 1")
@@ -566,6 +583,7 @@ def main():
         e = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=T, n_playouts=P,
                    variant="acp_prodigal", device_memory=DEVICE_MEMORY, ucb_c=2.0, seed=0, verbose_info=False)
         e.init_device_side_arrays()
+        apply_launch_options(e)
         return e
 
     with contextlib.redirect_stdout(quiet):
@@ -629,6 +647,7 @@ def main():
             wide = MCTSNC((M, N), A, A, search_time_limit=np.inf, search_steps_limit=STEPS, n_trees=512, n_playouts=P,
                           variant="acp_prodigal", device_memory=16.0, ucb_c=2.0, seed=0, verbose_info=False)
             wide.init_device_side_arrays()
+            apply_launch_options(wide)
             b, f, t = np.zeros((M, N), np.int8), np.zeros(N, np.int8), 1     # empty board
             for rep in range(2):
                 wide.reseed()

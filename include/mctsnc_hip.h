@@ -154,6 +154,45 @@ int mctsnc_run_batch_noalloc(mctsnc_engine **engines, int32_t n, const int8_t *b
                              const int32_t *turns, double steps_limit, double time_limit_s, double forced_steps_limit,
                              mctsnc_result *out);
 
+/* How the search is laid out on the device and test hooks; none of them changes a search's results.  No counterpart in
+ * the reference (it has one launch shape per kernel).  A batch call takes the options of its first engine.
+ *   MCTSNC_OPT_AGENT_FENCES       1: the all-children kernels never take the shortcuts for trees whose workgroups share an
+ *                                 XCC (full device-scope release and acquire every step: the path such trees take when
+ *                                 they do not); 0 (default)
+ *   MCTSNC_OPT_SOLO_TREES         Connect 4, all children: one workgroup per tree from this many trees of a pass on;
+ *                                 0 = never, -1 (default) = by the number of trees per compute unit
+ *   MCTSNC_OPT_SOLO_THREADS       threads of such a workgroup, a multiple of 64 up to 512; 0 (default) = by the playouts
+ *   MCTSNC_OPT_TEAM_POOL          Connect 4, all children: a team's workgroups play their playouts as a pool of jobs on
+ *                                 fewer lanes; 1 / 0 = always / never, -1 (default) = by the number of trees
+ *   MCTSNC_OPT_TEAM_POOL_THREADS  lanes of such a workgroup, a multiple of 64 up to 512; 0 (default) = half the playouts
+ *   MCTSNC_OPT_PREP_LEVELS        Gomoku, one child: the backup of paths up to this many levels is prepared during the
+ *                                 playouts (at most 48); -1 (default) = 48
+ *   MCTSNC_OPT_PLAIN_LAUNCH       1: the all-children kernels, whose workgroups wait for each other, are launched as
+ *                                 ordinary kernels instead of cooperatively (same grid, sized to what the device keeps
+ *                                 resident; what is given up is the runtime's guarantee of residency when other kernels
+ *                                 share the device: a workgroup that never gets scheduled then ends the launch with
+ *                                 MCTSNC_E_DEVICE_SYNC through the bounded waits).  For profilers that do not get along
+ *                                 with the runtime's cooperative queue; 0 (default)
+ *   MCTSNC_OPT_PROBE_STEPS        Connect 4 pass with more trees than stay resident: steps every tree runs before the
+ *                                 searches are put in the order of what they cost; 0 = keep the order by stones,
+ *                                 -1 (default) = a thirty-second of the step budget, 16 to 128
+ *   MCTSNC_OPT_SPIN_LIMIT         polls after which a workgroup's wait for the others of its tree gives up and ends the
+ *                                 launch (MCTSNC_E_DEVICE_SYNC); 0 (default) = 2^24.  1 makes the first wait that is not
+ *                                 met at once give up: the hook with which the tests drive that path.
+ * After MCTSNC_E_DEVICE_SYNC the search is void, the engines stay usable and their random streams are back at their
+ * seeds (as after mctsnc_reseed). */
+#define MCTSNC_OPT_AGENT_FENCES 0
+#define MCTSNC_OPT_SOLO_TREES 1
+#define MCTSNC_OPT_SOLO_THREADS 2
+#define MCTSNC_OPT_TEAM_POOL 3
+#define MCTSNC_OPT_TEAM_POOL_THREADS 4
+#define MCTSNC_OPT_PREP_LEVELS 5
+#define MCTSNC_OPT_PLAIN_LAUNCH 6
+#define MCTSNC_OPT_PROBE_STEPS 7
+#define MCTSNC_OPT_SPIN_LIMIT 8
+#define MCTSNC_OPT_COUNT 9
+int mctsnc_set_option(mctsnc_engine *e, int32_t option, int32_t value);
+
 /* Switches the per-stage device timers on (default) or off. */
 int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on);
 

@@ -43,6 +43,10 @@ ARRAYS = {  # name -> (id, dtype, trailing shape builder)
     "rng_playout": (15, np.uint64), "rng_expand": (16, np.uint64),
 }
 
+# mctsnc_set_option(): names of the MCTSNC_OPT_* constants of include/mctsnc_hip.h
+OPTIONS = {"agent_fences": 0, "solo_trees": 1, "solo_threads": 2, "team_pool": 3, "team_pool_threads": 4, "prep_levels": 5,
+           "plain_launch": 6, "probe_steps": 7, "spin_limit": 8}
+
 _lib = None
 
 
@@ -79,6 +83,8 @@ def lib():
         L.mctsnc_read.argtypes = [vp, ctypes.c_int32, ctypes.c_int32, vp, ctypes.c_size_t]
         L.mctsnc_reseed.restype = ctypes.c_int
         L.mctsnc_reseed.argtypes = [vp]
+        L.mctsnc_set_option.restype = ctypes.c_int
+        L.mctsnc_set_option.argtypes = [vp, ctypes.c_int32, ctypes.c_int32]
         L.mctsnc_set_stage_timing.restype = ctypes.c_int
         L.mctsnc_set_stage_timing.argtypes = [vp, ctypes.c_int32]
         L.mctsnc_destroy.restype = None

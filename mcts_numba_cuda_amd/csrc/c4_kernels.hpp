@@ -104,6 +104,7 @@ struct SearchArgs {
     int32_t stage_timing;   // accumulate per-stage device time in the tree headers
     int32_t agent_fences;   // never take the same-XCC shortcuts (full device-scope release and acquire every step)
     int32_t *abort_flag;
+    uint32_t spin_limit;    // polls after which a bounded wait gives up and ends the launch
     int32_t *queue;         // next tree not yet handed out, or null when every tree has its own workgroups
     uint32_t launch_seq;    // distinguishes the launches that use the queue
 };
@@ -730,7 +731,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                             uint32_t spins = 0;
                             while (atomicCAS(&s_lock, 0u, 1u) != 0u) {
                                 __builtin_amdgcn_s_sleep(4);
-                                if (++spins > kSpinLimit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                                if (++spins > args.spin_limit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
                             }
                         }
                         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -879,7 +880,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
                         if ((uint32_t)(v >> 32) == gen + 1u) break;
                         __builtin_amdgcn_s_sleep(1);
                         // a bounded wait: a lost workgroup must end the launch, never hang the device
-                        if (++spins > kSpinLimit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); bad = true; break; }
+                        if (++spins > args.spin_limit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); bad = true; break; }
                         if ((spins & 1023u) == 0 && __hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { bad = true; break; }
                     }
                 }
@@ -1023,7 +1024,10 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
         if (tid < kMaxCols) { hdr->poc[tid][0] = s_poc[tid][0]; hdr->poc[tid][1] = s_poc[tid][1]; }
         if (tid <= s_t.L && tid < kMaxPath) hdr->path[tid] = s_pnode[tid];
     }
-    if (SOLO) {
+    // (a launch that a bounded wait ended leaves the streams as it found them, like the tree headers: the host reports
+    // the failure and the search is void)
+    if (s_abort) {
+    } else if (SOLO) {
         uint64_t *p = const_cast<uint64_t *>(ref.rng_playout);
         for (int i = tid; i < ncols * P * 2; i += blockDim.x) p[i] = s_rng[i];
     } else if (POOL) {
@@ -1033,7 +1037,7 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
         uint64_t *p = ref.rng_playout + 2 * ((size_t)(ACP ? g * P : 0) + tid);
         p[0] = s0; p[1] = s1;
     }
-    if (!ACP && tid == 0) { ref.rng_expand[0] = e0; ref.rng_expand[1] = e1; }
+    if (!ACP && tid == 0 && !s_abort) { ref.rng_expand[0] = e0; ref.rng_expand[1] = e1; }
     for (int off = 32; off > 0; off >>= 1) { plies += __shfl_xor(plies, off); u1 += __shfl_xor(u1, off); }
     if (lane == 0) {
         if (plies) atomicAdd(&hdr->plies, (unsigned long long)plies);
@@ -1076,7 +1080,7 @@ __device__ __forceinline__ void search_trees(const SearchArgs &args) {
                     next = atomicAdd(args.queue, 1);
                     __hip_atomic_store(&hdr->next_job, ((unsigned long long)args.launch_seq << 32) | (uint32_t)(next + 1), __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
                 } else {
-                    for (uint32_t spins = 0; spins <= (kSpinLimit >> 4); spins++) {  // the others of the set finish within microseconds of each other
+                    for (uint32_t spins = 0; spins <= (args.spin_limit >> 4); spins++) {  // the others of the set finish within microseconds of each other
                         const unsigned long long v = __hip_atomic_load(&hdr->next_job, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
                         if ((uint32_t)(v >> 32) == args.launch_seq) { next = (int32_t)(uint32_t)v - 1; break; }
                         if ((spins & 1023u) == 1023u && __hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
@@ -1105,12 +1109,6 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(5, 5))
 // One workgroup per tree: the generators in LDS leave room for four workgroups per CU, i.e. four wavefronts per SIMD
 // and 128 vector registers (with 96 the playout loop spills).
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) search_kernel_solo(SearchArgs args) { search_trees<Connect4, true, true>(args); }
-
-// The same with up to 1024 threads (16 wavefronts: the four per SIMD that 128 registers allow, i.e. one workgroup per CU):
-// all children of a step at once with two playouts per lane, the form closest to a team's step a single workgroup can
-// take.  Only taken on request (MCTSNC_SOLO_THREADS above 512); see the design notes for what it measures.
-__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(4, 4))) search_kernel_solo_wide(SearchArgs args) { search_trees<Connect4, true, true>(args); }
-
 
 // Where the final reductions (reduce_kernels.hpp) find the root's visit count, the row memorised at the first step and
 // the counters of the root's children in this layout: a child's counters sit in the root's own record, slot = action.

@@ -104,6 +104,7 @@ struct SearchArgs {
     int32_t agent_fences;   // never take the same-XCC shortcuts (full device-scope release and acquire every step)
     int32_t prep_levels;    // one-child variants: paths up to this many levels have their backup prepared during the playouts (<= kPrepLevels)
     int32_t *abort_flag;
+    uint32_t spin_limit;    // polls after which a bounded wait gives up and ends the launch
 };
 
 __device__ __forceinline__ bool bb_test(const uint32_t *bb, int cell) { return (bb[cell >> 5] >> (cell & 31)) & 1u; }
@@ -850,7 +851,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 while (atomic_load_relaxed(&hdr->gen) != gen) {
                     __builtin_amdgcn_s_sleep(8);
                     // a bounded wait: a lost workgroup must end the launch, never hang the device
-                    if (++spins > kSpinLimit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); bad = true; break; }
+                    if (++spins > args.spin_limit) { __hip_atomic_store(args.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); bad = true; break; }
                     if ((spins & 1023u) == 0 && __hip_atomic_load(args.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { bad = true; break; }
                 }
                 if (bad) s_abort = 1;
@@ -870,8 +871,8 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
         if (timing) { const unsigned long long t2 = wall_clock64(); tk_backup += t2 - tk; tk = t2; }
     }
 
-    if (!ACP && tid == 0) { ref.rng_expand[0] = e0; ref.rng_expand[1] = e1; }
-    if (keep_rng && tid < P) { uint64_t *w = const_cast<uint64_t *>(ref.rng_playout); w[2 * tid] = k0; w[2 * tid + 1] = k1; }
+    if (!ACP && tid == 0 && !s_abort) { ref.rng_expand[0] = e0; ref.rng_expand[1] = e1; }
+    if (keep_rng && tid < P && !s_abort) { uint64_t *w = const_cast<uint64_t *>(ref.rng_playout); w[2 * tid] = k0; w[2 * tid + 1] = k1; }
     for (int off = 32; off > 0; off >>= 1) { plies += __shfl_xor(plies, off); u1 += __shfl_xor(u1, off); }
     if (lane == 0) {
         if (plies) atomicAdd(&hdr->plies, (unsigned long long)plies);

@@ -99,6 +99,7 @@ struct mctsnc_engine {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     bool has_run = false;
     bool stage_timing = true;
+    int options[MCTSNC_OPT_COUNT] = {0, -1, 0, -1, 0, -1, 0, -1, 0};   // mctsnc_set_option(): defaults, see include/mctsnc_hip.h
     std::vector<uint64_t> rng_init_playout, rng_init_expand;  // the streams as seeded, kept for reseed()
     std::vector<c4::TreeRef> h_refs;          // host copies of the per-tree pointer records (a batch gathers them)
     std::vector<gomoku::TreeRef> hg_refs;
@@ -193,15 +194,21 @@ int upload_rng(mctsnc_engine *e) {
     return MCTSNC_OK;
 }
 
-// MCTSNC_PLAIN_LAUNCH=1: launch the all-children kernels, whose workgroups wait for each other, as ordinary kernels
-// instead of cooperatively.  The grid is sized to what the device keeps resident either way, so on a device that runs
-// nothing else the workgroups are all resident and the search is the same; what is given up is the runtime's guarantee
-// of it when other kernels share the device (a workgroup that never gets scheduled ends the launch with
-// MCTSNC_E_DEVICE_SYNC through the bounded waits, it cannot hang).  For profilers that do not get along with the
-// runtime's cooperative queue.
-bool plain_launch_requested() {
-    const char *v = getenv("MCTSNC_PLAIN_LAUNCH");
-    return v && atoi(v) != 0;
+// A launch that a bounded wait ended (a workgroup of a tree did not turn up): the search is void.  The kernels leave the
+// random streams of such a launch alone where they live in registers, but earlier launches of the same search and the
+// variants that keep their streams in memory have consumed from them, so all engines of the call get the streams they
+// were seeded with, as after mctsnc_reseed(): the next run equals a new engine's first.
+int search_abandoned(mctsnc_engine **engines, int n, int64_t steps) {
+    for (int i = 0; i < n; i++)
+        if (int rc = upload_rng(engines[i])) return rc;
+    return fail(MCTSNC_E_DEVICE_SYNC, "device-side step synchronisation timed out after %lld steps; the search is void and the random "
+                "streams of its engines are back at their seeds", (long long)steps);
+}
+
+// MCTSNC_DEBUG=1 in the environment: print how a pass was laid out on the device (the one thing the environment decides).
+bool debug_enabled() {
+    static const bool on = [] { const char *v = getenv("MCTSNC_DEBUG"); return v && atoi(v) != 0; }();
+    return on;
 }
 
 struct Budget {
@@ -297,7 +304,7 @@ int budget_loop(mctsnc_engine *e0, const Budget &bud, Launch launch, int64_t &st
         steps += nsteps;
         int32_t aborted = 0;
         HIP_TRY(hipMemcpy(&aborted, e0->d_abort, sizeof aborted, hipMemcpyDeviceToHost));
-        if (aborted) return fail(MCTSNC_E_DEVICE_SYNC, "device-side step synchronisation timed out after %lld steps", (long long)steps);
+        if (aborted) return MCTSNC_E_DEVICE_SYNC;   // the caller puts the engines back into a defined state and reports
         if (first_chunk > 0 && steps == nsteps && (double)steps < step_budget) {
             rc = after_first();
             if (rc) return rc;
@@ -487,58 +494,45 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
     args.refs = d_refs; args.n_refs = n_refs; args.m = c.board_m; args.n = c.board_n; args.P = c.n_playouts; args.G = e0->G;
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
-    args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
+    const int *opt = e0->options;
+    args.agent_fences = opt[MCTSNC_OPT_AGENT_FENCES] ? 1 : 0;
+    args.spin_limit = opt[MCTSNC_OPT_SPIN_LIMIT] > 0 ? (uint32_t)opt[MCTSNC_OPT_SPIN_LIMIT] : c4::kSpinLimit;
     dim3 block(e0->block);
     // All-children playouts, three forms of the same step (identical results).  A team of one workgroup per column with one
     // lane per playout has the shortest step and is what one search or a few dozen run on.  One workgroup per tree (see
     // search_body) does no work twice, lets no lane idle while others finish their playouts and keeps every CU busy from
-    // the queue: the form for many hundreds of trees.  Between the two, teams whose workgroups play their child's playouts
-    // as a pool of jobs on half as many lanes: half the wavefronts per tree, so twice as many trees resident, and no
-    // idle lanes, at a step 1.4 times as long.  Measured (searches of 4 trees x 256 playouts, 5000 steps, different
-    // roots, G playouts/s in one pass, teams / teams with pools / one workgroup per tree): 64 searches 12.5 / 9.2 / 6.7,
-    // 96 searches 14.4 / 13.8 / 9.3, 112 searches 14.4 / 14.7 / 9.7, 128 searches 14.6 / 17.0 / 10.7, 192 searches
-    // 15.1 / 19.8 / 14.3, 256 searches 15.2 / 21.1 / 15.5, 304 searches 15.3 / 21.0 / 21.0, 320 searches 15.3 / 21.4 / 22.9,
-    // 384 searches 15.5 / 21.4 / 26.1, 512 searches 15.5 / 21.9 / 37.9, 768 searches 15 / - / 40.5; with 512 instead of 256
-    // threads (see below) one workgroup per tree reaches 16.8 at 192 searches, 20.9 at 224, 25.9 at 256, 21.5 at 288, 22.7
-    // at 304, 28.5 at 384: pools from 1.75 trees per CU on, one workgroup per tree from 3.5.  One search, whose trees all take about as long, ms per search: a
-    // single workgroup's step costs the same for any number of trees up to one per CU (155) and again up to two per CU
-    // (250), a team's search grows with the number of trees (192 trees 153, 256 trees 191, 320 trees 230, 384 trees 255,
-    // 448 trees 309, 512 trees 339): one workgroup per tree from 1.4 trees per CU on, and between 0.8 and 1.
-    // MCTSNC_SOLO_TREES sets one threshold for both (0 = never).
+    // the queue: the form for many hundreds of trees (from 3.5 trees per CU on in a batch; in one search from 1.4 trees
+    // per CU on, and between 0.8 and 1).  Between the two, teams whose workgroups play their child's playouts as a pool of
+    // jobs on half as many lanes: half the wavefronts per tree, so twice as many trees resident, and no idle lanes, at a
+    // step 1.4 times as long (from 1.75 trees per CU on).  MCTSNC_OPT_SOLO_TREES and MCTSNC_OPT_TEAM_POOL override the choice.
     int cus_now = 0;
     HIP_TRY(hipDeviceGetAttribute(&cus_now, hipDeviceAttributeMultiprocessorCount, c.device));
     bool solo = e0->acp && (n > 1 ? 2 * n_refs >= 7 * cus_now : (10 * n_refs >= 14 * cus_now || (10 * n_refs >= 8 * cus_now && n_refs <= cus_now)));
-    if (const char *v = getenv("MCTSNC_SOLO_TREES")) { const int from = atoi(v); solo = e0->acp && from > 0 && n_refs >= from; }
+    if (opt[MCTSNC_OPT_SOLO_TREES] >= 0) solo = e0->acp && opt[MCTSNC_OPT_SOLO_TREES] > 0 && n_refs >= opt[MCTSNC_OPT_SOLO_TREES];
     if (solo) {
         args.G = 1;
         // The workgroup plays all playouts of a step as one pool of jobs (lanes take further jobs as theirs end) with as many
         // lanes as one node has playouts, twice as many while there are no more than six trees per CU (64 to 512).  Fewer
         // lanes make better use of each but lengthen the step of the slowest tree, which a pass waits for; four workgroups
-        // of 256 threads per CU stay resident (LDS), two of 512 (registers).  Measured, G playouts/s, 256 / 512 threads:
-        // 320 searches of 4 trees 23.0 / 24.8, 384 searches 26.2 / 28.3, 448 searches 31.1 / 28.9, 512 searches 37.8 / 31.8,
-        // 768 searches 40.6 / 32.2 (192 threads 33.7, 384 threads 30.3); one search with 512 trees (two per CU) 15.8 / 17.6.
+        // of 256 threads per CU stay resident (LDS), two of 512 (registers).
         int threads = ((c.n_playouts + 63) / 64) * 64;
         if (n_refs <= 6 * cus_now) threads *= 2;
         threads = threads < 64 ? 64 : (threads > 512 ? 512 : threads);
-        if (const char *v = getenv("MCTSNC_SOLO_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 1024 && t % 64 == 0) threads = t; }   // for experiments
+        if (opt[MCTSNC_OPT_SOLO_THREADS] > 0) threads = opt[MCTSNC_OPT_SOLO_THREADS];
         block = dim3(threads);
     }
-    // Teams with pools (see above): half as many lanes as playouts (with a quarter the step gets too long: 192 searches
-    // 17.5 against 19.7, 288 searches 15.5 against 21.1; with three quarters the gain is gone).  MCTSNC_TEAM_POOL=0/1
-    // forces the form off/on, MCTSNC_TEAM_POOL_THREADS sets the lanes.
-    // One search of more trees than CUs, below the point where one workgroup per tree takes over: 320 trees 217 ms against
-    // 231 for plain teams (256 trees 186 against 192, 192 trees 152 against 152, 128 trees 122 against 114).
+    // Teams with pools (see above): half as many lanes as playouts.
     bool team_pool = e0->acp && !solo && c.n_playouts >= 128 && (n > 1 ? 4 * n_refs >= 7 * cus_now : n_refs > cus_now);
-    if (const char *v = getenv("MCTSNC_TEAM_POOL")) team_pool = e0->acp && !solo && atoi(v) != 0;
+    if (opt[MCTSNC_OPT_TEAM_POOL] >= 0) team_pool = e0->acp && !solo && opt[MCTSNC_OPT_TEAM_POOL] != 0;
     if (team_pool) {
         int threads = ((c.n_playouts / 2 + 63) / 64) * 64;
         if (threads < 64) threads = 64;
-        if (const char *v = getenv("MCTSNC_TEAM_POOL_THREADS")) { const int t = atoi(v); if (t >= 64 && t <= 512 && t % 64 == 0) threads = t; }
+        if (opt[MCTSNC_OPT_TEAM_POOL_THREADS] > 0) threads = opt[MCTSNC_OPT_TEAM_POOL_THREADS];
         block = dim3(threads);
     }
     const size_t lds = solo ? c4::solo_lds_bytes(c.board_m, c.board_n, c.n_playouts)
                             : (team_pool ? c4::team_pool_lds_bytes(c.board_m, c.board_n, c.n_playouts) : c4::search_lds_bytes(c.board_m, c.board_n));
-    const auto solo_kernel = block.x > 512 ? c4::search_kernel_solo_wide : c4::search_kernel_solo;
+    const auto solo_kernel = c4::search_kernel_solo;
     const auto team_kernel = team_pool ? c4::search_kernel_team_pool : c4::search_kernel<true>;
     if (solo) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(solo_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // Sets of G workgroups (8 sets per grid row, one per XCD).  The all-children kernel is launched cooperatively, so
@@ -554,23 +548,20 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         const int resident_sets = (int)((int64_t)per_cu * cus / (8 * args.G)) * 8;
         if (resident_sets < 8) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of one row of trees at once", 8 * args.G);
         if (sets > resident_sets) { sets = resident_sets; args.queue = e0->d_abort + 1; }
-        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets of %d (%d workgroups per CU resident)%s\n", n_refs, sets, args.G, per_cu, args.queue ? ", queue" : "");
+        if (debug_enabled()) fprintf(stderr, "[mctsnc] %d trees on %d workgroup sets of %d (%d workgroups per CU resident)%s\n", n_refs, sets, args.G, per_cu, args.queue ? ", queue" : "");
     }
     const dim3 grid(args.G * sets);
     // A pass that hands trees out through the queue lasts as long as its last search, and what a search costs is not
     // seen from its root (of two roots with as many stones one may be decided and ten times cheaper): so such a pass
     // first runs every tree for a few steps (a thirty-second of the step budget, 16 to 128), then puts the searches that
-    // played the most plies in front.  Splitting a search over launches does not change its result.  Measured, G
-    // playouts/s without / with: 768 searches of 4 trees 32 / 40.5, the 64 roots of the benchmark (256 trees on 176
-    // resident teams) 11.1 / 12.6; probes of 64 / 128 / 256 / 512 / 1024 steps: 38.9 / 40.5 / 41.7 / 38.8 / 38.0 and
-    // 11.6 / 12.6 / 12.0 / 12.4 / 12.0.
+    // played the most plies in front.  Splitting a search over launches does not change its result.
     int32_t probe_steps = 0;
     if (n > 1 && args.queue != nullptr) {
         const double budget = bud.forced < INFINITY ? bud.forced : bud.steps_limit;
         probe_steps = budget < 32.0 * 128.0 ? (budget < 32.0 * 16.0 ? 16 : (int32_t)(budget / 32.0)) : 128;
-        if (const char *v = getenv("MCTSNC_PROBE_STEPS")) probe_steps = atoi(v);   // for experiments (0 = keep the order by stones)
+        if (opt[MCTSNC_OPT_PROBE_STEPS] >= 0) probe_steps = opt[MCTSNC_OPT_PROBE_STEPS];
     }
-    const bool plain_launch = plain_launch_requested();
+    const bool plain_launch = opt[MCTSNC_OPT_PLAIN_LAUNCH] != 0;
     static std::atomic<uint32_t> launch_counter{0};
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
@@ -622,6 +613,7 @@ int run_many_c4(mctsnc_engine **engines, int n, const int8_t *boards, const int8
         HIP_TRY(hipMemcpy(d_refs, sorted.data(), sizeof(c4::TreeRef) * n_refs, hipMemcpyHostToDevice));
         return MCTSNC_OK;
     });
+    if (rc == MCTSNC_E_DEVICE_SYNC) return search_abandoned(engines, n, steps);
     if (rc) return rc;
 
     // the trees of a search stay together and in order under the sorts above: search j of the launch order
@@ -686,11 +678,15 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     if (e0->slots < 64 || (e0->slots & (e0->slots - 1))) return fail(MCTSNC_E_STATE, "playouts per round (%d) must be a power of two >= 64", e0->slots);
     args.S = (int32_t)c.max_tree_size; args.thrifty = e0->thrifty ? 1 : 0; args.ucb_c = c.ucb_c; args.abort_flag = e0->d_abort;
     args.stage_timing = e0->stage_timing ? 1 : 0;
-    args.agent_fences = getenv("MCTSNC_AGENT_FENCES") ? 1 : 0;   // for testing the path taken when a tree's workgroups span XCCs
-    args.prep_levels = gomoku::kPrepLevels;
-    if (const char *v = getenv("MCTSNC_PREP_LEVELS")) args.prep_levels = std::max(0, std::min(atoi(v), gomoku::kPrepLevels));   // for testing the path deep trees take
+    const int *opt = e0->options;
+    args.agent_fences = opt[MCTSNC_OPT_AGENT_FENCES] ? 1 : 0;
+    args.spin_limit = opt[MCTSNC_OPT_SPIN_LIMIT] > 0 ? (uint32_t)opt[MCTSNC_OPT_SPIN_LIMIT] : gomoku::kSpinLimit;
+    args.prep_levels = opt[MCTSNC_OPT_PREP_LEVELS] >= 0 ? std::min(opt[MCTSNC_OPT_PREP_LEVELS], gomoku::kPrepLevels) : gomoku::kPrepLevels;
     const dim3 block(e0->block);
     const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots);
+    // the limit is a setting of the kernel function, not of this engine: an engine of another shape may have changed it
+    if (e0->acp) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    else HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
     // whole: more trees than the device holds G workgroups each for are searched by consecutive launches over equal
     // groups of trees, every group for the same number of steps before the budget is looked at again.
@@ -703,9 +699,9 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         if (fit < 1) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of a tree at once", e0->G);
         const int64_t n_groups = (n_refs + fit - 1) / fit;
         group = (int)((n_refs + n_groups - 1) / n_groups);
-        if (getenv("MCTSNC_DEBUG")) fprintf(stderr, "[mctsnc] %d trees, %d workgroups per tree, %d resident workgroups per CU: launches of %d trees\n", n_refs, e0->G, per_cu, group);
+        if (debug_enabled()) fprintf(stderr, "[mctsnc] %d trees, %d workgroups per tree, %d resident workgroups per CU: launches of %d trees\n", n_refs, e0->G, per_cu, group);
     }
-    const bool plain_launch = plain_launch_requested();
+    const bool plain_launch = opt[MCTSNC_OPT_PLAIN_LAUNCH] != 0;
     int64_t steps; double dev_time, time_loop;
     int rc = budget_loop(e0, bud, [&](int32_t nsteps) -> int {
         args.nsteps = nsteps;
@@ -728,6 +724,7 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
         }
         return MCTSNC_OK;
     }, steps, dev_time, time_loop);
+    if (rc == MCTSNC_E_DEVICE_SYNC) return search_abandoned(engines, n, steps);
     if (rc) return rc;
 
     std::vector<int> search_of((size_t)n);
@@ -752,12 +749,14 @@ int run_many(mctsnc_engine **engines, int n, const int8_t *boards, const int8_t 
     // buffers, so it is turned away instead
     if (ds.busy.exchange(true, std::memory_order_acquire))
         return fail(MCTSNC_E_STATE, "the static scratch of device %d is in use by another mctsnc_run_batch_noalloc call", c.device);
+    struct Release {   // whatever way the call ends
+        std::atomic<bool> &flag;
+        ~Release() { flag.store(false, std::memory_order_release); }
+    } release{ds.busy};
     Workspace ws;
     ws.base = ds.ptr.load(std::memory_order_acquire); ws.size = MCTSNC_NOALLOC_SCRATCH_BYTES;
-    rc = e0->is_gomoku() ? run_many_gomoku(engines, n, boards, turns, bud, out, &ws)
-                         : run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out, &ws);
-    ds.busy.store(false, std::memory_order_release);
-    return rc;
+    return e0->is_gomoku() ? run_many_gomoku(engines, n, boards, turns, bud, out, &ws)
+                           : run_many_c4(engines, n, boards, extras, extra_len, turns, bud, out, &ws);
 }
 
 int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, size_t need) {
@@ -991,6 +990,23 @@ int mctsnc_run_batch_noalloc(mctsnc_engine **engines, int32_t n, const int8_t *b
     if (!engines || !boards || !turns || !out) return fail(MCTSNC_E_INVALID, "null argument");
     Budget b{steps_limit, time_limit_s, forced_steps_limit};
     return run_many(engines, n, boards, extras, extra_len, turns, b, out, true);
+}
+
+int mctsnc_set_option(mctsnc_engine *e, int32_t option, int32_t value) {
+    if (!e) return fail(MCTSNC_E_INVALID, "null engine");
+    bool ok = false;
+    switch (option) {
+    case MCTSNC_OPT_AGENT_FENCES: case MCTSNC_OPT_PLAIN_LAUNCH: ok = value == 0 || value == 1; break;
+    case MCTSNC_OPT_SOLO_TREES: case MCTSNC_OPT_PROBE_STEPS: ok = value >= -1; break;
+    case MCTSNC_OPT_TEAM_POOL: ok = value >= -1 && value <= 1; break;
+    case MCTSNC_OPT_PREP_LEVELS: ok = value >= -1; break;
+    case MCTSNC_OPT_SOLO_THREADS: case MCTSNC_OPT_TEAM_POOL_THREADS: ok = value == 0 || (value >= 64 && value <= 512 && value % 64 == 0); break;
+    case MCTSNC_OPT_SPIN_LIMIT: ok = value >= 0; break;
+    default: return fail(MCTSNC_E_INVALID, "unknown option %d", option);
+    }
+    if (!ok) return fail(MCTSNC_E_INVALID, "option %d does not take the value %d", option, value);
+    e->options[option] = value;
+    return MCTSNC_OK;
 }
 
 int mctsnc_set_stage_timing(mctsnc_engine *e, int32_t on) {

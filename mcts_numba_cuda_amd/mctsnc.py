@@ -210,6 +210,15 @@ class MCTSNC:
         self._require_engine()
         _lib.check(_lib.lib().mctsnc_reseed(self._engine))
 
+    def set_option(self, name, value):
+        """How the search is laid out on the device, and test hooks (``mctsnc_set_option`` of include/mctsnc_hip.h:
+        "agent_fences", "solo_trees", "solo_threads", "team_pool", "team_pool_threads", "prep_levels", "plain_launch",
+        "probe_steps", "spin_limit"); results do not depend on any of them.  ``run_batch`` takes those of its first engine."""
+        self._require_engine()
+        if name not in _lib.OPTIONS:
+            raise ValueError(f"unknown option {name!r}; known: {sorted(_lib.OPTIONS)}")
+        _lib.check(_lib.lib().mctsnc_set_option(self._engine, _lib.OPTIONS[name], int(value)))
+
     def _require_engine(self):
         if not self._engine:
             raise RuntimeError("init_device_side_arrays() must be called before run()")

@@ -4,13 +4,16 @@ import numpy as np
 M, N = 6, 7
 
 
-def make_engine(params, board_shape=(M, N), extra=N, actions=N, **kw):
-    """An initialised MCTSNC engine (HIP) for Connect 4 from a parameter dict as stored in the archive fixture."""
+def make_engine(params, board_shape=(M, N), extra=N, actions=N, options=None, **kw):
+    """An initialised MCTSNC engine (HIP) for Connect 4 from a parameter dict as stored in the archive fixture;
+    `options`: {name: value} for MCTSNC.set_option()."""
     from mcts_numba_cuda_amd import MCTSNC
     e = MCTSNC(board_shape, extra, actions, search_time_limit=np.inf, search_steps_limit=np.inf,
                n_trees=params["n_trees"], n_playouts=params["n_playouts"], variant=params["variant"],
                device_memory=params["device_memory"], ucb_c=params["ucb_c"], seed=params["seed"], verbose_info=False, **kw)
     e.init_device_side_arrays()
+    for name, value in (options or {}).items():
+        e.set_option(name, value)
     return e
 
 

@@ -57,15 +57,15 @@ def test_gomoku_children_that_complete_lines(variant, steps):
     compare_with_oracle(e, o, board, None, 1, steps)
 
 
-@pytest.mark.parametrize("levels", ["0", "2"])
-def test_gomoku_one_child_backup_of_paths_too_deep_to_prepare(monkeypatch, levels):
+@pytest.mark.parametrize("levels", [0, 2])
+def test_gomoku_one_child_backup_of_paths_too_deep_to_prepare(levels):
     """One-child variants prepare the backup's arg-max during the playouts for paths of up to 48 levels; deeper ones are
-    backed up after the playouts from memory.  MCTSNC_PREP_LEVELS lowers the limit so that ordinary searches take that
+    backed up after the playouts from memory.  Option prep_levels lowers the limit so that ordinary searches take that
     path at every step (0) or at the steps that select below the second level (2)."""
-    monkeypatch.setenv("MCTSNC_PREP_LEVELS", levels)
     rng = np.random.default_rng(21)
     for variant, (m, n), steps in (("ocp_thrifty", (15, 15), 80), ("ocp_prodigal", (6, 6), 250)):
         e, o = engines(variant, 2, 64, m, n)
+        e.set_option("prep_levels", levels)
         board, turn = random_gomoku_root(rng, m, n, 5)
         compare_with_oracle(e, o, board, None, turn, steps)
 

@@ -176,12 +176,11 @@ def test_other_connect4_boards(m, n, variant):
 
 
 @pytest.mark.parametrize("m,n", [(4, 5), (7, 8), (8, 7), (13, 4)])
-def test_other_connect4_boards_one_workgroup_per_tree(m, n, monkeypatch):
+def test_other_connect4_boards_one_workgroup_per_tree(m, n):
     """The same boards' extremes with every tree searched by a single workgroup (the pool of playout jobs)."""
-    monkeypatch.setenv("MCTSNC_SOLO_TREES", "1")
     rng = np.random.default_rng(100 * m + n + 1)
     params = dict(n_trees=3, n_playouts=64, variant="acp_prodigal", device_memory=0.25, ucb_c=2.0, seed=9)
-    e = make_engine(params, board_shape=(m, n), extra=n, actions=n)
+    e = make_engine(params, board_shape=(m, n), extra=n, actions=n, options=dict(solo_trees=1))
     from oracle.oracle import Oracle
     o = Oracle("c4", (m, n), n, n, 3, 64, "acp_prodigal", ucb_c=2.0, seed=9, device_memory=0.25, threads=8)
     for plies in (2, m * n // 2):
@@ -230,22 +229,20 @@ def test_search_ends_before_visit_counters_overflow():
     assert e.time_total < 30.0
 
 
-@pytest.mark.parametrize("threads", ["", "64", "192", "896"], ids=["default-workgroup", "one-wavefront", "three-wavefronts", "fourteen-wavefronts"])
+@pytest.mark.parametrize("threads", [0, 64, 192, 512], ids=["default-workgroup", "one-wavefront", "three-wavefronts", "eight-wavefronts"])
 @pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
-def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypatch):
+def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads):
     """With many trees in one pass the all-children search of a tree is done by a single workgroup instead of one per
-    column (MCTSNC_SOLO_TREES sets from how many trees on), which runs all playouts of a step as one pool of jobs that
-    its lanes take one after the other (MCTSNC_SOLO_THREADS overrides its size).  Forced here for small searches: full
+    column (option solo_trees sets from how many trees on), which runs all playouts of a step as one pool of jobs that
+    its lanes take one after the other (solo_threads overrides its size).  Forced here for small searches: full
     state against the oracle over two runs, a pool that fills up, late-game roots, and a batch against single runs."""
     from mcts_numba_cuda_amd import MCTSNC, run_batch
     from oracle.oracle import Oracle
-    monkeypatch.setenv("MCTSNC_SOLO_TREES", "1")
-    if threads:
-        monkeypatch.setenv("MCTSNC_SOLO_THREADS", threads)
+    forced = dict(solo_trees=1, solo_threads=threads)
     rng = np.random.default_rng(41)
     for T, P, steps in ((3, 64, 300), (4, 256, 150), (2, 16, 200)):
         params = dict(n_trees=T, n_playouts=P, variant=variant, device_memory=0.25, ucb_c=2.0, seed=7)
-        e = make_engine(params)
+        e = make_engine(params, options=forced)
         o = Oracle("c4", (6, 7), 7, 7, T, P, variant, ucb_c=2.0, seed=7, device_memory=0.25, threads=8)
         for plies in (8, 24):
             board, fills, turn = random_c4_root(rng, plies)
@@ -254,17 +251,18 @@ def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypat
                device_memory=2.0, ucb_c=2.0, seed=4, verbose_info=False)
     e.device_memory = float(2 * 95 * 50 + 2 * 8300)  # room for about 50 nodes per tree
     e.init_device_side_arrays()
+    for name, value in forced.items():
+        e.set_option(name, value)
     o = Oracle("c4", (6, 7), 7, 7, 2, 64, variant, ucb_c=2.0, seed=4, max_tree_size_override=e.max_tree_size, threads=4)
     for plies in (5, 30):
         board, fills, turn = random_c4_root(rng, plies)
         compare_with_oracle(e, o, board, fills, turn, steps=200)
     params = dict(n_trees=4, n_playouts=128, variant=variant, device_memory=0.1, ucb_c=2.0, seed=11)
     roots = [random_c4_root(rng, p) for p in (4, 9, 15, 22, 12)]
-    batch = [make_engine(params) for _ in roots]
+    batch = [make_engine(params, options=forced) for _ in roots]
     run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=400)
-    monkeypatch.setenv("MCTSNC_SOLO_TREES", "0")
     for eb, r in zip(batch, roots):
-        es = make_engine(params)
+        es = make_engine(params, options=dict(solo_trees=0))
         es.run(r[0], r[1], r[2], forced_search_steps_limit=400)
         assert eb.actions_info == es.actions_info
         for ti in range(4):
@@ -272,23 +270,20 @@ def test_one_workgroup_per_tree_gives_the_same_trees(variant, threads, monkeypat
             np.testing.assert_array_equal(eb.read_array("trees", ti), es.read_array("trees", ti))
 
 
-@pytest.mark.parametrize("threads", ["", "64", "192"], ids=["half-the-playouts", "one-wavefront", "three-wavefronts"])
+@pytest.mark.parametrize("threads", [0, 64, 192], ids=["half-the-playouts", "one-wavefront", "three-wavefronts"])
 @pytest.mark.parametrize("variant", ["acp_thrifty", "acp_prodigal"])
-def test_teams_with_playout_pools_give_the_same_trees(variant, threads, monkeypatch):
+def test_teams_with_playout_pools_give_the_same_trees(variant, threads):
     """A pass of a few hundred trees runs teams whose workgroups play their child's playouts as a pool of jobs on fewer
-    lanes than playouts (MCTSNC_TEAM_POOL forces the form on or off, MCTSNC_TEAM_POOL_THREADS sets the lanes).  Forced here
+    lanes than playouts (option team_pool forces the form on or off, team_pool_threads sets the lanes).  Forced here
     for small searches: full state against the oracle over two runs, a pool that fills up, late-game roots, a playout
     count smaller than a wavefront, and a batch through the queue against single runs without pools."""
     from mcts_numba_cuda_amd import MCTSNC, run_batch
     from oracle.oracle import Oracle
-    monkeypatch.setenv("MCTSNC_TEAM_POOL", "1")
-    monkeypatch.setenv("MCTSNC_SOLO_TREES", "0")
-    if threads:
-        monkeypatch.setenv("MCTSNC_TEAM_POOL_THREADS", threads)
+    forced = dict(team_pool=1, solo_trees=0, team_pool_threads=threads)
     rng = np.random.default_rng(43)
     for T, P, steps in ((3, 64, 300), (4, 256, 150), (2, 16, 200)):
         params = dict(n_trees=T, n_playouts=P, variant=variant, device_memory=0.25, ucb_c=2.0, seed=7)
-        e = make_engine(params)
+        e = make_engine(params, options=forced)
         o = Oracle("c4", (6, 7), 7, 7, T, P, variant, ucb_c=2.0, seed=7, device_memory=0.25, threads=8)
         for plies in (8, 24):
             board, fills, turn = random_c4_root(rng, plies)
@@ -297,16 +292,17 @@ def test_teams_with_playout_pools_give_the_same_trees(variant, threads, monkeypa
                device_memory=2.0, ucb_c=2.0, seed=4, verbose_info=False)
     e.device_memory = float(2 * 95 * 50 + 2 * 8300)  # room for about 50 nodes per tree
     e.init_device_side_arrays()
+    for name, value in forced.items():
+        e.set_option(name, value)
     o = Oracle("c4", (6, 7), 7, 7, 2, 64, variant, ucb_c=2.0, seed=4, max_tree_size_override=e.max_tree_size, threads=4)
     for plies in (5, 30):
         board, fills, turn = random_c4_root(rng, plies)
         compare_with_oracle(e, o, board, fills, turn, steps=200)
     params = dict(n_trees=4, n_playouts=128, variant=variant, device_memory=0.1, ucb_c=2.0, seed=11)
     roots = [random_c4_root(rng, int(rng.integers(4, 24))) for _ in range(96)]
-    batch = [make_engine(params) for _ in roots]
+    batch = [make_engine(params, options=forced) for _ in roots]
     run_batch(batch, [r[0] for r in roots], [r[1] for r in roots], [r[2] for r in roots], forced_search_steps_limit=300)
-    monkeypatch.setenv("MCTSNC_TEAM_POOL", "0")
-    es = make_engine(params)
+    es = make_engine(params, options=dict(team_pool=0, solo_trees=0))
     for k in range(0, len(roots), 7):
         eb, r = batch[k], roots[k]
         es.reseed()
@@ -447,16 +443,15 @@ def test_gomoku_run_batch_in_groups():
 
 
 @pytest.mark.parametrize("game,variant", [("c4", "acp_prodigal"), ("c4", "acp_thrifty"), ("gomoku", "acp_prodigal")])
-def test_device_scope_fences_give_the_same_trees(game, variant, monkeypatch):
+def test_device_scope_fences_give_the_same_trees(game, variant):
     """The all-child kernels skip L2 write-backs and invalidations once a tree's workgroups are known to share an
-    XCC.  MCTSNC_AGENT_FENCES keeps them on the general path (full device-scope release and acquire every step), which
+    XCC.  Option agent_fences keeps them on the general path (full device-scope release and acquire every step), which
     a device that spreads a tree over XCCs would take; results must not depend on it."""
-    monkeypatch.setenv("MCTSNC_AGENT_FENCES", "1")
     rng = np.random.default_rng(31)
     if game == "c4":
         from oracle.oracle import Oracle
         params = dict(n_trees=3, n_playouts=64, variant=variant, device_memory=0.25, ucb_c=2.0, seed=5)
-        e = make_engine(params)
+        e = make_engine(params, options=dict(agent_fences=1))
         o = Oracle("c4", (6, 7), 7, 7, 3, 64, variant, ucb_c=2.0, seed=5, device_memory=0.25, threads=8)
         board, fills, turn = random_c4_root(rng, 9)
         compare_with_oracle(e, o, board, fills, turn, 300)
@@ -464,20 +459,19 @@ def test_device_scope_fences_give_the_same_trees(game, variant, monkeypatch):
         from oracle.oracle import Oracle
         from helpers import random_gomoku_root
         params = dict(n_trees=2, n_playouts=64, variant=variant, device_memory=0.5, ucb_c=2.0, seed=5)
-        e = make_engine(params, board_shape=(9, 9), extra=0, actions=81, game="gomoku")
+        e = make_engine(params, board_shape=(9, 9), extra=0, actions=81, game="gomoku", options=dict(agent_fences=1))
         o = Oracle("gomoku", (9, 9), 0, 81, 2, 64, variant, ucb_c=2.0, seed=5, device_memory=0.5, threads=8)
         board, turn = random_gomoku_root(rng, 9, 9, 6)
         compare_with_oracle(e, o, board, None, turn, 12)
 
 
-def test_device_scope_fences_replay_a_recorded_game(archives, monkeypatch):
-    """The general path again (MCTSNC_AGENT_FENCES), over thousands of steps per search instead of hundreds: the first
+def test_device_scope_fences_replay_a_recorded_game(archives):
+    """The general path again (option agent_fences), over thousands of steps per search instead of hundreds: the first
     game of the reference's experiment with acp_prodigal 4 x 256 (17 searches of 5000 to 5900 steps with carried random
     streams) and of the one with acp_thrifty 8 x 256 (10 searches) must give the recorded root tables and tree statistics."""
-    monkeypatch.setenv("MCTSNC_AGENT_FENCES", "1")
     for a in ("mctsnc_5_inf_4_256_acp_prodigal", "mctsnc_1_inf_8_256_acp_thrifty"):
         key = replay.find_archive(archives, "mcts_5_inf_vanilla", a)
-        n = replay.replay_archive(archives[key], make_engine, engine_run_search, max_games=1)
+        n = replay.replay_archive(archives[key], lambda params: make_engine(params, options=dict(agent_fences=1)), engine_run_search, max_games=1)
         assert n >= 3, key
 
 

@@ -53,16 +53,17 @@ def assert_same_trees(got, want):
     ((16, 16), 1, 13, 200, 8192, 256, 3.0)])
 def test_search_equals_oracle(shape, stones, traversals, steps, max_nodes, depth, c_pw):
     """Any number of traversals per tree: every array of every created node, the last step's selections and paths and
-    the tallies equal the host oracle's, in one launch and in three launches per step; includes trees that fill up,
-    paths cut by the depth limit, boards that fill up (draws) and the widest board."""
+    the tallies equal the host oracle's, in one launch (with the new nodes' priors worked out by evaluator workgroups or
+    by the tree's own) and in three launches per step; includes trees that fill up, paths cut by the depth limit,
+    boards that fill up (draws) and the widest board."""
     from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
     rng = np.random.default_rng(shape[0] * 31 + stones)
     board, turn = random_gomoku_root(rng, shape[0], shape[1], stones)
     kw = dict(trees=5, traversals=traversals, max_nodes=max_nodes, path_depth=depth, cpuct=1.5, c_pw=c_pw, dirichlet_alpha=0.3, seed=9)
     want = po.gomoku_search(board, turn, steps, **kw)
     gc.check_trees(want, board, turn, shape[0], shape[1], max_nodes, depth)
-    for fused in (True, False):
-        e = PUCTGomoku(board_shape=shape, **kw)
+    for fused, evaluators in ((True, 4), (True, 0), (True, 8), (False, 0)):
+        e = PUCTGomoku(board_shape=shape, evaluators=evaluators, **kw)
         best = e.run(board, turn, steps, fused=fused)
         got = read_all(e)
         assert_same_trees(got, want)
@@ -100,6 +101,23 @@ def test_traversals_of_a_step_build_consistent_trees(shape, stones, trees, trave
     e.run(board, turn, steps)
     assert_same_trees(read_all(e), h)
     e.close()
+
+
+def test_repeated_searches_give_the_same_trees():
+    """Twenty searches of one configuration (many traversals meeting on few nodes, trees of some thousand nodes) must all
+    equal the host oracle's: a result that depends on when a store becomes visible to another wavefront shows up as a
+    search that differs.  (An earlier form of the loop, which let the traversals race for their claims, handed out an
+    expansion slot twice once in some thousand searches because a barrier did not wait for the stores before it.)"""
+    from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
+    board, turn = random_gomoku_root(np.random.default_rng(35), 15, 15, 20)
+    kw = dict(trees=16, traversals=16, max_nodes=4096, path_depth=64, cpuct=1.5, c_pw=3.0, dirichlet_alpha=0.3, seed=1)
+    want = po.gomoku_search(board, turn, 250, **kw)
+    for evaluators in (4, 0):
+        e = PUCTGomoku(board_shape=(15, 15), evaluators=evaluators, **kw)
+        for _ in range(10):
+            e.run(board, turn, 250)
+            assert_same_trees(read_all(e), want)
+        e.close()
 
 
 def test_expanded_edges_stay_contiguous_when_tickets_leave_holes():
@@ -224,7 +242,7 @@ def test_finds_the_winning_move():
 def test_configuration_and_root_errors():
     from mcts_numba_cuda_amd.puct_gomoku import EngineError, PUCTGomoku
     for bad in (dict(board_shape=(17, 17)), dict(traversals=17), dict(max_nodes=(1 << 20) + 1), dict(dirichlet_alpha=1.5),
-                dict(path_depth=0), dict(path_depth=257), dict(trees=0)):
+                dict(path_depth=0), dict(path_depth=257), dict(trees=0), dict(evaluators=9), dict(evaluators=-1)):
         with pytest.raises(EngineError):
             PUCTGomoku(**bad)
     e = PUCTGomoku(board_shape=(5, 5), trees=1, traversals=1, max_nodes=16)
