@@ -266,21 +266,27 @@ def cpu_oracle_baseline(roots):
                       "CPU oracle (scalar restatement of the reference's kernels) with OpenMP over playouts"}
 
 
-def bench_gomoku(args):
-    """Gomoku 15x15, 32 seeded roots with 0..20 stones placed alternately on random cells,
-    ocp_thrifty, n_trees=4, n_playouts=128, 2000 steps, device_memory=16 GiB; one bench step = one search."""
-    import contextlib
-    import io
-    from mcts_numba_cuda_amd import MCTSNC
-    rng = np.random.Generator(np.random.PCG64(0))
+def make_gomoku_roots(n_roots=32, seed=0):
+    """Seeded synthetic Gomoku roots: 0..20 stones placed alternately on random cells of the 15x15 board."""
+    rng = np.random.Generator(np.random.PCG64(seed))
     roots = []
-    for _ in range(32):
+    for _ in range(n_roots):
         board = np.zeros((15, 15), np.int8)
         turn = 1
         for c in rng.permutation(225)[:int(rng.integers(0, 21))]:
             board[c // 15, c % 15] = turn
             turn = -turn
         roots.append((board, turn))
+    return roots
+
+
+def bench_gomoku(args):
+    """Gomoku 15x15, 32 seeded roots with 0..20 stones placed alternately on random cells,
+    ocp_thrifty, n_trees=4, n_playouts=128, 2000 steps, device_memory=16 GiB; one bench step = one search."""
+    import contextlib
+    import io
+    from mcts_numba_cuda_amd import MCTSNC
+    roots = make_gomoku_roots()
     steps = min(args.steps, len(roots)) if args.steps != N_ROOTS else 8
     quiet = io.StringIO()
     prof = profile_json("search_kernel_gomoku_ocp_thrifty_4x128_counters.md")

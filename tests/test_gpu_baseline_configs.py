@@ -1,9 +1,10 @@
 """The benchmark configurations at their full sizes, engine against oracle: every node of every tree, the step scratch,
 the reduced root tables and the random streams must agree after the whole search (Connect 4 1x32 ocp_thrifty, 1000
 steps; Connect 4 8x256 acp_thrifty, 20000 steps, 16 GiB pools; Gomoku 15x15 4x128 ocp_thrifty, 2000 steps, 16 GiB
-pools; Connect 4 4x256 acp_prodigal, 5000 steps, on the benchmark's own 64 seeded roots: four of them against the
-oracle, all of them in one batched pass against their sequential searches -- the same configuration is also covered
-by the recorded A100 games).  The fifth configuration (PUCT on Gomoku) is in test_gpu_puct_gomoku.py."""
+pools, on a root of its own and on the benchmark's 32 seeded roots: three of them against the oracle, all of them in one
+batched pass against their sequential searches; Connect 4 4x256 acp_prodigal, 5000 steps, on the benchmark's own 64
+seeded roots: four of them against the oracle, all of them in one batched pass against their sequential searches -- the
+same configuration is also covered by the recorded A100 games).  The fifth configuration (PUCT on Gomoku) is in test_gpu_puct_gomoku.py."""
 import numpy as np
 import pytest
 
@@ -40,6 +41,63 @@ def test_gomoku_ocp_thrifty_4x128_2000_steps():
     o = Oracle("gomoku", (15, 15), 0, 225, 4, 128, "ocp_thrifty", ucb_c=2.0, seed=0, device_memory=16.0, threads=16)
     compare_with_oracle(e, o, board, None, turn, steps=2000)
     assert e.performance_info["playouts"] == 2000 * 4 * 128
+
+
+GOMOKU_PARAMS = dict(n_trees=4, n_playouts=128, variant="ocp_thrifty", device_memory=16.0, ucb_c=2.0, seed=0)
+
+
+def gomoku_bench_roots():
+    import bench
+    return bench.make_gomoku_roots()
+
+
+def test_gomoku_benchmark_roots_are_what_the_configuration_says():
+    roots = gomoku_bench_roots()
+    stones = [int(np.count_nonzero(b)) for b, _ in roots]
+    assert len(roots) == 32 and 0 <= min(stones) <= 2 and 18 <= max(stones) <= 20
+    for board, turn in roots:
+        plus, minus = int((board == 1).sum()), int((board == -1).sum())
+        assert plus - minus in (0, 1) and turn == (1 if plus == minus else -1)
+
+
+@pytest.mark.parametrize("stones", [0, 10, 20])
+def test_gomoku_ocp_thrifty_4x128_2000_steps_on_a_benchmark_root(stones):
+    """Three of the 32 roots bench.py times (the one with the fewest stones, one in the middle, the one with the most),
+    the full 2000 steps."""
+    roots = gomoku_bench_roots()
+    k = min(range(len(roots)), key=lambda i: (abs(int(np.count_nonzero(roots[i][0])) - stones), i))
+    board, turn = roots[k]
+    e = make_engine(GOMOKU_PARAMS, board_shape=(15, 15), extra=0, actions=225, game="gomoku")
+    o = Oracle("gomoku", (15, 15), 0, 225, 4, 128, "ocp_thrifty", ucb_c=2.0, seed=0, device_memory=16.0, threads=16)
+    compare_with_oracle(e, o, board, None, turn, steps=2000)
+    assert e.performance_info["playouts"] == 2000 * 4 * 128
+
+
+def test_gomoku_ocp_thrifty_4x128_all_benchmark_roots_batched_equal_sequential():
+    """What bench.py times twice: the roots one MCTSNC.run() after the other (streams restarted per root), and all 32 in one
+    run_batch pass on 32 engines: root tables, best actions, tree statistics and the visit counts of every tree."""
+    from helpers import engine_result
+    from mcts_numba_cuda_amd import run_batch
+    roots = gomoku_bench_roots()
+    mk = lambda: make_engine(GOMOKU_PARAMS, board_shape=(15, 15), extra=0, actions=225, game="gomoku")
+    one = mk()
+    one.search_steps_limit = 2000.0
+    sequential = []
+    for board, turn in roots:
+        one.reseed()
+        one.run(board, None, turn)
+        sequential.append((engine_result(one), [one.read_array("ns", t).copy() for t in range(4)]))
+    one._release()
+    engines = [mk() for _ in roots]
+    for e in engines:
+        e.search_steps_limit = 2000.0
+    run_batch(engines, [r[0] for r in roots], None, [r[1] for r in roots])
+    for k, e in enumerate(engines):
+        assert e.steps == 2000 and e.performance_info["playouts"] == 2000 * 4 * 128
+        assert engine_result(e) == sequential[k][0], f"root {k}"
+        for t in range(4):
+            np.testing.assert_array_equal(e.read_array("ns", t), sequential[k][1][t], err_msg=f"root {k}, tree {t}")
+        e._release()
 
 
 def bench_roots():

@@ -1,6 +1,7 @@
-"""GPU parity of the Gomoku engine against the CPU oracle (the reference's Gomoku archives are missing from its
-checkout, so the oracle -- pinned on Connect 4 and, for the Gomoku rules, by brute-force checks -- is the only
-reference here: "oracle-pinned")."""
+"""GPU parity of the Gomoku engine against the CPU oracle, array for array.  The oracle is pinned end to end on Gomoku by
+the reference's one recorded Gomoku search (its README printout, tests/test_readme_examples.py, which the engine also
+reproduces directly), on Connect 4 by the reference's tree dumps and recorded games, and for the Gomoku rules by brute
+force (the reference's Gomoku archives are missing from its checkout)."""
 import numpy as np
 import pytest
 
