@@ -229,20 +229,36 @@ def bench_puct_select(args):
         cpu = {"value": sample * warps / dt, "unit": "selections/s", "cores": 1, "kind": "port",
                "sample": f"first {sample} trees of the same workload, one launch ({sample * warps} selections of {depth} levels), "
                          "sequential CPU oracle"}
-    out = {"metric": "PUCT selections/s, deep-wide select benchmark of the reference (winner_recalc, 8 traversals per tree)",
-           "value": selections / (ms * 1e-3), "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+    prof = profile_json(f"select_kernel_puct_{args.puct_shape}.md")
+    launch_s = ms / steps * 1e-3
+    traffic = (prof or {}).get("traffic_bytes_per_launch")
+    completed = selections * (1.0 - busy_share)     # busy share of the last launch; the launches are alike
+    out = {"metric": "PUCT selections/s that complete (reach the depth limit), deep-wide select benchmark of the reference "
+                     "(winner_recalc, 8 traversals per tree)",
+           "value": completed / (ms * 1e-3), "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
            "ms_per_step": ms / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32 scores + int32 atomics",
            "data": "synthetic",
            "config": {"workload": f"{args.puct_shape}: {trees} trees x {warps} traversals, {actions} edges per node, depth {depth}, "
                                   "equal priors, c_pw=0, terminal by depth limit; one puct_select_winner_recalc_launch per step"},
-           "valid": ok and ok_soft, "busy_share_last_launch": busy_share, "wall_s_incl_release": wall,
+           "valid": ok and ok_soft, "selections_per_s": {"all": selections / (ms * 1e-3), "completed": completed / (ms * 1e-3),
+                                                         "busy": selections * busy_share / (ms * 1e-3)},
+           "busy_share_last_launch": busy_share, "wall_s_incl_release": wall,
            "soft_winner": {"value": selections / (ms_soft * 1e-3), "unit": "selections/s", "ms_per_step": ms_soft / steps,
                            "busy_share_last_launch": busy_soft, "levels_per_s": selections * depth / (ms_soft * 1e-3),
-                           "algorithmic_GB_per_s": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9,
-                           "hbm_frac": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9 / HBM_PEAK_GBS},
-           "roofline": {"bound": "hbm", "achieved": alg_bytes / (ms / steps * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": alg_bytes / (ms / steps * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": (profile_json(f"select_kernel_puct_{args.puct_shape}.md") or {}).get("traffic_bytes_per_launch"),
-                        "kernel": "select_kernel", "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": ms / steps},
+                           "l2_level_GB_per_s": alg_bytes_soft / (ms_soft / steps * 1e-3) / 1e9,
+                           "note": "bytes requested by the traversals; the 8 traversals of a tree read the same rows, so most "
+                                   "of them are served by the L2, not by HBM"},
+           # The traversals of a tree read the same edge rows, so the bytes they request (the per-traversal algorithmic
+           # count) are an L2-level figure; what HBM delivers is what the counters measured, and that is the roofline entry.
+           "roofline": {"bound": "hbm", "achieved": traffic / launch_s / 1e9 if traffic else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": traffic / launch_s / 1e9 / HBM_PEAK_GBS if traffic else None, "traffic": traffic,
+                        "basis": "HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE summary over this run's launch time",
+                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
+                        "kernel": "select_kernel", "avg_launch_ms": ms / steps,
+                        "l2_level": {"requested_bytes_per_launch_completed_traversals": alg_bytes,
+                                     "requested_GB_per_s": alg_bytes / launch_s / 1e9,
+                                     "note": "node word, ticket counter and five 4-byte fields per edge and level, for the "
+                                             "traversals that complete; busy ones stop after a third of the levels on average"}},
            "cpu_baseline": cpu}
     print(json.dumps(out))
 
@@ -723,6 +739,9 @@ def main():
            "mcts_steps_per_s": mcts_steps / elapsed,
            "device_loop_share": dev_time / elapsed,
            "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
+           # algorithmic bytes of a stage over the device time of that stage (the stage clock of one workgroup of tree 0)
+           "stage_achieved_gbs": {k: alg[k] / stage[k] / 1e9 for k in ("select", "expand", "playout", "backup") if stage.get(k)},
+           "stage_hbm_frac": {k: alg[k] / stage[k] / 1e9 / HBM_PEAK_GBS for k in ("select", "expand", "playout", "backup") if stage.get(k)},
            "batched": batched, "trees_512": trees_512,
            "roofline": roofline, "roofline_valu": roofline_valu, "cpu_baseline": cpu_baseline, "cpu_mcts": cpu_mcts}
     print(json.dumps(out))

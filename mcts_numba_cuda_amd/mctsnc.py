@@ -176,6 +176,17 @@ class MCTSNC:
         max_tree_size = (int(self.device_memory) - self.n_trees * per_tree_additional_memory) // (per_state_memory * self.n_trees)
         return per_state_memory, min(max_tree_size, self.MAX_TREE_SIZE)
 
+    def _engine_shape_limit(self):
+        """What of the engine's shape limits (narrower than the reference's MAX_STATE_BOARD_SHAPE / MAX_STATE_MAX_ACTIONS)
+        the configured board exceeds, or None."""
+        m, n = int(self.state_board_shape[0]), int(self.state_board_shape[1])
+        if self.game == "gomoku":
+            if m > 16 or n > 16:
+                return "placement games are held on up to 16 x 16 cells (256 actions)"
+        elif (m + 1) * n > 64 or n > 8 or m > 13:
+            return "drop games are held in 64-bit column bitboards: (rows + 1) * columns <= 64, columns <= 8, rows <= 13"
+        return None
+
     def init_device_side_arrays(self):
         """Allocates the node pools in HBM and seeds the random streams (src/mctsnc.py:318-407).  ``device_memory``
         fixes the number of nodes per tree exactly as in the reference; a node record here is one 128-byte line, so
@@ -186,6 +197,13 @@ class MCTSNC:
         per_state_memory, self.max_tree_size = self._per_state_memory()
         if self.max_tree_size < 1:
             raise ValueError("device_memory too small for a single node per tree")
+        limit = self._engine_shape_limit()
+        if limit:
+            # in the style of the reference's own cap messages (src/mctsnc.py:240-249); its caps (32 x 32 cells, 512
+            # actions) are wider than what this engine's kernels take
+            message = f"[MCTSNC._init_device_side_arrays(): exiting due to state board shape {tuple(self.state_board_shape)} beyond this engine's {self.game} kernels: {limit}]"
+            print(message)
+            raise ValueError(message)
         L = _lib.lib()
         self._release()
         cfg = _lib.Config(game=self.GAMES[self.game], board_m=self.state_board_shape[0], board_n=self.state_board_shape[1],
