@@ -391,6 +391,91 @@ def bench_gomoku(args):
     print(json.dumps(out))
 
 
+def readme_gomoku_position():
+    """The position of the reference's README showcase ("Example usage 2": 15 stones on 15x15, white to move), kept as data
+    with the run's printed results in tests/golden/readme_examples.json."""
+    with open(os.path.join(ROOT, "tests", "golden", "readme_examples.json")) as f:
+        ex = json.load(f)["gomoku"]
+    board = np.array([[{"X": 1, "O": -1, ".": 0}[ch] for ch in row] for row in ex["board_rows"]], dtype=np.int8)
+    return ex, board
+
+
+def bench_gomoku_acp(args):
+    """The reference's README showcase: Gomoku 15x15, acp_prodigal, n_trees=8, n_playouts=128, device_memory=2 GiB, seed 0,
+    from its 15-stone position for the 442 steps its 5 s run took (the engine reproduces the printed root table:
+    tests/test_readme_examples.py).  All 210 children of every expanded node are played out: 210 x 128 playouts per
+    tree and step.  One bench step = one such search."""
+    import contextlib
+    import io
+    from mcts_numba_cuda_amd import MCTSNC
+    ex, board = readme_gomoku_position()
+    p = ex["params"]
+    steps = args.steps if args.steps != N_ROOTS else 8
+    prof = profile_json("search_kernel_gomoku_acp_prodigal_8x128_counters.md")
+    quiet = io.StringIO()
+    with contextlib.redirect_stdout(quiet):
+        e = MCTSNC((15, 15), 0, 225, search_time_limit=np.inf, search_steps_limit=ex["steps"], n_trees=p["n_trees"], n_playouts=p["n_playouts"],
+                   variant=p["variant"], device_memory=p["device_memory"], ucb_c=p["ucb_c"], seed=p["seed"], verbose_info=False, game="gomoku")
+        e.init_device_side_arrays()
+        apply_launch_options(e)
+        for _ in range(max(args.warmup, 1)):
+            e.reseed()
+            e.run(board, None, ex["turn"])
+        assert e.performance_info["playouts"] == ex["playouts"]      # the printed run
+        playouts = mcts_steps = plies = 0
+        dev = 0.0
+        stage = dict(select=0.0, expand=0.0, playout=0.0, backup=0.0)
+        alg = dict(select=0, expand=0, playout=0, backup=0, total=0)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            e.reseed()
+            e.run(board, None, ex["turn"])
+            playouts += e.performance_info["playouts"]
+            mcts_steps += e.steps
+            plies += e.performance_info["playout_plies"]
+            dev += e.time_device_loop
+            for k in stage:
+                stage[k] += getattr(e, "time_" + k)
+            ab = algorithmic_bytes(e._result, e.steps * p["n_trees"], acp=True, mn_e=225 + 1, A=225, P=p["n_playouts"])
+            for key in alg:
+                alg[key] += ab[key]
+        wall = time.perf_counter() - t0
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle.oracle import Oracle
+        cores = min(16, os.cpu_count() or 1)
+        o = Oracle("gomoku", (15, 15), 0, 225, p["n_trees"], p["n_playouts"], p["variant"], ucb_c=p["ucb_c"], seed=p["seed"],
+                   device_memory=p["device_memory"], threads=cores)
+        t1 = time.perf_counter()
+        o.run(board, None, ex["turn"], 40)
+        dt = time.perf_counter() - t1
+        cpu = {"value": int(o.result("root_ns").max()) / dt, "unit": "playouts/s", "cores": cores, "kind": "port",
+               "mcts_steps_per_s": 40 / dt, "sample": "the same position, 40 MCTS steps, CPU oracle with OpenMP over playouts"}
+    out = {"metric": "playouts/s + steps/s, Gomoku 15x15 ACP-prodigal 8x128 (the reference's README showcase) on 1 MI355X",
+           "value": playouts / wall, "unit": "playouts/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+           "ms_per_step": wall / steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bit boards + int32 counters (UCB in f64 rounded to f32)", "data": "synthetic",
+           "config": {"workload": "Gomoku 15x15, the 15-stone position of the reference's README, acp_prodigal n_trees=8 n_playouts=128 "
+                                  "ucb_c=2.0 device_memory=2GiB seed=0, 442 steps (what the reference's 5 s run reached: 88 steps/s, "
+                                  "18.8 M playouts/s there)"},
+           "mcts_steps_per_s": mcts_steps / wall, "playout_plies_per_s": plies / dev, "device_loop_share": dev / wall,
+           "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
+           "stage_achieved_gbs": {k: alg[k] / stage[k] / 1e9 for k in stage if stage[k]},
+           "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_launch"), dev / steps, prof or {},
+                                          "one search, gomoku::search_kernel_for<Gomoku, true> on 512 workgroups of 128 threads"),
+           "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
+                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
+                        "kernel": "mctsnc::gomoku::search_kernel_for<Gomoku, true>", "algorithmic_bytes_per_launch": alg["total"] / steps,
+                        "avg_launch_ms": dev / steps * 1e3,
+                        "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
+                        "note": "1.7 M playouts per step whose generators stay on chip: bound by the instruction stream of the "
+                                "playouts (LDS-resident boards, two workgroups per CU), not by memory"},
+           "cpu_baseline": cpu}
+    e._release()
+    print(json.dumps(out))
+
+
 def puct_gomoku_search(board, steps, search_steps, warmup, **kw):
     """`steps` timed searches of `search_steps` steps each; returns totals and the algorithmic bytes by phase."""
     from mcts_numba_cuda_amd.puct_gomoku import PUCTGomoku
@@ -562,7 +647,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device-to-device copy (the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE readings are scaled by) and exit")
-    ap.add_argument("--workload", default="c4", choices=("c4", "c4_many", "gomoku", "puct_select", "puct_gomoku"),
+    ap.add_argument("--workload", default="c4", choices=("c4", "c4_many", "gomoku", "gomoku_acp", "puct_select", "puct_gomoku"),
                     help="c4: the headline MCTS-NC search (default); puct_select: the reference's deep-wide PUCT selection "
                          "benchmark through puct_select_winner_recalc_launch; puct_gomoku: the Gomoku PUCT search loop")
     ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
@@ -586,6 +671,8 @@ def main():
 
     if args.workload == "gomoku":
         return bench_gomoku(args)
+    if args.workload == "gomoku_acp":
+        return bench_gomoku_acp(args)
     if args.workload == "c4_many":
         return bench_c4_many(args)
     if args.workload == "puct_select":
