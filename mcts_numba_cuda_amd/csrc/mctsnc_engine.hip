@@ -217,24 +217,29 @@ struct Budget {
 
 // Root of a Gomoku search: bitboards with bit = row * n + column; any arrangement of stones is accepted, as in the
 // reference (its outcome test only looks through the last stone placed).
-int gomoku_encode_root(const mctsnc_config &c, const int8_t *board, uint32_t bb[16]) {
-    for (int i = 0; i < 16; i++) bb[i] = 0;
+// Words per colour of a Gomoku position: 8 for boards of up to 16 x 16, 12 beyond (the kernels' two board formats).
+int gomoku_words(const mctsnc_config &c) { return (c.board_m > 16 || c.board_n > 16) ? gomoku::kMaxWords : 8; }
+
+int gomoku_encode_root(const mctsnc_config &c, const int8_t *board, uint32_t *bb /* [2 W] */) {
+    const int W = gomoku_words(c);
+    for (int i = 0; i < 2 * W; i++) bb[i] = 0;
     for (int cell = 0; cell < c.board_m * c.board_n; cell++) {
         const int8_t v = board[cell];
         if (v != -1 && v != 0 && v != 1) return fail(MCTSNC_E_ROOT, "board holds %d at cell %d; cells must be -1, 0 or +1", v, cell);
         if (v == 1) bb[cell >> 5] |= 1u << (cell & 31);
-        if (v == -1) bb[8 + (cell >> 5)] |= 1u << (cell & 31);
+        if (v == -1) bb[W + (cell >> 5)] |= 1u << (cell & 31);
     }
     return MCTSNC_OK;
 }
 
 // Playouts a Gomoku workgroup runs at a time (a power of two, as n_playouts is: the kernel finds a playout's line words
 // with a shift): as many as there are playouts, up to 256, and no more than fit the LDS of a CU beside the kernel's own
-// 8 KB (16 x 16 boards: 128; more playouts then run in rounds).
+// 8 KB (16 x 16 boards: 128, 19 x 19: 64; more playouts then run in rounds).
 int gomoku_block(const mctsnc_config &c) {
     int slots = c.n_playouts < 64 ? 64 : (c.n_playouts > gomoku::kMaxThreads ? gomoku::kMaxThreads : c.n_playouts);
     const size_t lds_of_a_cu = 160 * 1024, kernels_own = 8 * 1024;
-    while (slots > 64 && gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, slots) + kernels_own > lds_of_a_cu) slots /= 2;
+    const bool wide = gomoku_words(c) > 8;
+    while (slots > 64 && gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, slots, wide) + kernels_own > lds_of_a_cu) slots /= 2;
     return slots;
 }
 
@@ -387,7 +392,7 @@ C4BatchBuffers carve_c4(Workspace &w, size_t n_refs, size_t n, int A) {
 struct GomokuBatchBuffers { gomoku::TreeRef *refs; uint32_t *root_bb; int32_t *turns; unsigned char *reduced; };
 GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t n, int A) {
     GomokuBatchBuffers b;
-    b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(16 * n_refs); b.turns = w.take<int32_t>(n_refs);
+    b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(2 * gomoku::kMaxWords * n_refs); b.turns = w.take<int32_t>(n_refs);
     b.reduced = w.take<unsigned char>(n * reduced_stride(A));
     return b;
 }
@@ -628,13 +633,15 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     const int T = c.n_trees, cells = c.board_m * c.board_n, A = c.max_actions;
     const int n_refs = n * T;
     const double t_start = now_s();
-    std::vector<uint32_t> bb((size_t)n_refs * 16);
+    const int W = gomoku_words(c), RW = 2 * W;   // words of a root position
+    const bool wide = W > 8;
+    std::vector<uint32_t> bb((size_t)n_refs * RW);
     std::vector<int32_t> tr((size_t)n_refs);
     for (int i = 0; i < n; i++) {
-        uint32_t b16[16];
-        int rc = gomoku_encode_root(c, boards + (size_t)i * cells, b16);
+        uint32_t root[2 * gomoku::kMaxWords];
+        int rc = gomoku_encode_root(c, boards + (size_t)i * cells, root);
         if (rc) return rc;
-        for (int t = 0; t < T; t++) { memcpy(&bb[16 * ((size_t)i * T + t)], b16, sizeof b16); tr[(size_t)i * T + t] = turns[i]; }
+        for (int t = 0; t < T; t++) { memcpy(&bb[RW * ((size_t)i * T + t)], root, sizeof(uint32_t) * RW); tr[(size_t)i * T + t] = turns[i]; }
     }
     // trees of the searches with the fewest stones on the board (the longest playouts) first, as for Connect 4; the
     // groups of trees that consecutive launches take then hold searches of similar length
@@ -643,11 +650,11 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     if (n > 1) {
         std::vector<int> stones((size_t)n, 0);
         for (int i = 0; i < n; i++)
-            for (int w = 0; w < 16; w++) stones[i] += __builtin_popcount(bb[16 * (size_t)i * T + w]);
+            for (int w = 0; w < RW; w++) stones[i] += __builtin_popcount(bb[RW * (size_t)i * T + w]);
         std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return stones[a / T] < stones[b / T]; });
         std::vector<uint32_t> bb2(bb.size());
         std::vector<int32_t> tr2(tr.size());
-        for (int k = 0; k < n_refs; k++) { memcpy(&bb2[16 * (size_t)k], &bb[16 * (size_t)order[k]], 16 * sizeof(uint32_t)); tr2[k] = tr[order[k]]; }
+        for (int k = 0; k < n_refs; k++) { memcpy(&bb2[RW * (size_t)k], &bb[RW * (size_t)order[k]], RW * sizeof(uint32_t)); tr2[k] = tr[order[k]]; }
         bb.swap(bb2); tr.swap(tr2);
     }
     GomokuBatchBuffers buf{e0->g_refs, e0->g_root_bb, e0->d_root_turns, e0->d_reduced};
@@ -666,7 +673,7 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     uint32_t *const d_bb = buf.root_bb;
     int32_t *const d_turns = buf.turns;
     hipStream_t stream = e0->stream;
-    HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint32_t) * 16 * n_refs, hipMemcpyHostToDevice, stream));
+    HIP_TRY(hipMemcpyAsync(d_bb, bb.data(), sizeof(uint32_t) * RW * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemcpyAsync(d_turns, tr.data(), sizeof(int32_t) * n_refs, hipMemcpyHostToDevice, stream));
     HIP_TRY(hipMemsetAsync(e0->d_abort, 0, sizeof(int32_t), stream));
     hipLaunchKernelGGL(gomoku::reset_kernel, dim3((n_refs + 63) / 64), dim3(64), 0, stream, d_refs, n_refs, d_bb, d_turns);
@@ -683,10 +690,12 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     args.spin_limit = opt[MCTSNC_OPT_SPIN_LIMIT] > 0 ? (uint32_t)opt[MCTSNC_OPT_SPIN_LIMIT] : gomoku::kSpinLimit;
     args.prep_levels = opt[MCTSNC_OPT_PREP_LEVELS] >= 0 ? std::min(opt[MCTSNC_OPT_PREP_LEVELS], gomoku::kPrepLevels) : gomoku::kPrepLevels;
     const dim3 block(e0->block);
-    const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots);
+    const size_t lds = gomoku::playout_lds_bytes(cells, 3 * (c.board_m + c.board_n) - 2, e0->slots, wide);
+    // the kernel of this engine's variant and board format
+    auto *const kernel = e0->acp ? (wide ? gomoku::search_kernel<true, gomoku::kMaxWords> : gomoku::search_kernel<true, 8>)
+                                 : (wide ? gomoku::search_kernel<false, gomoku::kMaxWords> : gomoku::search_kernel<false, 8>);
     // the limit is a setting of the kernel function, not of this engine: an engine of another shape may have changed it
-    if (e0->acp) HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    else HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // The all-children kernel synchronises the workgroups of a tree with each other, so a launch must be resident as a
     // whole: more trees than the device holds G workgroups each for are searched by consecutive launches over equal
     // groups of trees, every group for the same number of steps before the budget is looked at again.
@@ -694,7 +703,7 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     if (e0->acp) {
         int per_cu = 0, cus = 0;
         HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
-        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e0->block, lds));
+        HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, e0->block, lds));
         const int64_t fit = (int64_t)per_cu * cus / e0->G;   // trees per launch
         if (fit < 1) return fail(MCTSNC_E_INVALID, "the device cannot hold the %d workgroups of a tree at once", e0->G);
         const int64_t n_groups = (n_refs + fit - 1) / fit;
@@ -709,16 +718,11 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
             args.refs = d_refs + start;
             args.n_refs = std::min(group, n_refs - start);
             const dim3 grid(e0->G * args.n_refs);
-            if (e0->acp) {
-                if (plain_launch) {
-                    hipLaunchKernelGGL(gomoku::search_kernel<true>, grid, block, lds, stream, args);
-                    HIP_TRY(hipGetLastError());
-                } else {
-                    void *kargs[] = {&args};
-                    HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(gomoku::search_kernel<true>), grid, block, kargs, (unsigned)lds, stream));
-                }
+            if (e0->acp && !plain_launch) {
+                void *kargs[] = {&args};
+                HIP_TRY(hipLaunchCooperativeKernel(reinterpret_cast<void *>(kernel), grid, block, kargs, (unsigned)lds, stream));
             } else {
-                hipLaunchKernelGGL(gomoku::search_kernel<false>, grid, block, lds, stream, args);
+                hipLaunchKernelGGL(kernel, grid, block, lds, stream, args);
                 HIP_TRY(hipGetLastError());
             }
         }
@@ -774,6 +778,7 @@ int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, siz
     }
     const int64_t sz = h.size;
     const size_t S = (size_t)c.max_tree_size;
+    const int W = gomoku_words(c);
     std::vector<gomoku::Node> nd((size_t)sz);
     std::vector<gomoku::Stat> st((size_t)sz);
     HIP_TRY(hipMemcpy(nd.data(), e->g_nodes + (size_t)tree * S, sizeof(gomoku::Node) * (size_t)sz, hipMemcpyDeviceToHost));
@@ -788,7 +793,7 @@ int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, siz
                 int rank = 0;
                 const bool expanded = !(x.flags & gomoku::kLeaf);
                 for (int a = 0; a < A; a++) {
-                    const bool empty = !((x.bb_pos[a >> 5] | x.bb_neg[a >> 5]) >> (a & 31) & 1u);
+                    const bool empty = !((x.bb[a >> 5] | x.bb[W + (a >> 5)]) >> (a & 31) & 1u);
                     row[1 + a] = (expanded && empty && rank < x.n_children) ? x.child_base + rank : -1;
                     if (empty) rank++;
                 }
@@ -804,7 +809,7 @@ int read_gomoku(mctsnc_engine *e, int32_t array_id, int32_t tree, void *dst, siz
             case MCTSNC_ARR_BOARDS: {
                 int8_t *b = (int8_t *)dst + i * m * n;
                 for (int cell = 0; cell < m * n; cell++)
-                    b[cell] = ((x.bb_pos[cell >> 5] >> (cell & 31)) & 1u) ? 1 : (((x.bb_neg[cell >> 5] >> (cell & 31)) & 1u) ? -1 : 0);
+                    b[cell] = ((x.bb[cell >> 5] >> (cell & 31)) & 1u) ? 1 : (((x.bb[W + (cell >> 5)] >> (cell & 31)) & 1u) ? -1 : 0);
                 break;
             }
             case MCTSNC_ARR_EXTRA_INFOS: memset((int8_t *)dst + i * E, 0, (size_t)E); break;
@@ -831,8 +836,8 @@ int mctsnc_create(const mctsnc_config *cfg, mctsnc_engine **out) {
         if (c.max_actions != c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 has one action per column (%d), got max_actions = %d", c.board_n, c.max_actions);
         if (c.extra_info_memory < c.board_n) return fail(MCTSNC_E_INVALID, "Connect 4 keeps the column fills in extra_info: needs >= %d bytes", c.board_n);
     } else {
-        if (c.board_m < 5 || c.board_n < 5 || c.board_m > 16 || c.board_n > 16)
-            return fail(MCTSNC_E_INVALID, "Gomoku board %dx%d unsupported: sides must be in [5, 16]", c.board_m, c.board_n);
+        if (c.board_m < 5 || c.board_n < 5 || c.board_m > gomoku::kMaxSide || c.board_n > gomoku::kMaxSide || c.board_m * c.board_n > gomoku::kMaxCells)
+            return fail(MCTSNC_E_INVALID, "Gomoku board %dx%d unsupported: sides must be in [5, %d] and the board at most %d cells", c.board_m, c.board_n, gomoku::kMaxSide, gomoku::kMaxCells);
         if (c.max_actions != c.board_m * c.board_n) return fail(MCTSNC_E_INVALID, "Gomoku has one action per cell (%d), got max_actions = %d", c.board_m * c.board_n, c.max_actions);
         if (c.extra_info_memory < 1) return fail(MCTSNC_E_INVALID, "extra_info_memory must be >= 1");
     }
@@ -914,7 +919,7 @@ static int init_device_impl(mctsnc_engine *e) {
         HIP_TRY(hipMalloc(&e->g_poc, sizeof(int32_t) * 2 * A * T));
         HIP_TRY(hipMemset(e->g_poc, 0, sizeof(int32_t) * 2 * A * T));
         HIP_TRY(hipMalloc(&e->g_path, sizeof(int32_t) * gomoku::kMaxPath * T));
-        HIP_TRY(hipMalloc(&e->g_root_bb, sizeof(uint32_t) * 16 * T));
+        HIP_TRY(hipMalloc(&e->g_root_bb, sizeof(uint32_t) * 2 * gomoku::kMaxWords * T));
         std::vector<gomoku::TreeRef> refs((size_t)T);
         for (int t = 0; t < T; t++) {
             refs[t].nodes = e->g_nodes + (size_t)t * S;
@@ -926,17 +931,20 @@ static int init_device_impl(mctsnc_engine *e) {
             refs[t].root_ae = e->g_root_ae + (size_t)t * (A + 2);
             refs[t].poc = e->g_poc + (size_t)t * 2 * A;
             refs[t].path = e->g_path + (size_t)t * gomoku::kMaxPath;
+            refs[t].words = gomoku_words(c);
         }
         HIP_TRY(hipMemcpy(e->g_refs, refs.data(), sizeof(gomoku::TreeRef) * T, hipMemcpyHostToDevice));
         e->hg_refs = refs;
         // the playout state of a workgroup can need more LDS than the default limit allows
-        const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->slots);
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(gomoku::search_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        const bool wide = gomoku_words(c) > 8;
+        const size_t lds = gomoku::playout_lds_bytes(c.board_m * c.board_n, 3 * (c.board_m + c.board_n) - 2, e->slots, wide);
+        auto *const kernel = e->acp ? (wide ? gomoku::search_kernel<true, gomoku::kMaxWords> : gomoku::search_kernel<true, 8>)
+                                    : (wide ? gomoku::search_kernel<false, gomoku::kMaxWords> : gomoku::search_kernel<false, 8>);
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         if (e->acp) {
             // as many workgroups per tree as stay resident together (each takes every G-th child of the expanded node)
             int per_cu = 0, cus = 0;
-            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gomoku::search_kernel<true>, e->block, lds));
+            HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, e->block, lds));
             HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, c.device));
             const int64_t resident = (int64_t)per_cu * cus;
             const int64_t g_fit = resident / T;

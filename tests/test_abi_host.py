@@ -152,7 +152,8 @@ def test_board_shapes_beyond_the_engine_get_a_reference_style_message(capsys):
     """The reference's caps (32 x 32 cells, 512 actions, src/mctsnc.py:180-197) admit boards this engine's kernels do
     not take; the class says so in the reference's message style before it raises, without touching the device."""
     from mcts_numba_cuda_amd import MCTSNC
-    for kw, part in ((dict(state_board_shape=(19, 19), state_extra_info_memory=0, state_max_actions=361, game="gomoku"), "16 x 16"),
+    for kw, part in ((dict(state_board_shape=(20, 24), state_extra_info_memory=0, state_max_actions=480, game="gomoku"), "384 cells"),
+                     (dict(state_board_shape=(5, 25), state_extra_info_memory=0, state_max_actions=125, game="gomoku"), "sides up to 24"),
                      (dict(state_board_shape=(6, 10), state_extra_info_memory=10, state_max_actions=10), "columns <= 8")):
         e = MCTSNC(verbose_info=False, **kw)
         with pytest.raises(ValueError):

@@ -111,6 +111,63 @@ def test_gomoku_sixteen_wide_boards(variant):
         compare_with_oracle(e, o, board, None, turn, steps if variant.startswith("ocp") else max(3, steps // 10))
 
 
+@pytest.mark.parametrize("variant,steps", [("ocp_thrifty", 40), ("ocp_prodigal", 40), ("acp_thrifty", 3), ("acp_prodigal", 3)])
+def test_gomoku_boards_beyond_sixteen(variant, steps):
+    """Boards with a side beyond 16 are held in the engine's second format (12 words per colour, 16-bit list entries,
+    one line word per colour): 19 x 19, a rectangle, the 384 cells the format holds at most, and boards one line of
+    which is 24 long while the other side is short (deep trees, wins, draws).  Two consecutive searches each, every
+    array against the oracle; more than 256 children per node exercise the arg-max tie rule on nine bits."""
+    rng = np.random.default_rng(19)
+    for (m, n), scale in (((19, 19), 1.0), ((17, 20), 1.0), ((24, 16), 0.5), ((5, 24), 3.0), ((20, 5), 3.0)):
+        e, o = engines(variant, 2, 64, m, n, seed=7)
+        for stones in (0, 12):
+            board, turn = random_gomoku_root(rng, m, n, stones)
+            compare_with_oracle(e, o, board, None, turn, max(2, int(steps * scale)))
+
+
+def test_gomoku_wide_board_children_that_complete_lines():
+    """19 x 19: cells that complete exactly five in the part of the board the 16-wide format does not reach (columns and
+    rows 16 to 18, the diagonals that end there), a cell that would make six, and a row of five that ends on the last
+    column."""
+    board = np.zeros((19, 19), np.int8)
+    board[17, 14:18] = 1                                # four in row 17, columns 14..17: (17,13) and (17,18) win
+    board[2, [12, 13, 15, 16, 17]] = 1                  # (2,14) makes six: not a win
+    board[14:18, 18] = 1                                # column 18, rows 14..17: (13,18) and (18,18) win
+    for k in range(4):
+        board[14 + k, 3 - k] = 1                        # anti-diagonal (14,3)..(17,0): (13,4) wins, the other end is off the board
+        board[5 + k, 14 + k] = -1                       # diagonal of -1 (5,14)..(8,17): its replies at (4,13) and (9,18) win
+    board[[0, 0, 9, 12, 18], [0, 7, 2, 9, 10]] = -1
+    for variant, steps in (("acp_prodigal", 4), ("ocp_thrifty", 120)):
+        e, o = engines(variant, 2, 64, 19, 19, seed=9)
+        compare_with_oracle(e, o, board, None, 1, steps)
+
+
+def test_gomoku_wide_board_other_playout_counts_and_batches():
+    """19 x 19 with 256 playouts (the workgroup holds 64 at a time: four rounds) and with 16; three searches in one
+    pass against separate runs."""
+    from mcts_numba_cuda_amd import MCTSNC, run_batch
+    rng = np.random.default_rng(23)
+    for variant, P, steps in (("ocp_prodigal", 256, 12), ("acp_thrifty", 256, 2), ("ocp_thrifty", 16, 40)):
+        e, o = engines(variant, 2, P, 19, 19, seed=2)
+        board, turn = random_gomoku_root(rng, 19, 19, 20)
+        compare_with_oracle(e, o, board, None, turn, steps)
+
+    def mk():
+        e = MCTSNC((19, 19), 0, 361, search_time_limit=np.inf, n_trees=2, n_playouts=64, variant="acp_prodigal", device_memory=0.5,
+                   seed=6, verbose_info=False, game="gomoku")
+        e.init_device_side_arrays()
+        return e
+    roots = [random_gomoku_root(rng, 19, 19, stones) for stones in (30, 2, 11)]
+    batch, single = [mk() for _ in roots], [mk() for _ in roots]
+    run_batch(batch, [r[0] for r in roots], None, [r[1] for r in roots], forced_search_steps_limit=3)
+    for e, r in zip(single, roots):
+        e.run(r[0], None, r[1], forced_search_steps_limit=3)
+    for eb, es in zip(batch, single):
+        assert eb.actions_info == es.actions_info
+        for name in ("trees", "ns", "ns_wins", "boards"):
+            np.testing.assert_array_equal(eb.read_array(name, 1), es.read_array(name, 1))
+
+
 @pytest.mark.parametrize("variant,steps", [("ocp_prodigal", 20), ("acp_thrifty", 3)])
 def test_gomoku_largest_board_with_256_playouts(variant, steps):
     """On 16x16 the lists and line words of 256 playouts do not fit the LDS of a CU: the workgroup then holds 128 at a
