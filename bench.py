@@ -354,13 +354,13 @@ def bench_gomoku(args):
                        "mcts_steps_per_s_all_roots": sum(x.steps for x in engines) / bt, "ms_per_pass": bt * 1e3, "kernel_ms": kt * 1e3,
                        "playout_plies_per_s": bplies / kt, "algorithmic_GB_per_s": bbytes / kt / 1e9, "hbm_frac": bbytes / kt / 1e9 / HBM_PEAK_GBS,
                        "valu": valu_roofline((prof or {}).get("batched_32_roots", {}).get("sq_insts_valu_per_pass"), kt, prof or {},
-                                             "one pass over the 32 roots, gomoku::search_kernel_for<Gomoku, false> with 128 workgroups")}
+                                             "one pass over the 32 roots, gomoku::search_kernel_for<Gomoku, false, 8> with 128 workgroups")}
             for x in engines[1:]:
                 x._release()
     per_root = (prof or {}).get("sq_insts_valu_per_root")
     roofline_valu = None
     if per_root and len(per_root) >= steps:
-        roofline_valu = valu_roofline(sum(per_root[:steps]), dev, prof, "the timed single searches, gomoku::search_kernel_for<Gomoku, false> on 4 workgroups")
+        roofline_valu = valu_roofline(sum(per_root[:steps]), dev, prof, "the timed single searches, gomoku::search_kernel_for<Gomoku, false, 8> on 4 workgroups")
     cpu = None
     if not args.no_cpu_baseline:
         from oracle.oracle import Oracle
@@ -381,7 +381,7 @@ def bench_gomoku(args):
            "batched": batched, "roofline_valu": roofline_valu,
            "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
-                        "kernel": "mctsnc::gomoku::search_kernel_for<Gomoku, false>", "algorithmic_bytes_per_launch": alg["total"] / steps,
+                        "kernel": "mctsnc::gomoku::search_kernel_for<Gomoku, false, 8>", "algorithmic_bytes_per_launch": alg["total"] / steps,
                         "avg_launch_ms": dev / steps * 1e3,
                         "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
                         "note": "four workgroups of two wavefronts: bound by the length of the longest playout "
@@ -462,11 +462,11 @@ def bench_gomoku_acp(args):
            "stage_ms_per_mcts_step": {k: v / mcts_steps * 1e3 for k, v in stage.items()},
            "stage_achieved_gbs": {k: alg[k] / stage[k] / 1e9 for k in stage if stage[k]},
            "roofline_valu": valu_roofline((prof or {}).get("sq_insts_valu_per_launch"), dev / steps, prof or {},
-                                          "one search, gomoku::search_kernel_for<Gomoku, true> on 512 workgroups of 128 threads"),
+                                          "one search, gomoku::search_kernel_for<Gomoku, true, 8> on 512 workgroups of 128 threads"),
            "roofline": {"bound": "hbm", "achieved": alg["total"] / dev / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": alg["total"] / dev / 1e9 / HBM_PEAK_GBS, "traffic": (prof or {}).get("traffic_bytes_per_launch"),
                         "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
-                        "kernel": "mctsnc::gomoku::search_kernel_for<Gomoku, true>", "algorithmic_bytes_per_launch": alg["total"] / steps,
+                        "kernel": "mctsnc::gomoku::search_kernel_for<Gomoku, true, 8>", "algorithmic_bytes_per_launch": alg["total"] / steps,
                         "avg_launch_ms": dev / steps * 1e3,
                         "stage_bytes_per_launch": {k: v / steps for k, v in alg.items() if k != "total"},
                         "note": "1.7 M playouts per step whose generators stay on chip: bound by the instruction stream of the "

@@ -59,7 +59,7 @@ struct __attribute__((aligned(128))) Node {
     uint8_t pad0;
     int16_t action;          // action that led here
     int32_t pad1[2];
-    uint32_t bb[24];         // W words of the stones of player +1, then W words of those of player -1 (W = 8 or 12), rest zero
+    uint32_t bb[24];         // W words of the stones of player +1, then W words of those of player -1 (W = 8 or 12), rest unused
 };
 static_assert(sizeof(Node) == 128, "node record must be 128 bytes");
 
@@ -457,7 +457,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             const uint32_t hit2 = Game::winning_starts(__builtin_amdgcn_perm(w_col, w_ant, sel)) & (win_j | (win_i << 16));
             return (hit | hit2) != 0 ? mover : (empties == 1 ? 0 : 2);
         };
-        // Records and counters of the children j0, j0 + stride, ...: the record as eight 16-byte stores (field layout of
+        // Records and counters of the children j0, j0 + stride, ...: the record as 2 + W / 2 16-byte stores (field layout of
         // Node), typed as device memory; the counters of child `played` are left to the thread that stores its result.
         auto create_children = [=](int j0, int stride, int played) {
             typedef __attribute__((address_space(1))) i32x4 *DeviceQuads;
@@ -466,23 +466,19 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 const uint32_t a_word = (uint32_t)a >> 5, a_bit = 1u << (a & 31);
                 const int outcome = child_outcome(a);
                 s_out[j] = (int8_t)outcome;
-                uint32_t bb[24];   // (constant indices after unrolling: registers)
+                uint32_t bb[2 * W];   // (constant indices after unrolling: registers)
 #pragma unroll
                 for (int w = 0; w < W; w++) {
                     const uint32_t add = (uint32_t)w == a_word ? a_bit : 0u;
                     bb[w] = s_bb[w] | (mover == 1 ? add : 0u); bb[W + w] = s_bb[W + w] | (mover == 1 ? 0u : add);
                 }
-#pragma unroll
-                for (int w = 2 * W; w < 24; w++) bb[w] = 0u;
                 const uint32_t flags = (uint32_t)kLeaf | (outcome != 2 ? (uint32_t)kTerminal : 0u);
                 const DeviceQuads rec = (DeviceQuads)(nodes + size + j);
-                const i32x4 zero = {0, 0, 0, 0};
                 rec[0] = i32x4{-1, leaf.node, 0, -1};   // child_base, parent, n_children, best_child
                 rec[1] = i32x4{(int32_t)(((uint32_t)(L + 1) & 0xffffu) | (((uint32_t)(-mover) & 0xffu) << 16) | (((uint32_t)outcome & 0xffu) << 24)),
                                (int32_t)(flags | ((uint32_t)a << 16)), 0, 0};   // depth, turn, outcome; flags, action
 #pragma unroll
-                for (int q = 0; q < 6; q++) rec[2 + q] = i32x4{(int32_t)bb[4 * q], (int32_t)bb[4 * q + 1], (int32_t)bb[4 * q + 2], (int32_t)bb[4 * q + 3]};
-                (void)zero;
+                for (int q = 0; q < W / 2; q++) rec[2 + q] = i32x4{(int32_t)bb[4 * q], (int32_t)bb[4 * q + 1], (int32_t)bb[4 * q + 2], (int32_t)bb[4 * q + 3]};
                 if (j != played) *(DeviceQuads)(stats + size + j) = i32x4{0, 0, a, 0};
             }
         };

@@ -390,9 +390,9 @@ C4BatchBuffers carve_c4(Workspace &w, size_t n_refs, size_t n, int A) {
 }
 
 struct GomokuBatchBuffers { gomoku::TreeRef *refs; uint32_t *root_bb; int32_t *turns; unsigned char *reduced; };
-GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t n, int A) {
+GomokuBatchBuffers carve_gomoku(Workspace &w, size_t n_refs, size_t n, int A, int words) {
     GomokuBatchBuffers b;
-    b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(2 * gomoku::kMaxWords * n_refs); b.turns = w.take<int32_t>(n_refs);
+    b.refs = w.take<gomoku::TreeRef>(n_refs); b.root_bb = w.take<uint32_t>(2 * (size_t)words * n_refs); b.turns = w.take<int32_t>(n_refs);
     b.reduced = w.take<unsigned char>(n * reduced_stride(A));
     return b;
 }
@@ -661,10 +661,10 @@ int run_many_gomoku(mctsnc_engine **engines, int n, const int8_t *boards, const 
     BlockHolder block_holder;
     if (n > 1 || fixed) {
         Workspace count, ws;
-        carve_gomoku(count, (size_t)n_refs, (size_t)n, A);
+        carve_gomoku(count, (size_t)n_refs, (size_t)n, A, W);
         int rc = block_holder.get(fixed, count.used, ws);
         if (rc) return rc;
-        buf = carve_gomoku(ws, (size_t)n_refs, (size_t)n, A);
+        buf = carve_gomoku(ws, (size_t)n_refs, (size_t)n, A, W);
         std::vector<gomoku::TreeRef> sorted((size_t)n_refs);
         for (int k = 0; k < n_refs; k++) sorted[k] = engines[order[k] / T]->hg_refs[order[k] % T];
         HIP_TRY(hipMemcpy(buf.refs, sorted.data(), sizeof(gomoku::TreeRef) * n_refs, hipMemcpyHostToDevice));

@@ -98,7 +98,7 @@ def test_two_calls_in_a_row_equal_the_allocating_entry_point(game, variant, n_tr
 
 def test_a_batch_beyond_the_scratch_is_rejected_with_both_sizes():
     from mcts_numba_cuda_amd import MCTSNC, _lib
-    n = 60   # 60 x 512 trees of a 9x9 board need 140 bytes per tree + 2560 per search = 4.5 MB, more than the 4 MiB of the static array
+    n = 60   # 60 x 512 trees of a 9x9 board need 148 bytes per tree + 2560 per search = 4.7 MB, more than the 4 MiB of the static array
     engines = []
     for _ in range(n):
         e = MCTSNC((9, 9), 0, 81, search_time_limit=np.inf, search_steps_limit=np.inf, n_trees=512, n_playouts=1, variant="ocp_prodigal",
