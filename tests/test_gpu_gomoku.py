@@ -197,6 +197,21 @@ def test_gomoku_many_trees(variant, T, steps):
         compare_with_oracle(e, o, board, None, turn, steps)
 
 
+def test_gomoku_engines_of_different_shapes_alive_together():
+    """The dynamic-LDS limit is a setting of the kernel function, not of an engine: an engine created earlier, whose
+    playouts need more LDS than the latest one's, must still launch.  Three engines (16 x 16 with 128 slots: 81 KB;
+    6 x 6: 3 KB; 19 x 19 in the other board format: 104 KB) are created first and then used in turn, twice."""
+    rng = np.random.default_rng(31)
+    made = []
+    for variant, (m, n), P, steps in (("acp_thrifty", (16, 16), 256, 2), ("ocp_prodigal", (6, 6), 64, 60), ("acp_prodigal", (19, 19), 64, 2),
+                                      ("ocp_thrifty", (15, 15), 128, 30)):
+        e, o = engines(variant, 2, P, m, n, seed=13)
+        made.append((e, o, random_gomoku_root(rng, m, n, 6), steps))
+    for _ in range(2):
+        for e, o, (board, turn), steps in made:
+            compare_with_oracle(e, o, board, None, turn, steps)
+
+
 def test_gomoku_one_child_batch_equals_single_runs():
     """Five one-child searches of positions with different numbers of stones in one pass (the library orders the trees
     of a batch by stones on the board) against separate runs, twice, so that the generators carry over on both sides."""
