@@ -85,6 +85,37 @@ int puct_edge_backup_launch(int virtual_loss, float *edge_W, int *edge_N, int *e
                             int trees, int nodes, int edges, int warps, int path_depth, void *stream);
 
 /*
+ * PUCT selection with node-level virtual loss (node_inflight[tree, child] += 1 along the selected path), the
+ * counterpart of puct_node_backup_launch below.  The reference has these two kernels in numba only, so there is no C
+ * symbol to replace: the entry points take the kernels' arguments in the kernels' order, the array shapes as trailing
+ * integers and the stream, like the launchers above.
+ *   puct_node_select_preclaim_launch       _select_kernel_native, src/puct/puct_gpu_v2.py:573-697: every candidate
+ *                                          child is claimed before it is scored (the score sees the claims of the
+ *                                          traversals ahead of it), the losers are released afterwards; ties go to
+ *                                          the edge index rotated by wid.
+ *   puct_node_select_winner_recalc_launch  _select_kernel_winner_recalc, :700-840: scores from the counters as read,
+ *                                          a counter compare-and-swap on the winner only; when that child already
+ *                                          carried claims the claim is released and the edges are scored once more
+ *                                          without it; ties go to the smaller edge index.
+ * Selection word (:352-354, no reason field, no BUSY kind): (kind << 22) | (expand_slot << 14) | node; a traversal
+ * that ends without a selection (no expansion ticket left, no edge that leads to a node of the tree, inconsistent
+ * node words) has given its claims back and reports PUCT_PACKED_INVALID_V2 with path length 0.
+ */
+#define PUCT_PACKED_INVALID_V2 ((PUCT_SELECT_INVALID << PUCT_PACKED_KIND_SHIFT) | PUCT_PACKED_NODE_MASK)
+int puct_node_select_preclaim_launch(float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                                     const float *edge_prior, const float *edge_W, const int *edge_N,
+                                     int *node_inflight, int *node_expand_inflight, const int *node_expanded,
+                                     const int *node_count, int *out_selected_node, int *out_path_eids,
+                                     int *out_path_len, int trees, int nodes, int edges, int warps, int path_depth,
+                                     void *stream);
+int puct_node_select_winner_recalc_launch(float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                                          const float *edge_prior, const float *edge_W, const int *edge_N,
+                                          int *node_inflight, int *node_expand_inflight, const int *node_expanded,
+                                          const int *node_count, int *out_selected_node, int *out_path_eids,
+                                          int *out_path_len, int trees, int nodes, int edges, int warps,
+                                          int path_depth, void *stream);
+
+/*
  * Backup with node-level virtual loss: the kernel _backup_kernel_native of src/puct/puct_gpu_v2.py:847-927 with its
  * argument order (array shapes become the trailing integers).  The selection word is read with the v2 layout
  * (kind = word >> 22, no reason field, :879,903-905).

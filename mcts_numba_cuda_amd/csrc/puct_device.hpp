@@ -1,6 +1,7 @@
 // Device side of PUCT selection and backup with virtual loss for gfx950 (wave64): one 64-lane wavefront per traversal.
 //
-// Semantics follow src/puct/puct_gpu_v3_cpp.cu:38-448 (selection) and src/puct/puct_gpu_v2.py:847-927 (backup); the
+// Semantics follow src/puct/puct_gpu_v3_cpp.cu:38-448 (selection with edge-level virtual loss),
+// src/puct/puct_gpu_v2.py:573-840 (the two selections with node-level virtual loss) and :847-927 (backup); the
 // wavefront-level organisation is this library's own:
 //   * the first 64 edges of a node (all of them for almost every node under progressive widening) are loaded once,
 //     together with the node's own words, before anything about the node is known, so a level costs one round of
@@ -334,6 +335,251 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
             atomicAdd(&a.work[(size_t)tree * 8 + 6], (unsigned long long)levels);
             atomicAdd(&a.work[(size_t)tree * 8 + 7], (unsigned long long)edges_seen);
         }
+    }
+}
+
+// ---- selection with node-level virtual loss ------------------------------------------------------------------------
+// The two selection kernels of src/puct/puct_gpu_v2.py, whose virtual loss lives in node_inflight[tree, child] and is
+// what backup_traversal<true> below takes back: _select_kernel_native (:573-697; every candidate child is claimed
+// before it is scored and the losers are released afterwards) and _select_kernel_winner_recalc (:700-840; scores from
+// the counters as read, a counter compare-and-swap on the winner only, one re-evaluation without the first winner
+// when that child already carried claims).  Their selection word has no reason field and no BUSY kind: a traversal
+// that cannot get an expansion ticket, or finds no edge, gives its claims back and reports PACKED_INVALID with length 0.
+struct NodeSelectArgs {
+    float cpuct, c_pw, alpha_pw;
+    const int *edge_child_id;
+    const float *edge_prior;
+    const float *edge_W;
+    const int *edge_N;
+    int *node_inflight;
+    int *node_expand_inflight;
+    const int *node_expanded;
+    const int *node_count;
+    int *out_selected_node;
+    int *out_path_eids;
+    int *out_path_len;
+    int trees, nodes, edges, warps, path_depth;
+};
+
+constexpr int kClaimAttempts = 8;   // MAX_SELECT_RETRY, src/puct/puct_gpu_v2.py:33
+constexpr int kPackedInvalidV2 = (PUCT_SELECT_INVALID << PUCT_PACKED_KIND_SHIFT) | PUCT_PACKED_NODE_MASK;
+
+__device__ __forceinline__ int pack_selection_v2(int kind, int node, int slot) {
+    return (kind << PUCT_PACKED_KIND_SHIFT) | (slot << PUCT_PACKED_SLOT_SHIFT) | node;
+}
+
+// src/puct/puct_gpu_v2.py:291-310: the claims of the first `depth` path entries live on the child each entry leads to.
+__device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, const int *path, int tree, int depth, int lane,
+                                                   int node_limit) {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");   // lane 0 stored the entries
+    for (int d = lane; d < depth; d += kWave) {
+        const int encoded = load_relaxed(path + d);
+        if (encoded < 0) continue;
+        const int parent = encoded >> 8, slot = encoded & 0xFF;
+        if (parent < node_limit && slot < a.edges) {
+            const int child = a.edge_child_id[((size_t)tree * a.nodes + parent) * a.edges + slot];
+            if (child >= 0 && child < node_limit) atomicSub(&a.node_inflight[(size_t)tree * a.nodes + child], 1);
+        }
+    }
+}
+
+// src/puct/puct_gpu_v2.py:313-349, called by one lane: one more virtual visit on `counter`, taken with compare-and-swap
+// on the value read (a counter, not a lock), after kClaimAttempts lost exchanges with a plain atomic add.
+// conflict = the counter already held visits when this claim went in.
+__device__ __forceinline__ void claim_counter(int *counter, int &held, int &conflict) {
+    held = 0, conflict = 0;
+    bool can_claim = true;
+    for (int attempt = 0; attempt < kClaimAttempts && !held; ++attempt) {
+        const int old = load_relaxed(counter);
+        if (old < 0 || old >= INT32_MAX) {
+            can_claim = false;
+            break;
+        }
+        if (atomicCAS(counter, old, old + 1) == old) {
+            held = 1;
+            conflict = old > 0 ? 1 : 0;
+        }
+    }
+    if (!held && can_claim) {
+        const int old = atomicAdd(counter, 1);
+        held = 1;
+        conflict = old > 0 ? 1 : 0;
+    }
+}
+
+// One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.
+template <bool PRECLAIM>
+__device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, int tree, int wid, int lane) {
+    const size_t out = (size_t)tree * a.warps + wid;
+    int *path = a.out_path_eids + out * a.path_depth;
+    const int node_limit = a.node_count[tree];
+    const int nodes = a.nodes, edges = a.edges;
+    const size_t trow = (size_t)tree * nodes;
+
+    int final_packed = kPackedInvalidV2, final_len = 0;
+    // src/puct/puct_gpu_v2.py:357-366
+    if (a.path_depth >= 1 && nodes > 0 && node_limit > 0 && node_limit <= nodes && node_limit <= PUCT_PACKED_NODE_LIMIT &&
+        edges > 0 && edges <= PUCT_PACKED_EDGE_MASK + 1) {
+        int node = 0, depth = 0;
+        while (true) {
+            if (node < 0 || node >= node_limit) {
+                rollback_node_path(a, path, tree, depth, lane, node_limit);
+                break;
+            }
+            if (depth >= a.path_depth) {   // the path buffer is full: stop before reading or claiming anything here
+                final_packed = pack_selection_v2(PUCT_SELECT_DEPTH_LIMIT, node, 0);
+                final_len = depth + 1;
+                break;
+            }
+            const size_t nrow = trow + node, erow = nrow * edges;
+            // the first 64 edges are requested together with the node's own words, before the node's width is known
+            int n[kPasses], f[kPasses], c[kPasses];
+            float p[kPasses], w[kPasses];
+            n[0] = 0, c[0] = -1, p[0] = 0.0f, w[0] = 0.0f;
+            if (lane < edges) {
+                c[0] = a.edge_child_id[erow + lane];
+                n[0] = a.edge_N[erow + lane];
+                p[0] = a.edge_prior[erow + lane];
+                w[0] = a.edge_W[erow + lane];
+            }
+            const int node_info = a.node_expanded[nrow];
+            const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
+            if (node_info == PUCT_NODE_EXPANDED_TERMINAL) {
+                final_packed = pack_selection_v2(PUCT_SELECT_TERMINAL, node, 0);
+                final_len = depth + 1;
+                break;
+            }
+            if (node_info < 0 || node_info > edges) {
+                rollback_node_path(a, path, tree, depth, lane, node_limit);
+                break;
+            }
+            const int cur_expanded = node_info;
+#pragma unroll
+            for (int i = 1; i < kPasses; ++i) {
+                n[i] = 0, c[i] = -1, p[i] = 0.0f, w[i] = 0.0f;
+                const int eid = lane + i * kWave;
+                if (i * kWave < cur_expanded && eid < cur_expanded) {
+                    c[i] = a.edge_child_id[erow + eid];
+                    n[i] = a.edge_N[erow + eid];
+                    p[i] = a.edge_prior[erow + eid];
+                    w[i] = a.edge_W[erow + eid];
+                }
+            }
+            // an edge takes part when it is expanded and leads to a node of the tree; its virtual visits are its child's
+            bool valid[kPasses];
+            int total = 0;
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) {
+                valid[i] = lane + i * kWave < cur_expanded && c[i] >= 0 && c[i] < node_limit;
+                f[i] = (i * kWave < cur_expanded && valid[i]) ? load_relaxed(a.node_inflight + trow + c[i]) : 0;
+            }
+#pragma unroll
+            for (int i = 0; i < kPasses; ++i) total += valid[i] ? n[i] + f[i] : 0;
+            total = wave_sum(total);
+            const int parent_eff = total > 1 ? total : 1;   // :407-416
+            const int allowed = (PRECLAIM && cur_expanded == 0) ? 1 : allowed_children(a.c_pw, a.alpha_pw, parent_eff, edges);
+
+            if (allowed > cur_expanded) {
+                // Expansion ticket, :389-403.  Tickets are only given back by the backup, and a ticket beyond the quota is
+                // returned at once, so a counter that already shows the quota used up stays that way for this launch.
+                int expand_slot = -1;
+                if (cur_expanded + expand_inflight < allowed) {
+                    if (lane == 0) {
+                        const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
+                        if (slot < allowed)
+                            expand_slot = slot;
+                        else
+                            atomicSub(&a.node_expand_inflight[nrow], 1);
+                    }
+                    expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
+                }
+                if (expand_slot >= 0) {
+                    final_packed = pack_selection_v2(PUCT_SELECT_EXPAND, node, expand_slot);
+                    final_len = depth + 1;
+                } else {
+                    rollback_node_path(a, path, tree, depth, lane, node_limit);
+                }
+                break;
+            }
+
+            const float sqrt_parent = sqrtf((float)parent_eff);
+            int best_eid = kNoEdge, held = 0;
+            if (PRECLAIM) {
+                // :448-483: claim every candidate, score it with the count found, keep the winner's claim
+                int tie_offset = wid;
+                if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
+                uint64_t key = 0;
+#pragma unroll
+                for (int i = 0; i < kPasses; ++i) {
+                    if (i * kWave < cur_expanded && valid[i]) {
+                        const int before = atomicAdd(&a.node_inflight[trow + c[i]], 1);
+                        const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], before, sqrt_parent),
+                                                         lane + i * kWave, tie_offset, cur_expanded);
+                        key = k > key ? k : key;
+                    }
+                }
+                const uint64_t best = wave_max(key);
+                if (best != 0) best_eid = (int)(best & 0xFFFFu);
+#pragma unroll
+                for (int i = 0; i < kPasses; ++i)
+                    if (i * kWave < cur_expanded && valid[i] && lane + i * kWave != best_eid)
+                        atomicSub(&a.node_inflight[trow + c[i]], 1);
+                held = best_eid != kNoEdge ? 1 : 0;
+            } else {
+                // :520-560
+                int skip_eid = -1;
+                for (int retry = 0; retry < kRecalcAttempts; ++retry) {
+                    uint64_t key = 0;
+#pragma unroll
+                    for (int i = 0; i < kPasses; ++i) {
+                        const int eid = lane + i * kWave;
+                        if (i * kWave < cur_expanded && valid[i] && eid != skip_eid) {
+                            const int fi = retry == 0 ? f[i] : load_relaxed(a.node_inflight + trow + c[i]);
+                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], fi, sqrt_parent), eid, 0,
+                                                             cur_expanded);   // ties: the smaller edge index (:110-117)
+                            key = k > key ? k : key;
+                        }
+                    }
+                    const uint64_t best = wave_max(key);
+                    best_eid = best != 0 ? (int)(best & 0xFFFFu) : kNoEdge;
+                    if (best_eid == kNoEdge) {
+                        if (skip_eid < 0) break;
+                        best_eid = skip_eid;
+                    }
+                    const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
+                    int claim_child = __builtin_amdgcn_readlane(c[0], best_lane);
+#pragma unroll
+                    for (int i = 1; i < kPasses; ++i)
+                        if (best_pass == i) claim_child = __builtin_amdgcn_readlane(c[i], best_lane);
+                    int got = 0, conflict = 0;
+                    if (lane == 0) claim_counter(&a.node_inflight[trow + claim_child], got, conflict);
+                    held = __builtin_amdgcn_readfirstlane(got);
+                    conflict = __builtin_amdgcn_readfirstlane(conflict);
+                    if (held == 0) break;
+                    if (conflict == 0 || cur_expanded <= 1 || retry + 1 >= kRecalcAttempts) break;
+                    if (lane == 0) atomicSub(&a.node_inflight[trow + claim_child], 1);
+                    skip_eid = best_eid;
+                    held = 0;
+                }
+            }
+            if (held == 0) {   // no edge leads anywhere (or the winner's counter cannot be claimed)
+                rollback_node_path(a, path, tree, depth, lane, node_limit);
+                break;
+            }
+            const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
+            int best_child = __builtin_amdgcn_readlane(c[0], best_lane);
+#pragma unroll
+            for (int i = 1; i < kPasses; ++i)
+                if (best_pass == i) best_child = __builtin_amdgcn_readlane(c[i], best_lane);
+            // (only edges that lead to a node of the tree were candidates, so best_child is one)
+            if (lane == 0) path[depth] = (node << 8) | best_eid;
+            node = best_child;
+            depth += 1;
+        }
+    }
+    if (lane == 0) {
+        a.out_selected_node[out] = final_packed;
+        a.out_path_len[out] = final_len;
     }
 }
 

@@ -10,6 +10,13 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_kernel(const 
     select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
+template <bool PRECLAIM>
+__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void node_select_kernel(const NodeSelectArgs a) {
+    const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (wid >= a.warps) return;
+    node_select_traversal<PRECLAIM>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
+}
+
 template <bool NODE_LEVEL>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_kernel(const BackupArgs a) {
     const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -40,6 +47,45 @@ extern "C" int puct_select_winner_recalc_launch(float cpuct, float c_pw, float a
     launch_shape(trees, warps, grid, block);
     hipLaunchKernelGGL(select_kernel, grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
     return static_cast<int>(hipGetLastError());
+}
+
+namespace {
+template <bool PRECLAIM>
+int launch_node_select(float cpuct, float c_pw, float alpha_pw, const int *edge_child_id, const float *edge_prior,
+                       const float *edge_W, const int *edge_N, int *node_inflight, int *node_expand_inflight,
+                       const int *node_expanded, const int *node_count, int *out_selected_node, int *out_path_eids,
+                       int *out_path_len, int trees, int nodes, int edges, int warps, int path_depth, void *stream) {
+    NodeSelectArgs a{cpuct,         c_pw,         alpha_pw,          edge_child_id, edge_prior,   edge_W, edge_N,
+                     node_inflight, node_expand_inflight, node_expanded, node_count,    out_selected_node,
+                     out_path_eids, out_path_len, trees,             nodes,         edges,        warps,  path_depth};
+    dim3 grid, block;
+    launch_shape(trees, warps, grid, block);
+    hipLaunchKernelGGL(node_select_kernel<PRECLAIM>, grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
+    return static_cast<int>(hipGetLastError());
+}
+}  // namespace
+
+extern "C" int puct_node_select_preclaim_launch(float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                                                const float *edge_prior, const float *edge_W, const int *edge_N,
+                                                int *node_inflight, int *node_expand_inflight, const int *node_expanded,
+                                                const int *node_count, int *out_selected_node, int *out_path_eids,
+                                                int *out_path_len, int trees, int nodes, int edges, int warps,
+                                                int path_depth, void *stream) {
+    return launch_node_select<true>(cpuct, c_pw, alpha_pw, edge_child_id, edge_prior, edge_W, edge_N, node_inflight,
+                                    node_expand_inflight, node_expanded, node_count, out_selected_node, out_path_eids,
+                                    out_path_len, trees, nodes, edges, warps, path_depth, stream);
+}
+
+extern "C" int puct_node_select_winner_recalc_launch(float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                                                     const float *edge_prior, const float *edge_W, const int *edge_N,
+                                                     int *node_inflight, int *node_expand_inflight,
+                                                     const int *node_expanded, const int *node_count,
+                                                     int *out_selected_node, int *out_path_eids, int *out_path_len,
+                                                     int trees, int nodes, int edges, int warps, int path_depth,
+                                                     void *stream) {
+    return launch_node_select<false>(cpuct, c_pw, alpha_pw, edge_child_id, edge_prior, edge_W, edge_N, node_inflight,
+                                     node_expand_inflight, node_expanded, node_count, out_selected_node, out_path_eids,
+                                     out_path_len, trees, nodes, edges, warps, path_depth, stream);
 }
 
 extern "C" const char *puct_cpp_cuda_error_string(int code) { return hipGetErrorString(static_cast<hipError_t>(code)); }

@@ -46,6 +46,9 @@ def _lib():
         lib.puct_cpp_cuda_error_string.restype = ctypes.c_char_p
         lib.puct_edge_backup_launch.argtypes = [c_int] + [c_void] * 9 + [c_int] * 5 + [c_void]
         lib.puct_edge_backup_launch.restype = c_int
+        for fn in (lib.puct_node_select_preclaim_launch, lib.puct_node_select_winner_recalc_launch):
+            fn.argtypes = [c_float] * 3 + [c_void] * 11 + [c_int] * 5 + [c_void]
+            fn.restype = c_int
         lib.puct_node_backup_launch.argtypes = [c_int] + [c_void] * 10 + [c_int] * 5 + [c_void]
         lib.puct_node_backup_launch.restype = c_int
         _LIB = lib
@@ -130,6 +133,32 @@ def launch_select(d, cpuct=1.0, c_pw=1.0, alpha_pw=0.5, soft_winner=0):
         _device_ptr(d["out_selected"], i32, "out_selected"), _device_ptr(d["out_path"], i32, "out_path"),
         _device_ptr(d["out_len"], i32, "out_len"), trees, nodes, edges, warps, path_depth, _stream_handle(d))
     _check(code, "select")
+
+
+VARIANT_PRECLAIM, VARIANT_WINNER_RECALC = "preclaim", "winner_recalc"   # src/puct/test_puct_gpu_v2.py:317-352
+
+
+def launch_node_select(d, cpuct=1.0, c_pw=1.0, alpha_pw=0.5, variant=VARIANT_PRECLAIM):
+    """Asynchronous PUCT selection with node-level virtual loss (d["node_inflight"], int32 [trees, nodes]): the two
+    kernels of src/puct/puct_gpu_v2.py:573-840, chosen by `variant` as in the reference's launch helper
+    (src/puct/test_puct_gpu_v2.py:317-352).  Selection words have the v2 layout (no reason field, no BUSY kind)."""
+    trees, nodes, edges, warps, path_depth = _shape(d)
+    i32, f32 = np.int32, np.float32
+    if variant == VARIANT_PRECLAIM:
+        fn = _lib().puct_node_select_preclaim_launch
+    elif variant == VARIANT_WINNER_RECALC:
+        fn = _lib().puct_node_select_winner_recalc_launch
+    else:
+        raise ValueError(f"unknown select variant: {variant}")
+    code = fn(cpuct, c_pw, alpha_pw,
+              _device_ptr(d["edge_child"], i32, "edge_child"), _device_ptr(d["edge_prior"], f32, "edge_prior"),
+              _device_ptr(d["edge_w"], f32, "edge_w"), _device_ptr(d["edge_n"], i32, "edge_n"),
+              _device_ptr(d["node_inflight"], i32, "node_inflight"),
+              _device_ptr(d["node_expand_inflight"], i32, "node_expand_inflight"),
+              _device_ptr(d["node_expanded"], i32, "node_expanded"), _device_ptr(d["node_count"], i32, "node_count"),
+              _device_ptr(d["out_selected"], i32, "out_selected"), _device_ptr(d["out_path"], i32, "out_path"),
+              _device_ptr(d["out_len"], i32, "out_len"), trees, nodes, edges, warps, path_depth, _stream_handle(d))
+    _check(code, "node select")
 
 
 def launch_edge_backup(d, path_edge_values=None, virtual_loss=1):

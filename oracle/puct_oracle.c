@@ -4,6 +4,7 @@
  *
  * Restates, as plain sequential C over host arrays, the algorithm of
  *   - puct_select_winner_recalc_kernel, src/puct/puct_gpu_v3_cpp.cu:277-448 (helpers :38-275);
+ *   - _select_kernel_native and _select_kernel_winner_recalc, src/puct/puct_gpu_v2.py:573-840 (helpers :109-566);
  *   - _backup_kernel_native, src/puct/puct_gpu_v2.py:847-927;
  *   - _release_claims_kernel, src/puct/test_puct_gpu_v3.py:275-333 (edge-level claim release).
  *
@@ -196,6 +197,155 @@ void po_select(float cpuct, float c_pw, float alpha_pw, int soft_winner, const i
     select_all(cpuct, c_pw, alpha_pw, soft_winner, edge_child_id, edge_prior, edge_W, edge_N, edge_inflight,
                node_expand_inflight, node_expanded, tree_nodes, out_selected_node, out_path_eids, out_path_len, trees,
                nodes, edges, warps, path_depth, NULL);
+}
+
+/* ---------------------------------------------------------------------------------------------------------------------
+ * Selection with node-level virtual loss: _select_kernel_native (preclaim != 0) and _select_kernel_winner_recalc
+ * (preclaim == 0) of src/puct/puct_gpu_v2.py:573-840 with their helpers (:109-566), one traversal after another.
+ * Sequentially, a preclaim that claims every candidate, scores it with the count found and releases the losers comes
+ * to: score every candidate with its child's present count, then claim the winner; the counter compare-and-swap of
+ * the winner-recalc variant never loses, and its conflict bit is "the child already carried claims".
+ * Selection word: (kind << 22) | (slot << 14) | node, PACKED_INVALID = 0x3FFF with length 0 for every failure.
+ * Pins: the known answers of src/puct/test_puct_gpu_v2.py:1006-1166 and hand-computed scores in
+ * tests/test_puct_node_oracle.py.
+ * ------------------------------------------------------------------------------------------------------------------ */
+static void node_rollback(const int *edge_child_id, int *node_inflight, const int *path, int depth, size_t tree_row,
+                          int limit, int edges) {
+    for (int d = 0; d < depth; ++d) {      /* :291-310 */
+        if (path[d] < 0) continue;
+        const int parent = path[d] >> 8, slot = path[d] & 0xFF;
+        if (parent < limit && slot < edges) {
+            const int child = edge_child_id[(tree_row + parent) * edges + slot];
+            if (child >= 0 && child < limit) node_inflight[tree_row + child] -= 1;
+        }
+    }
+}
+
+/* :420-445 / :448-472: the best candidate edge by (score, tie key), skipping `skip`; INT32_MAX when there is none */
+static int node_best_edge(float cpuct, const int *edge_child_id, const float *edge_prior, const float *edge_W,
+                          const int *edge_N, const int *node_inflight, size_t tree_row, size_t erow, int expanded,
+                          int limit, float sqrt_parent, int skip, int tie_offset) {
+    float best_score = -FLT_MAX;
+    int best = INT32_MAX;
+    for (int e = 0; e < expanded; ++e) {
+        const int child = edge_child_id[erow + e];
+        if (e == skip || child < 0 || child >= limit) continue;
+        const int n = edge_N[erow + e];
+        const float q = n > 0 ? edge_W[erow + e] / (float)n : 0.0f;
+        const float u = cpuct * edge_prior[erow + e] * sqrt_parent / (float)(n + node_inflight[tree_row + child] + 1);
+        const float score = q + u;
+        if (ahead(score, e, best_score, best, tie_offset, expanded)) {
+            best_score = score;
+            best = e;
+        }
+    }
+    return best;
+}
+
+static void node_select_one(int preclaim, float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                            const float *edge_prior, const float *edge_W, const int *edge_N, int *node_inflight,
+                            int *node_expand_inflight, const int *node_expanded, int limit, int *out_selected, int *path,
+                            int *out_len, int tree, int wid, int nodes, int edges, int path_depth) {
+    *out_selected = (K_INVALID << KIND_SHIFT) | NODE_MASK;
+    *out_len = 0;
+    if (!(path_depth >= 1 && nodes > 0 && limit > 0 && limit <= nodes && limit <= NODE_LIMIT && edges > 0 &&
+          edges <= EDGE_MASK + 1))
+        return;                                                                   /* :357-366 */
+    const size_t tree_row = (size_t)tree * nodes;
+    int node = 0, depth = 0;
+    for (;;) {
+        if (node < 0 || node >= limit) {
+            node_rollback(edge_child_id, node_inflight, path, depth, tree_row, limit, edges);
+            return;
+        }
+        if (depth >= path_depth) {
+            *out_selected = (K_DEPTH_LIMIT << KIND_SHIFT) | node;
+            *out_len = depth + 1;
+            return;
+        }
+        const size_t nrow = tree_row + node, erow = nrow * edges;
+        const int info = node_expanded[nrow];
+        if (info == TERMINAL) {
+            *out_selected = (K_TERMINAL << KIND_SHIFT) | node;
+            *out_len = depth + 1;
+            return;
+        }
+        if (info < 0 || info > edges) {
+            node_rollback(edge_child_id, node_inflight, path, depth, tree_row, limit, edges);
+            return;
+        }
+        const int expanded = info;
+        int total = 0;                                                            /* :407-416 */
+        for (int e = 0; e < expanded; ++e) {
+            const int child = edge_child_id[erow + e];
+            if (child >= 0 && child < limit) total += edge_N[erow + e] + node_inflight[tree_row + child];
+        }
+        const int parent_eff = total > 1 ? total : 1;
+        const int allowed = (preclaim && expanded == 0) ? 1 : allowed_children(c_pw, alpha_pw, parent_eff, edges);
+        if (allowed > expanded) {                                                 /* :389-403 */
+            const int ticket = node_expand_inflight[nrow]++;
+            if (expanded + ticket < allowed) {
+                *out_selected = (K_EXPAND << KIND_SHIFT) | ((expanded + ticket) << SLOT_SHIFT) | node;
+                *out_len = depth + 1;
+            } else {
+                node_expand_inflight[nrow]--;
+                node_rollback(edge_child_id, node_inflight, path, depth, tree_row, limit, edges);
+            }
+            return;
+        }
+        const float sqrt_parent = sqrtf((float)parent_eff);
+        int best, held = 0;
+        if (preclaim) {
+            int tie_offset = wid;
+            if (tie_offset >= expanded) tie_offset %= expanded;
+            best = node_best_edge(cpuct, edge_child_id, edge_prior, edge_W, edge_N, node_inflight, tree_row, erow, expanded,
+                                  limit, sqrt_parent, -1, tie_offset);
+            if (best != INT32_MAX) {
+                node_inflight[tree_row + edge_child_id[erow + best]] += 1;
+                held = 1;
+            }
+        } else {
+            int skip = -1;
+            best = INT32_MAX;
+            for (int retry = 0; retry < 2; ++retry) {                             /* :520-560, MAX_RECALC_RETRY = 2 */
+                best = node_best_edge(cpuct, edge_child_id, edge_prior, edge_W, edge_N, node_inflight, tree_row, erow,
+                                      expanded, limit, sqrt_parent, skip, 0);
+                if (best == INT32_MAX) {
+                    if (skip < 0) break;
+                    best = skip;
+                }
+                int *counter = &node_inflight[tree_row + edge_child_id[erow + best]];
+                if (*counter < 0 || *counter >= INT32_MAX) break;                 /* :329-331: not claimable */
+                const int conflict = *counter > 0;
+                *counter += 1;
+                held = 1;
+                if (!conflict || expanded <= 1 || retry + 1 >= 2) break;
+                *counter -= 1;
+                skip = best;
+                held = 0;
+            }
+        }
+        if (!held) {
+            node_rollback(edge_child_id, node_inflight, path, depth, tree_row, limit, edges);
+            return;
+        }
+        path[depth] = (node << 8) | best;
+        node = edge_child_id[erow + best];
+        depth += 1;
+    }
+}
+
+void po_node_select(int preclaim, float cpuct, float c_pw, float alpha_pw, const int *edge_child_id,
+                    const float *edge_prior, const float *edge_W, const int *edge_N, int *node_inflight,
+                    int *node_expand_inflight, const int *node_expanded, const int *node_count, int *out_selected_node,
+                    int *out_path_eids, int *out_path_len, int trees, int nodes, int edges, int warps, int path_depth) {
+    for (int tree = 0; tree < trees; ++tree)
+        for (int wid = 0; wid < warps; ++wid) {
+            const size_t out = (size_t)tree * warps + wid;
+            node_select_one(preclaim, cpuct, c_pw, alpha_pw, edge_child_id, edge_prior, edge_W, edge_N, node_inflight,
+                            node_expand_inflight, node_expanded, node_count[tree], out_selected_node + out,
+                            out_path_eids + out * path_depth, out_path_len + out, tree, wid, nodes, edges, path_depth);
+        }
 }
 
 /* node_level != 0: src/puct/puct_gpu_v2.py:847-927 as written.  node_level == 0: the same conversion applied to

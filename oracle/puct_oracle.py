@@ -20,6 +20,8 @@ def lib():
         vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
         L.po_select.restype = None
         L.po_select.argtypes = [cf, cf, cf, ci] + [vp] * 11 + [ci] * 5
+        L.po_node_select.restype = None
+        L.po_node_select.argtypes = [ci, cf, cf, cf] + [vp] * 11 + [ci] * 5
         L.po_backup.restype = None
         L.po_backup.argtypes = [ci, ci] + [vp] * 11 + [ci] * 5
         _lib = L
@@ -44,6 +46,24 @@ def select(h, cpuct=1.0, c_pw=1.0, alpha_pw=0.5, soft_winner=0):
                     _ptr(h["edge_w"]), _ptr(h["edge_n"]), _ptr(h["edge_inflight"]), _ptr(h["node_expand_inflight"]),
                     _ptr(h["node_expanded"]), _ptr(h["node_count"]), _ptr(h["out_selected"]), _ptr(h["out_path"]),
                     _ptr(h["out_len"]), trees, nodes, edges, warps, depth)
+    return h
+
+
+def node_select(h, cpuct=1.0, c_pw=1.0, alpha_pw=0.5, variant="preclaim"):
+    """Selection with node-level virtual loss (h["node_inflight"]), src/puct/puct_gpu_v2.py:573-840, the traversals one
+    after another (tree-major, wid ascending), in place; variant "preclaim" or "winner_recalc"."""
+    trees, nodes, edges = h["edge_child"].shape
+    warps, depth = h["out_path"].shape[1:]
+    for k in ("edge_child", "edge_n", "node_inflight", "node_expand_inflight", "node_expanded", "node_count",
+              "out_selected", "out_path", "out_len"):
+        assert h[k].dtype == np.int32 and h[k].flags.c_contiguous, k
+    for k in ("edge_prior", "edge_w"):
+        assert h[k].dtype == np.float32 and h[k].flags.c_contiguous, k
+    assert variant in ("preclaim", "winner_recalc")
+    lib().po_node_select(int(variant == "preclaim"), cpuct, c_pw, alpha_pw, _ptr(h["edge_child"]), _ptr(h["edge_prior"]),
+                         _ptr(h["edge_w"]), _ptr(h["edge_n"]), _ptr(h["node_inflight"]), _ptr(h["node_expand_inflight"]),
+                         _ptr(h["node_expanded"]), _ptr(h["node_count"]), _ptr(h["out_selected"]), _ptr(h["out_path"]),
+                         _ptr(h["out_len"]), trees, nodes, edges, warps, depth)
     return h
 
 

@@ -130,7 +130,8 @@ def test_puct_library_exports_every_declared_symbol(tmp_path):
     text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
     names = sorted(set(re.findall(r"\b(puct_[a-z_]+)\s*\(", text)))
     assert {"puct_select_winner_recalc_launch", "puct_cpp_cuda_error_string", "puct_edge_backup_launch",
-            "puct_node_backup_launch"} == set(names)
+            "puct_node_backup_launch", "puct_node_select_preclaim_launch",
+            "puct_node_select_winner_recalc_launch"} == set(names)
     for name in names:
         assert hasattr(lib, name), name
     src = tmp_path / "probe.c"
