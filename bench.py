@@ -263,6 +263,86 @@ def bench_puct_select(args):
     print(json.dumps(out))
 
 
+# published by the reference for its node-level select kernels on this benchmark (8 traversals per tree; hardware not
+# stated, its notes mention an RTX 4090): shape -> (preclaim, winner_recalc) selections/s
+PUCT_NODE_PUBLISHED = {"eq256_d1024": (242e3, 376e3), "eq128_d1024": (410e3, 641e3), "eq64_d512": (1.21e6, 1.63e6)}
+
+
+def bench_puct_node_select(args):
+    """The reference's large-scale deep-wide select benchmark on its own two kernels with node-level virtual loss
+    (src/puct/test_puct_gpu_v2.py:1802-1915): one bench step = one selection launch over all trees, timed with HIP events
+    on the launch stream, followed by an untimed node-level backup (path values zero), as the reference times it."""
+    from mcts_numba_cuda_amd import puct
+    from mcts_numba_cuda_amd.hipmem import DeviceArray, Event, synchronize
+    variant = {"node_preclaim": puct.VARIANT_PRECLAIM, "node_winner_recalc": puct.VARIANT_WINNER_RECALC}[args.select_variant]
+    trees, actions, depth = PUCT_SHAPES[args.puct_shape]
+    warps = PUCT_TRAVERSALS
+    steps = args.steps if args.steps != N_ROOTS else 10
+    case = puct_wide_case(trees, actions, depth, warps)
+    del case["edge_inflight"]
+    case["node_inflight"] = np.zeros((trees, actions + 1), np.int32)
+    d = {k: DeviceArray(v) for k, v in case.items()}
+    values = DeviceArray(np.zeros((trees, warps, depth), np.float32))
+    for _ in range(max(args.warmup, 1)):
+        puct.launch_node_select(d, cpuct=1.0, c_pw=0.0, variant=variant)
+        puct.launch_node_backup(d, values)
+    synchronize()
+    pairs = []
+    for _ in range(steps):
+        a, b = Event(), Event()
+        a.record()
+        puct.launch_node_select(d, cpuct=1.0, c_pw=0.0, variant=variant)
+        b.record()
+        sel, lens = d["out_selected"], d["out_len"]
+        puct.launch_node_backup(d, values)
+        pairs.append((a, b))
+    synchronize()
+    ms = sum(a.elapsed_ms(b) for a, b in pairs)
+    kinds = sel.numpy() >> 22
+    lens = lens.numpy()
+    # the reference's criterion (:1876-1880): some valid selections, full-length paths, nothing left in flight
+    ok = bool(np.any(kinds != 0) and lens.max() == depth + 1 and not d["node_inflight"].numpy().any()
+              and not d["node_expand_inflight"].numpy().any())
+    invalid_share = float((kinds == 0).mean())
+    selections = steps * trees * warps
+    # per level: the node word and ticket counter, child / N / W / prior of every edge and the child's counter (a gather);
+    # the preclaim kernel also adds to and takes from every child's counter: two atomic read-modify-writes per edge
+    level_bytes = 8 + (20 + (8 if variant == puct.VARIANT_PRECLAIM else 0)) * actions + 4
+    alg_bytes = trees * warps * depth * level_bytes
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import puct_oracle as po
+        sample = 64
+        h = {k: np.ascontiguousarray(v[:sample]) for k, v in case.items()}
+        t1 = time.perf_counter()
+        po.node_select(h, cpuct=1.0, c_pw=0.0, variant=variant)
+        dt = time.perf_counter() - t1
+        cpu = {"value": sample * warps / dt, "unit": "selections/s", "cores": 1, "kind": "port",
+               "sample": f"first {sample} trees of the same workload, one launch ({sample * warps} selections of {depth} levels), "
+                         "sequential CPU oracle"}
+    launch_s = ms / steps * 1e-3
+    published = PUCT_NODE_PUBLISHED[args.puct_shape][0 if variant == puct.VARIANT_PRECLAIM else 1]
+    value = selections / (ms * 1e-3)
+    out = {"metric": f"PUCT selections/s, deep-wide select benchmark of the reference, its {variant} kernel with node-level virtual loss "
+                     "(8 traversals per tree)",
+           "value": value, "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
+           "ms_per_step": ms / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": value / published,
+           "baseline": {"value": published, "unit": "selections/s", "hardware": "not stated by the reference (its notes mention an RTX 4090)",
+                        "source": "puct_gpu_v2_select_experiments.md:519-528 as quoted in BASELINE.md"},
+           "dtype": "f32 scores + int32 atomics", "data": "synthetic",
+           "config": {"workload": f"{args.puct_shape}: {trees} trees x {warps} traversals, {actions} edges per node, depth {depth}, equal "
+                                  f"priors, c_pw=0, terminal by depth limit; one puct_node_select_{variant}_launch per step"},
+           "valid": ok, "invalid_share_last_launch": invalid_share, "levels_per_s": selections * depth / (ms * 1e-3),
+           # no counter summary exists for these kernels: the entry is the L2-level figure (bytes the traversals request; the
+           # eight traversals of a tree read the same rows), not an HBM fraction
+           "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                        "kernel": f"node_select_kernel<{str(variant == puct.VARIANT_PRECLAIM).lower()}>", "avg_launch_ms": ms / steps,
+                        "l2_level": {"requested_bytes_per_launch": alg_bytes, "requested_GB_per_s": alg_bytes / launch_s / 1e9,
+                                     "note": "bytes requested by the traversals (L2 level); no rocprofv3 counters were taken for this kernel"}},
+           "cpu_baseline": cpu}
+    print(json.dumps(out))
+
+
 def cpu_oracle_baseline(roots):
     """The CPU oracle (scalar restatement of the reference's kernels, OpenMP over playouts) on a bounded sample of the
     headline workload: the first 8 roots, 400 MCTS steps each."""
@@ -651,6 +731,9 @@ def main():
                     help="c4: the headline MCTS-NC search (default); puct_select: the reference's deep-wide PUCT selection "
                          "benchmark through puct_select_winner_recalc_launch; puct_gomoku: the Gomoku PUCT search loop")
     ap.add_argument("--puct-shape", default="eq64_d512", choices=sorted(PUCT_SHAPES))
+    ap.add_argument("--select-variant", default="edge_winner_recalc", choices=("edge_winner_recalc", "node_preclaim", "node_winner_recalc"),
+                    help="puct_select: the C-ABI kernel with edge-level virtual loss (default) or one of the reference's two kernels "
+                         "with node-level virtual loss")
     ap.add_argument("--searches", type=int, default=768, help="c4_many: concurrent searches in the pass")
     args = ap.parse_args()
     global PLAIN_LAUNCH
@@ -676,7 +759,7 @@ def main():
     if args.workload == "c4_many":
         return bench_c4_many(args)
     if args.workload == "puct_select":
-        return bench_puct_select(args)
+        return bench_puct_select(args) if args.select_variant == "edge_winner_recalc" else bench_puct_node_select(args)
     if args.workload == "puct_gomoku":
         return bench_puct_gomoku(args)
 

@@ -361,7 +361,6 @@ struct NodeSelectArgs {
     int trees, nodes, edges, warps, path_depth;
 };
 
-constexpr int kClaimAttempts = 8;   // MAX_SELECT_RETRY, src/puct/puct_gpu_v2.py:33
 constexpr int kPackedInvalidV2 = (PUCT_SELECT_INVALID << PUCT_PACKED_KIND_SHIFT) | PUCT_PACKED_NODE_MASK;
 
 __device__ __forceinline__ int pack_selection_v2(int kind, int node, int slot) {
@@ -383,29 +382,13 @@ __device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, cons
     }
 }
 
-// src/puct/puct_gpu_v2.py:313-349, called by one lane: one more virtual visit on `counter`, taken with compare-and-swap
-// on the value read (a counter, not a lock), after kClaimAttempts lost exchanges with a plain atomic add.
-// conflict = the counter already held visits when this claim went in.
-__device__ __forceinline__ void claim_counter(int *counter, int &held, int &conflict) {
-    held = 0, conflict = 0;
-    bool can_claim = true;
-    for (int attempt = 0; attempt < kClaimAttempts && !held; ++attempt) {
-        const int old = load_relaxed(counter);
-        if (old < 0 || old >= INT32_MAX) {
-            can_claim = false;
-            break;
-        }
-        if (atomicCAS(counter, old, old + 1) == old) {
-            held = 1;
-            conflict = old > 0 ? 1 : 0;
-        }
-    }
-    if (!held && can_claim) {
-        const int old = atomicAdd(counter, 1);
-        held = 1;
-        conflict = old > 0 ? 1 : 0;
-    }
-}
+// The claim of the winner-recalc kernel (src/puct/puct_gpu_v2.py:313-349) is one more virtual visit on the child's
+// counter; "conflict" = the counter already held visits when the claim went in.  The reference moves the counter from the
+// value it read to that value plus one with compare-and-swap, reads again when the exchange is lost, and after
+// MAX_SELECT_RETRY lost exchanges adds one atomically instead: a counter, not a lock, so every claim goes in and all it
+// learns is the value it found.  That is a fetch-and-add, which is what node_select_traversal does, without the lost
+// exchanges (the traversals of a tree that reach a node together all claim the same child, and compare-and-swap then
+// costs a round trip per traversal ahead).
 
 // One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.
 template <bool PRECLAIM>
@@ -526,40 +509,93 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         atomicSub(&a.node_inflight[trow + c[i]], 1);
                 held = best_eid != kNoEdge ? 1 : 0;
             } else {
-                // :520-560
-                int skip_eid = -1;
-                for (int retry = 0; retry < kRecalcAttempts; ++retry) {
+                // :520-560 with MAX_RECALC_RETRY = 2 written out: the best edge by the counters as read; its child is
+                // claimed; if that child already carried claims and the node has other edges, the claim is given back and
+                // the best of the other edges is claimed and kept whatever it carries (none: the first winner again).
+                // The counters for the second evaluation are requested together with the first claim, before it is known
+                // whether they will be needed: the reference reads them after its release, but nothing orders those
+                // loads after its relaxed atomics on other counters, and the first winner's own counter is not among the
+                // ones the second evaluation looks at.
+                auto best_by = [&](const int (&counts)[kPasses], int skip) {
                     uint64_t key = 0;
 #pragma unroll
                     for (int i = 0; i < kPasses; ++i) {
                         const int eid = lane + i * kWave;
-                        if (i * kWave < cur_expanded && valid[i] && eid != skip_eid) {
-                            const int fi = retry == 0 ? f[i] : load_relaxed(a.node_inflight + trow + c[i]);
-                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], fi, sqrt_parent), eid, 0,
+                        if (i * kWave < cur_expanded && valid[i] && eid != skip) {
+                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], counts[i], sqrt_parent), eid, 0,
                                                              cur_expanded);   // ties: the smaller edge index (:110-117)
                             key = k > key ? k : key;
                         }
                     }
                     const uint64_t best = wave_max(key);
-                    best_eid = best != 0 ? (int)(best & 0xFFFFu) : kNoEdge;
-                    if (best_eid == kNoEdge) {
-                        if (skip_eid < 0) break;
-                        best_eid = skip_eid;
-                    }
-                    const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
-                    int claim_child = __builtin_amdgcn_readlane(c[0], best_lane);
+                    return best != 0 ? (int)(best & 0xFFFFu) : kNoEdge;
+                };
+                auto child_of = [&](int eid) {
+                    const int at = eid & (kWave - 1), pass = eid / kWave;
+                    int child = __builtin_amdgcn_readlane(c[0], at);
 #pragma unroll
                     for (int i = 1; i < kPasses; ++i)
-                        if (best_pass == i) claim_child = __builtin_amdgcn_readlane(c[i], best_lane);
-                    int got = 0, conflict = 0;
-                    if (lane == 0) claim_counter(&a.node_inflight[trow + claim_child], got, conflict);
-                    held = __builtin_amdgcn_readfirstlane(got);
-                    conflict = __builtin_amdgcn_readfirstlane(conflict);
-                    if (held == 0) break;
-                    if (conflict == 0 || cur_expanded <= 1 || retry + 1 >= kRecalcAttempts) break;
-                    if (lane == 0) atomicSub(&a.node_inflight[trow + claim_child], 1);
-                    skip_eid = best_eid;
-                    held = 0;
+                        if (pass == i) child = __builtin_amdgcn_readlane(c[i], at);
+                    return child;
+                };
+                // one more visit on `child`'s counter, kept unless the counter was negative or full (:329-331): the value found
+                auto claim = [&](int child, int &found) {
+                    int v = 0;
+                    if (lane == 0) v = atomicAdd(&a.node_inflight[trow + child], 1);
+                    found = __builtin_amdgcn_readfirstlane(v);
+                    if (found < 0 || found >= INT32_MAX) {
+                        if (lane == 0) atomicSub(&a.node_inflight[trow + child], 1);
+                        return 0;
+                    }
+                    return 1;
+                };
+                best_eid = best_by(f, -1);
+                if (best_eid != kNoEdge) {
+                    const int first_child = child_of(best_eid), first_eid = best_eid;
+                    const int seen = [&] {
+                        const int at = first_eid & (kWave - 1), pass = first_eid / kWave;
+                        int v = __builtin_amdgcn_readlane(f[0], at);
+#pragma unroll
+                        for (int i = 1; i < kPasses; ++i)
+                            if (pass == i) v = __builtin_amdgcn_readlane(f[i], at);
+                        return v;
+                    }();
+                    bool second_round = false;
+                    int again[kPasses];
+                    if (seen > 0 && seen < INT32_MAX && cur_expanded > 1) {
+                        // The winner's counter already held visits when it was read.  In the execution in which no other
+                        // traversal acts between that read and this traversal's claim, the claim finds the same value: a
+                        // conflict, upon which the claim is given back and the other edges are evaluated on counters
+                        // that are still the ones read.  That execution is the one taken: nothing is added to the first
+                        // winner's counter and nothing taken back.  (A claim that is added and taken back differs from it
+                        // only in what other traversals may see in passing, and costs two of the three atomics and two of
+                        // the five round trips of a level.)
+                        second_round = true;
+#pragma unroll
+                        for (int i = 0; i < kPasses; ++i) again[i] = f[i];
+                    } else {
+                        int found = 0, v = 0;
+                        if (lane == 0) v = atomicAdd(&a.node_inflight[trow + first_child], 1);
+#pragma unroll
+                        for (int i = 0; i < kPasses; ++i)
+                            again[i] = (cur_expanded > 1 && i * kWave < cur_expanded && valid[i])
+                                           ? load_relaxed(a.node_inflight + trow + c[i]) : 0;
+                        found = __builtin_amdgcn_readfirstlane(v);
+                        if (found < 0 || found >= INT32_MAX) {
+                            if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
+                        } else if (found == 0 || cur_expanded <= 1) {
+                            held = 1;
+                        } else {
+                            if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
+                            second_round = true;
+                        }
+                    }
+                    if (second_round) {
+                        const int second = best_by(again, first_eid);
+                        if (second != kNoEdge) best_eid = second;
+                        int found2;
+                        held = claim(child_of(best_eid), found2);
+                    }
                 }
             }
             if (held == 0) {   // no edge leads anywhere (or the winner's counter cannot be claimed)
