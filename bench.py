@@ -321,6 +321,8 @@ def bench_puct_node_select(args):
                "sample": f"first {sample} trees of the same workload, one launch ({sample * warps} selections of {depth} levels), "
                          "sequential CPU oracle"}
     launch_s = ms / steps * 1e-3
+    prof = profile_json(f"node_select_kernel_{variant}_puct_{args.puct_shape}.md")
+    traffic = (prof or {}).get("traffic_bytes_per_launch")
     published = PUCT_NODE_PUBLISHED[args.puct_shape][0 if variant == puct.VARIANT_PRECLAIM else 1]
     value = selections / (ms * 1e-3)
     out = {"metric": f"PUCT selections/s, deep-wide select benchmark of the reference, its {variant} kernel with node-level virtual loss "
@@ -333,12 +335,15 @@ def bench_puct_node_select(args):
            "config": {"workload": f"{args.puct_shape}: {trees} trees x {warps} traversals, {actions} edges per node, depth {depth}, equal "
                                   f"priors, c_pw=0, terminal by depth limit; one puct_node_select_{variant}_launch per step"},
            "valid": ok, "invalid_share_last_launch": invalid_share, "levels_per_s": selections * depth / (ms * 1e-3),
-           # no counter summary exists for these kernels: the entry is the L2-level figure (bytes the traversals request; the
-           # eight traversals of a tree read the same rows), not an HBM fraction
-           "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+           # HBM bytes per launch from the counter summary of this kernel and shape, where one exists, over this run's launch
+           # time; the bytes the traversals request (the eight traversals of a tree read the same rows) are an L2-level figure
+           "roofline": {"bound": "hbm", "achieved": traffic / launch_s / 1e9 if traffic else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": traffic / launch_s / 1e9 / HBM_PEAK_GBS if traffic else None, "traffic": traffic,
+                        "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
                         "kernel": f"node_select_kernel<{str(variant == puct.VARIANT_PRECLAIM).lower()}>", "avg_launch_ms": ms / steps,
                         "l2_level": {"requested_bytes_per_launch": alg_bytes, "requested_GB_per_s": alg_bytes / launch_s / 1e9,
-                                     "note": "bytes requested by the traversals (L2 level); no rocprofv3 counters were taken for this kernel"}},
+                                     "note": "node word, ticket counter, child / N / W / prior of every edge and the child's counter "
+                                             "per level and traversal; the preclaim kernel adds two atomic updates per edge"}},
            "cpu_baseline": cpu}
     print(json.dumps(out))
 

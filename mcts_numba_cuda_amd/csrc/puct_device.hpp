@@ -561,7 +561,6 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         return v;
                     }();
                     bool second_round = false;
-                    int again[kPasses];
                     if (seen > 0 && seen < INT32_MAX && cur_expanded > 1) {
                         // The winner's counter already held visits when it was read.  In the execution in which no other
                         // traversal acts between that read and this traversal's claim, the claim finds the same value: a
@@ -571,15 +570,12 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         // only in what other traversals may see in passing, and costs two of the three atomics and two of
                         // the five round trips of a level.)
                         second_round = true;
-#pragma unroll
-                        for (int i = 0; i < kPasses; ++i) again[i] = f[i];
                     } else {
                         int found = 0, v = 0;
                         if (lane == 0) v = atomicAdd(&a.node_inflight[trow + first_child], 1);
 #pragma unroll
-                        for (int i = 0; i < kPasses; ++i)
-                            again[i] = (cur_expanded > 1 && i * kWave < cur_expanded && valid[i])
-                                           ? load_relaxed(a.node_inflight + trow + c[i]) : 0;
+                        for (int i = 0; i < kPasses; ++i)   // (the counters as first read are not needed any more)
+                            if (cur_expanded > 1 && i * kWave < cur_expanded && valid[i]) f[i] = load_relaxed(a.node_inflight + trow + c[i]);
                         found = __builtin_amdgcn_readfirstlane(v);
                         if (found < 0 || found >= INT32_MAX) {
                             if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
@@ -591,7 +587,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         }
                     }
                     if (second_round) {
-                        const int second = best_by(again, first_eid);
+                        const int second = best_by(f, first_eid);
                         if (second != kNoEdge) best_eid = second;
                         int found2;
                         held = claim(child_of(best_eid), found2);
