@@ -516,17 +516,20 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                 // whether they will be needed: the reference reads them after its release, but nothing orders those
                 // loads after its relaxed atomics on other counters, and the first winner's own counter is not among the
                 // ones the second evaluation looks at.
-                auto best_by = [&](const int (&counts)[kPasses], int skip) {
+                // every candidate's place in the order "higher score first, then the smaller edge index" (:110-117), 0 = none
+                uint64_t keys[kPasses];
+                auto score_edges = [&] {
+#pragma unroll
+                    for (int i = 0; i < kPasses; ++i)
+                        keys[i] = (i * kWave < cur_expanded && valid[i])
+                                      ? candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], f[i], sqrt_parent), lane + i * kWave, 0, cur_expanded)
+                                      : 0;
+                };
+                auto best_without = [&](int skip) {
                     uint64_t key = 0;
 #pragma unroll
-                    for (int i = 0; i < kPasses; ++i) {
-                        const int eid = lane + i * kWave;
-                        if (i * kWave < cur_expanded && valid[i] && eid != skip) {
-                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], counts[i], sqrt_parent), eid, 0,
-                                                             cur_expanded);   // ties: the smaller edge index (:110-117)
-                            key = k > key ? k : key;
-                        }
-                    }
+                    for (int i = 0; i < kPasses; ++i)
+                        if (lane + i * kWave != skip) key = keys[i] > key ? keys[i] : key;
                     const uint64_t best = wave_max(key);
                     return best != 0 ? (int)(best & 0xFFFFu) : kNoEdge;
                 };
@@ -549,7 +552,8 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                     }
                     return 1;
                 };
-                best_eid = best_by(f, -1);
+                score_edges();
+                best_eid = best_without(-1);
                 if (best_eid != kNoEdge) {
                     const int first_child = child_of(best_eid), first_eid = best_eid;
                     const int seen = [&] {
@@ -565,10 +569,10 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         // The winner's counter already held visits when it was read.  In the execution in which no other
                         // traversal acts between that read and this traversal's claim, the claim finds the same value: a
                         // conflict, upon which the claim is given back and the other edges are evaluated on counters
-                        // that are still the ones read.  That execution is the one taken: nothing is added to the first
-                        // winner's counter and nothing taken back.  (A claim that is added and taken back differs from it
-                        // only in what other traversals may see in passing, and costs two of the three atomics and two of
-                        // the five round trips of a level.)
+                        // that are still the ones read (so the scores stand).  That execution is the one taken: nothing is
+                        // added to the first winner's counter and nothing taken back.  (A claim that is added and taken back
+                        // differs from it only in what other traversals may see in passing, and costs two of the three
+                        // atomics and two of the five round trips of a level.)
                         second_round = true;
                     } else {
                         int found = 0, v = 0;
@@ -584,10 +588,11 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         } else {
                             if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
                             second_round = true;
+                            score_edges();   // on the counters read again
                         }
                     }
                     if (second_round) {
-                        const int second = best_by(f, first_eid);
+                        const int second = best_without(first_eid);
                         if (second != kNoEdge) best_eid = second;
                         int found2;
                         held = claim(child_of(best_eid), found2);
