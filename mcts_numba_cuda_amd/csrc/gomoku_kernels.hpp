@@ -23,16 +23,17 @@ namespace mctsnc {
 namespace gomoku {
 
 // Two board formats.  Up to 16 x 16 cells: 8 words per colour, a legal-list entry is a byte (row << 4 | column), a line
-// word holds both colours (low half +1, high half -1) and two lines are tested at a time.  Beyond that, up to 384 cells
-// with sides up to 24 (19 x 19, 17 x 20 ...): 12 words per colour, 16-bit list entries (row << 5 | column), one line word
-// per colour.  W, the words per colour, is a template parameter of the kernels: the narrow format compiles to what it was
-// before the wide one existed.
-constexpr int kMaxWords = 12;
-constexpr int kMaxCells = 32 * kMaxWords;   // 384
-constexpr int kMaxSide = 24;
+// word holds both colours (low half +1, high half -1) and two lines are tested at a time.  Beyond that, up to the
+// reference's own caps of 512 actions and sides of 32 (19 x 19, 17 x 20, 22 x 22, 32 x 16 ...): 16-bit list entries
+// (row << 5 | column), one line word per colour, and 12 words per colour (up to 384 cells, which still fit the 128-byte
+// node record) or 16 (a 256-byte record).  W, the words per colour, is a template parameter of the kernels: the narrow
+// format compiles to what it was before the wide ones existed.
+constexpr int kMaxWords = 16;
+constexpr int kMaxCells = 32 * kMaxWords;   // 512: MAX_STATE_MAX_ACTIONS of the reference (src/mctsnc.py:193)
+constexpr int kMaxSide = 32;                // MAX_STATE_BOARD_SHAPE (src/mctsnc.py:191)
 constexpr int kMaxPath = kMaxCells + 2;     // a tree can be m * n + 1 levels deep
 constexpr int kMaxLines = 96;     // narrow boards: 3 * (m + n) - 2 <= 94
-constexpr int kMaxLinesWide = 3 * 2 * kMaxSide - 2;   // 142
+constexpr int kMaxLinesWide = 142;   // 3 * (m + n) - 2 with m * n <= 512 and m, n <= 32: at most 3 * (32 + 16) - 2
 template <int W> struct Board {
     static constexpr bool kWide = W > 8;
     static constexpr int kCells = 32 * W;
@@ -47,7 +48,11 @@ constexpr uint8_t kLeaf = 1, kTerminal = 2;
 constexpr int kModeExpand = 0, kModeTerminal = 1, kModeFull = 2;
 constexpr uint32_t kSpinLimit = 1u << 24;
 
-struct __attribute__((aligned(128))) Node {
+// (bytes of a node record: 128 while the two stone sets fit beside the 32-byte head, 256 beyond)
+constexpr int node_bytes(int words) { return words > 12 ? 256 : 128; }
+
+template <int W>
+struct __attribute__((aligned(128))) NodeT {
     int32_t child_base;      // index of the first child, -1 for a leaf
     int32_t parent;
     int32_t n_children;
@@ -59,9 +64,10 @@ struct __attribute__((aligned(128))) Node {
     uint8_t pad0;
     int16_t action;          // action that led here
     int32_t pad1[2];
-    uint32_t bb[24];         // W words of the stones of player +1, then W words of those of player -1 (W = 8 or 12), rest unused
+    uint32_t bb[node_bytes(W) / 4 - 8];   // W words of the stones of player +1, then W words of those of player -1, rest unused
 };
-static_assert(sizeof(Node) == 128, "node record must be 128 bytes");
+using Node = NodeT<8>;       // the head of every record, whatever its format
+static_assert(sizeof(NodeT<8>) == 128 && sizeof(NodeT<12>) == 128 && sizeof(NodeT<16>) == 256, "node records are whole 128-byte lines");
 
 struct Stat { int32_t ns, wins, action, pad; };
 
@@ -91,7 +97,7 @@ struct __attribute__((aligned(128))) TreeHdr {
 };
 
 struct TreeRef {
-    Node *nodes;
+    Node *nodes;             // records of node_bytes(words) bytes each
     Stat *stats;
     TreeHdr *hdr;
     uint64_t *rng_playout;   // ACP [A][P][2], OCP [P][2]
@@ -225,6 +231,7 @@ struct Gomoku {
     static __device__ __forceinline__ uint32_t winning_starts(uint32_t packed) { return exact_five_starts(packed); }
     static __device__ __forceinline__ uint32_t winning_starts_wide(uint32_t word) { return exact_five_starts_wide(word); }
     static __device__ __forceinline__ uint32_t reach(uint32_t p) { return (0x1fu << p) >> 4; }   // starts of a run of five through position p
+    static __device__ __forceinline__ uint32_t reach_wide(uint32_t p) { return (uint32_t)((0x1full << p) >> 4); }   // (p up to 31)
     static __device__ __forceinline__ int exact_outcome(ExactScratch &s, int m, int n, int turn, int last_action) {
         return gomoku::exact_outcome(s, m, n, turn, last_action);
     }
@@ -243,8 +250,10 @@ __global__ void reset_kernel(const TreeRef *refs, int n_refs, const uint32_t *ro
     Node nd;
     nd.child_base = -1; nd.parent = -1; nd.n_children = 0; nd.best_child = -1; nd.depth = 0; nd.turn = (int8_t)root_turns[r];
     nd.outcome = 2; nd.flags = kLeaf; nd.pad0 = 0; nd.action = 0; nd.pad1[0] = nd.pad1[1] = 0;
-    for (int i = 0; i < 24; i++) nd.bb[i] = i < 2 * ref.words ? root_bb[2 * ref.words * r + i] : 0u;
+    for (int i = 0; i < 24; i++) nd.bb[i] = 0u;
     ref.nodes[0] = nd;
+    uint32_t *const stones = reinterpret_cast<uint32_t *>(ref.nodes) + 8;   // (a record's stone sets follow its 32-byte head)
+    for (int i = 0; i < 2 * ref.words; i++) stones[i] = root_bb[2 * ref.words * r + i];
     Stat st; st.ns = 0; st.wins = 0; st.action = 0; st.pad = 0;
     ref.stats[0] = st;
     TreeHdr *h = ref.hdr;
@@ -289,7 +298,8 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
     const int r = ACP ? b / G : b, g = ACP ? b - r * G : 0;
     if (r >= args.n_refs) return;
     const TreeRef ref = args.refs[r];
-    Node *const nodes = ref.nodes;
+    using NodeW = NodeT<W>;
+    NodeW *const nodes = reinterpret_cast<NodeW *>(ref.nodes);
     Stat *const stats = ref.stats;
     TreeHdr *const hdr = ref.hdr;
     const int nthreads = blockDim.x, nwaves = (nthreads + 63) >> 6, lane = threadIdx.x & 63;
@@ -368,7 +378,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
             int node = 0, depth = 0;
             uint32_t w, meta;
             for (;;) {
-                w = reinterpret_cast<const uint32_t *>(nodes + node)[lane & 31];
+                w = reinterpret_cast<const uint32_t *>(nodes + node)[lane & (int)(sizeof(NodeW) / 4 - 1)];
                 meta = (uint32_t)__builtin_amdgcn_readlane((int)w, 5);   // flags | pad << 8 | action << 16
                 if (lane == 0) s_path[depth] = node;
                 if (meta & kLeaf) break;
@@ -444,7 +454,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                 const uint32_t w_row = s_lleaf[2 * ai + side] | (1u << aj), w_col = s_lleaf[2 * ((uint32_t)m + aj) + side] | (1u << ai);
                 const uint32_t w_dia = s_lleaf[2 * ((uint32_t)(m + n + n - 1) + ai - aj) + side] | (1u << aj);
                 const uint32_t w_ant = s_lleaf[2 * ((uint32_t)(m + n + m + n - 1) + ai + aj) + side] | (1u << aj);
-                const uint32_t win_j = Game::reach(aj), win_i = Game::reach(ai);
+                const uint32_t win_j = Game::reach_wide(aj), win_i = Game::reach_wide(ai);
                 const uint32_t hit = ((Game::winning_starts_wide(w_row) | Game::winning_starts_wide(w_dia) | Game::winning_starts_wide(w_ant)) & win_j) |
                                      (Game::winning_starts_wide(w_col) & win_i);
                 return hit != 0 ? mover : (empties == 1 ? 0 : 2);
@@ -645,7 +655,7 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                                 uint32_t *const p_ant = line_word((uint32_t)(m + n + m + n - 1) + i + jj);
                                 const uint32_t w_row = *p_row | (1u << jj), w_col = *p_col | (1u << i), w_dia = *p_dia | (1u << jj), w_ant = *p_ant | (1u << jj);
                                 *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
-                                const uint32_t win_j = Game::reach(jj), win_i = Game::reach(i);
+                                const uint32_t win_j = Game::reach_wide(jj), win_i = Game::reach_wide(i);
                                 const uint32_t hit = ((Game::winning_starts_wide(w_row) | Game::winning_starts_wide(w_dia) | Game::winning_starts_wide(w_ant)) & win_j) |
                                                      (Game::winning_starts_wide(w_col) & win_i);
                                 if (hit != 0) { status = 1; outcome = outcome_if_win; }
@@ -984,8 +994,7 @@ struct RootView {
         base = root->child_base; kids = (root->flags & kLeaf) ? 0 : root->n_children;
     }
     static __device__ __forceinline__ int action_slot(const Ref &r, int a) {
-        const Node *root = r.nodes;
-        const uint32_t *pos = root->bb, *neg = root->bb + r.words;
+        const uint32_t *pos = reinterpret_cast<const uint32_t *>(r.nodes) + 8, *neg = pos + r.words;
         if (bb_test(pos, a) || bb_test(neg, a)) return -1;
         int rank = __popc(~(pos[a >> 5] | neg[a >> 5]) & ((1u << (a & 31)) - 1u));
         for (int w = 0; w < (a >> 5); w++) rank += 32 - __popc(pos[w] | neg[w]);
@@ -997,7 +1006,7 @@ struct RootView {
         ns = st.ns; wins = st.wins;
     }
     static __device__ __forceinline__ void child_state(const Ref &r, int32_t base, int32_t, int slot, int, bool &terminal, int &outcome) {
-        const Node *c = r.nodes + base + slot;
+        const Node *c = reinterpret_cast<const Node *>(reinterpret_cast<const unsigned char *>(r.nodes) + (size_t)(base + slot) * node_bytes(r.words));
         terminal = (c->flags & kTerminal) != 0; outcome = c->outcome;
     }
 };

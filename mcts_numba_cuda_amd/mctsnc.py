@@ -181,8 +181,8 @@ class MCTSNC:
         the configured board exceeds, or None."""
         m, n = int(self.state_board_shape[0]), int(self.state_board_shape[1])
         if self.game == "gomoku":
-            if m > 24 or n > 24 or m * n > 384:
-                return "placement games are held on boards with sides up to 24 and up to 384 cells (384 actions)"
+            if m > 32 or n > 32 or m * n > 512:     # (the reference's own caps; it reports them itself before this is reached)
+                return "placement games are held on boards with sides up to 32 and up to 512 cells"
         elif (m + 1) * n > 64 or n > 8 or m > 13:
             return "drop games are held in 64-bit column bitboards: (rows + 1) * columns <= 64, columns <= 8, rows <= 13"
         return None

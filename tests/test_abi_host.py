@@ -150,12 +150,12 @@ def test_bench_refuses_more_than_one_gpu():
 
 
 def test_board_shapes_beyond_the_engine_get_a_reference_style_message(capsys):
-    """The reference's caps (32 x 32 cells, 512 actions, src/mctsnc.py:180-197) admit boards this engine's kernels do
-    not take; the class says so in the reference's message style before it raises, without touching the device."""
+    """The reference's caps (32 x 32 cells, 512 actions, src/mctsnc.py:180-197) admit drop-game boards this engine's
+    bitboard kernels do not take (placement games are taken up to those caps); the class says so in the reference's
+    message style before it raises, without touching the device."""
     from mcts_numba_cuda_amd import MCTSNC
-    for kw, part in ((dict(state_board_shape=(20, 24), state_extra_info_memory=0, state_max_actions=480, game="gomoku"), "384 cells"),
-                     (dict(state_board_shape=(5, 25), state_extra_info_memory=0, state_max_actions=125, game="gomoku"), "sides up to 24"),
-                     (dict(state_board_shape=(6, 10), state_extra_info_memory=10, state_max_actions=10), "columns <= 8")):
+    for kw, part in ((dict(state_board_shape=(6, 10), state_extra_info_memory=10, state_max_actions=10), "columns <= 8"),
+                     (dict(state_board_shape=(14, 4), state_extra_info_memory=4, state_max_actions=4), "rows <= 13")):
         e = MCTSNC(verbose_info=False, **kw)
         with pytest.raises(ValueError):
             e.init_device_side_arrays()

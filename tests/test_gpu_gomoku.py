@@ -125,6 +125,34 @@ def test_gomoku_boards_beyond_sixteen(variant, steps):
             compare_with_oracle(e, o, board, None, turn, max(2, int(steps * scale)))
 
 
+@pytest.mark.parametrize("variant,steps", [("ocp_thrifty", 30), ("ocp_prodigal", 30), ("acp_thrifty", 2), ("acp_prodigal", 2)])
+def test_gomoku_boards_up_to_the_references_caps(variant, steps):
+    """Boards of more than 384 cells need 16 words per colour and a 256-byte node record: 22 x 22, the two extreme shapes
+    of the reference's caps (512 actions, sides of 32: src/mctsnc.py:191-193), 20 x 25, and 32 x 5 (a line of 32 cells in a
+    32-bit line word; the format is chosen by the cell count, so this one runs in the 12-word format)."""
+    rng = np.random.default_rng(32)
+    for (m, n), scale in (((22, 22), 1.0), ((32, 16), 1.0), ((16, 32), 1.0), ((20, 25), 0.5), ((32, 5), 3.0), ((5, 32), 3.0)):
+        e, o = engines(variant, 2, 64, m, n, seed=11)
+        for stones in (0, 14):
+            board, turn = random_gomoku_root(rng, m, n, stones)
+            compare_with_oracle(e, o, board, None, turn, max(2, int(steps * scale)))
+
+
+def test_gomoku_fives_at_the_far_end_of_32_cell_lines():
+    """32 x 16: runs of five that end on the last cell of a 32-cell column (bit 31 of a line word), a six there, and a row
+    of five on the last row."""
+    board = np.zeros((32, 16), np.int8)
+    board[27:31, 3] = 1                                 # column 3, rows 27..30: (31,3) and (26,3) win
+    board[26:31, 9] = 1; board[25, 9] = -1              # five already there is not checked; (31,9) would make six: no win
+    board[31, 10:14] = 1                                # last row: (31,9)? occupied later; (31,14) wins, (31,9) makes a row five too
+    for k in range(4):
+        board[27 + k, 12 - k] = -1                      # anti-diagonal of -1 towards the last row
+    board[[0, 2, 9, 14, 20], [0, 7, 2, 9, 10]] = -1
+    for variant, steps in (("acp_prodigal", 3), ("ocp_thrifty", 100)):
+        e, o = engines(variant, 2, 64, 32, 16, seed=9)
+        compare_with_oracle(e, o, board, None, 1, steps)
+
+
 def test_gomoku_wide_board_children_that_complete_lines():
     """19 x 19: cells that complete exactly five in the part of the board the 16-wide format does not reach (columns and
     rows 16 to 18, the diagonals that end there), a cell that would make six, and a row of five that ends on the last
