@@ -114,7 +114,7 @@ def test_gomoku_sixteen_wide_boards(variant):
 @pytest.mark.parametrize("variant,steps", [("ocp_thrifty", 40), ("ocp_prodigal", 40), ("acp_thrifty", 3), ("acp_prodigal", 3)])
 def test_gomoku_boards_beyond_sixteen(variant, steps):
     """Boards with a side beyond 16 are held in the engine's second format (12 words per colour, 16-bit list entries,
-    one line word per colour): 19 x 19, a rectangle, the 384 cells the format holds at most, and boards one line of
+    one line word per colour): 19 x 19, a rectangle, the 384 cells that still fit the 128-byte record, and boards one line of
     which is 24 long while the other side is short (deep trees, wins, draws).  Two consecutive searches each, every
     array against the oracle; more than 256 children per node exercise the arg-max tie rule on nine bits."""
     rng = np.random.default_rng(19)
