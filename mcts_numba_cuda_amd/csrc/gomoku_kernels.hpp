@@ -632,34 +632,52 @@ __global__ void __launch_bounds__(kMaxThreads) search_kernel_for(SearchArgs args
                         // pipelined: while cell k is judged, cell k + 1 is already drawn.  When ply k ends the game, the
                         // generator goes back to its state after draw k; what draw k + 1 did to the list no longer matters.
                         if constexpr (WIDE) {
-                            // Wide boards: 16-bit list entries, one word per line and colour; one ply after the other,
-                            // without the narrow format's pipelining and packing (same draws, same order, same rule).
+                            // Wide boards: 16-bit list entries, one word per line and colour, four tests on single words;
+                            // the same draws in the same order by the same rule, pipelined as below.
                             uint16_t *const lw = reinterpret_cast<uint16_t *>(s_list + tid);   // entry i: lw[(i >> 1) * stride2 + (i & 1)]
                             const uint32_t stride2 = nt << 1;
-                            uint32_t side = pturn == 1 ? 0u : 1u;
-                            while (status == 0) {
+                            uint32_t side = pturn == 1 ? 0u : 1u, a = 0;
+                            if (status == 0) {
                                 uint32_t xl, xh;
-                                const Rng32 rg_before = rg;
                                 rng_next32(rg, xl, xh);
                                 const int ord = (int)(uniform_from_bits(xl, xh) * (float)count);
-                                if (ord >= count) { status = 3; rg = rg_before; break; }
-                                count--;
-                                uint16_t *const slot = lw + __umul24((uint32_t)ord >> 1, stride2) + (ord & 1);
-                                const uint32_t cell = *slot;
-                                *slot = lw[__umul24((uint32_t)count >> 1, stride2) + (count & 1)];
+                                if (ord >= count) status = 3;
+                                else {
+                                    count--;
+                                    uint16_t *const slot = lw + __umul24((uint32_t)ord >> 1, stride2) + (ord & 1);
+                                    a = *slot;
+                                    *slot = lw[__umul24((uint32_t)count >> 1, stride2) + (count & 1)];
+                                }
+                            }
+                            while (status == 0) {
                                 plies++;
-                                const uint32_t i = cell >> 5, jj = cell & 31u;
+                                const uint32_t i = a >> 5, jj = a & 31u;
                                 auto line_word = [&](uint32_t line) { return reinterpret_cast<uint32_t *>(reinterpret_cast<unsigned char *>(lp) + ((2u * line + side) << line_shift)); };
                                 uint32_t *const p_row = line_word(i), *const p_col = line_word((uint32_t)m + jj);
                                 uint32_t *const p_dia = line_word((uint32_t)(m + n + n - 1) + i - jj);
                                 uint32_t *const p_ant = line_word((uint32_t)(m + n + m + n - 1) + i + jj);
-                                const uint32_t w_row = *p_row | (1u << jj), w_col = *p_col | (1u << i), w_dia = *p_dia | (1u << jj), w_ant = *p_ant | (1u << jj);
+                                uint32_t w_row = *p_row, w_col = *p_col, w_dia = *p_dia, w_ant = *p_ant;
+                                __builtin_amdgcn_sched_barrier(0);   // the line reads are in flight while the next cell is drawn
+                                const Rng32 rg_now = rg;
+                                uint32_t xl, xh;
+                                rng_next32(rg, xl, xh);
+                                const int ord_n = (int)(uniform_from_bits(xl, xh) * (float)count);
+                                const bool stale_n = ord_n >= count;
+                                const int count_n = count > 0 ? count - 1 : 0;
+                                uint16_t *const slot_n = lw + __umul24((uint32_t)ord_n >> 1, stride2) + (ord_n & 1);
+                                const uint32_t a_n = *slot_n;
+                                const uint16_t last_n = lw[__umul24((uint32_t)count_n >> 1, stride2) + (count_n & 1)];
+                                w_row |= 1u << jj; w_col |= 1u << i; w_dia |= 1u << jj; w_ant |= 1u << jj;
                                 *p_row = w_row; *p_col = w_col; *p_dia = w_dia; *p_ant = w_ant;
                                 const uint32_t win_j = Game::reach_wide(jj), win_i = Game::reach_wide(i);
                                 const uint32_t hit = ((Game::winning_starts_wide(w_row) | Game::winning_starts_wide(w_dia) | Game::winning_starts_wide(w_ant)) & win_j) |
                                                      (Game::winning_starts_wide(w_col) & win_i);
-                                if (hit != 0) { status = 1; outcome = outcome_if_win; }
-                                else if (count == 0) { status = 2; outcome = 0; }
+                                __builtin_amdgcn_sched_barrier(0);
+                                *slot_n = last_n;   // swap-remove of the next draw
+                                if (hit != 0) { status = 1; outcome = outcome_if_win; rg = rg_now; }
+                                else if (count == 0) { status = 2; outcome = 0; rg = rg_now; }
+                                else if (stale_n) status = 3;
+                                count = count_n; a = a_n;
                                 outcome_if_win = -outcome_if_win;
                                 side ^= 1u;
                             }
