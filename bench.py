@@ -330,7 +330,7 @@ def bench_puct_node_select(args):
            "value": value, "unit": "selections/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 1),
            "ms_per_step": ms / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": value / published,
            "baseline": {"value": published, "unit": "selections/s", "hardware": "not stated by the reference (its notes mention an RTX 4090)",
-                        "source": "puct_gpu_v2_select_experiments.md:519-528 as quoted in BASELINE.md"},
+                        "source": "the reference's puct_gpu_v2_select_experiments.md:519-528"},
            "dtype": "f32 scores + int32 atomics", "data": "synthetic",
            "config": {"workload": f"{args.puct_shape}: {trees} trees x {warps} traversals, {actions} edges per node, depth {depth}, equal "
                                   f"priors, c_pw=0, terminal by depth limit; one puct_node_select_{variant}_launch per step"},
