@@ -441,10 +441,55 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
     int tickets = ni.tickets;
     const int legal = ni.legal_turn & 0xFFFF, n_members = __popcll(members);
 
+    // Every one of these traversals takes the same edge: all of them at once, a traversal per lane.
+    auto take_all = [&](uint32_t link, int eid) {
+        const int child = (int)(link >> 8);
+        const bool leads_somewhere = child > 0 && child < g.max_nodes;
+        if (lane < kTrav && ((members >> lane) & 1ull)) {
+            if (leads_somewhere) {
+                paths[lane * g.path_depth + depth] = (node << 8) | eid;
+                next[lane] = child;
+            } else {
+                s.sel[lane] = pack_sel(PUCT_SELECT_INVALID, PUCT_GOMOKU_SEL_NODE_MASK, 0);
+                s.len[lane] = 0;
+                s.claims[lane] = depth;
+                next[lane] = -1;
+            }
+        }
+        if (leads_somewhere && lane == 0) row[eid].link = link + (uint32_t)n_members;
+    };
+    // No expansion ticket is to be had here however many of these traversals have claimed: the widening limit grows with
+    // the claims, and its largest value, the one the last of them sees, does not exceed the children there are.
+    const auto no_ticket_for_anyone = [&] {
+        if (expanded < 1) return false;
+        if (expanded == 1 && g.c_pw == 0.0f) return true;
+        const int eff_last = total + n_members - 1 > 1 ? total + n_members - 1 : 1;
+        return allowed_children(g.c_pw, g.alpha_pw, eff_last, sqrtf((float)eff_last), legal) <= expanded;
+    };
+
     if (expanded <= kWave) {
-        EdgeSet<1> one{{all.q[0]}, {all.cp[0]}, {all.den[0]}, {all.link[0]}, {all.link_loaded[0]}, {all.eid[0]}};
-        decide_in_turn<1>(g, s, paths, next, one, node, members, depth, lane, expanded, legal, total, tickets);
-        if (one.link[0] != one.link_loaded[0]) row[lane].link = one.link[0];
+        bool taken = false;
+        if (n_members >= 3 && no_ticket_for_anyone()) {
+            // one edge per lane: which of them can come first for any of these traversals (the bounds of the wide case below)
+            uint64_t in = 1ull;   // (a node's only edge is taken whatever its score)
+            if (expanded > 1) {
+                const int now = total > 1 ? total : 1, then = total + n_members > 1 ? total + n_members : 1;
+                const uint32_t l = all.eid[0] >= 0 ? score_image(edge_score(all, 0, sqrtf((float)now), n_members)) : 0u;
+                const uint32_t h = all.eid[0] >= 0 ? score_image(edge_score(all, 0, sqrtf((float)then), 0)) : 0u;
+                const uint32_t low = wave_max_u32(l);
+                in = __ballot(low != 0 && h >= low && h != 0);
+            }
+            if (__popcll(in) == 1) {
+                const int at = __builtin_ctzll(in);
+                take_all((uint32_t)__builtin_amdgcn_readlane((int)all.link[0], at), at);
+                taken = true;
+            }
+        }
+        if (!taken) {
+            EdgeSet<1> one{{all.q[0]}, {all.cp[0]}, {all.den[0]}, {all.link[0]}, {all.link_loaded[0]}, {all.eid[0]}};
+            decide_in_turn<1>(g, s, paths, next, one, node, members, depth, lane, expanded, legal, total, tickets);
+            if (one.link[0] != one.link_loaded[0]) row[lane].link = one.link[0];
+        }
     } else {
         // A wide node with several traversals on it: most edges cannot come first for any of them.  While these
         // traversals decide, sqrt(parent) only grows (by their own claims) and an edge's claims only grow, and every
@@ -465,14 +510,26 @@ __device__ void select_group(const LoopArgs &g, StepLds &s, int *paths, int *nex
             }
             low = wave_max_u32(low);
             int kept = 0, place[kSlices];
+            uint64_t in_slice[kSlices];
 #pragma unroll
             for (int i = 0; i < kSlices; ++i) {
                 const bool in = low != 0 && high[i] >= low && high[i] != 0;
                 const uint64_t mask = __ballot(in);
+                in_slice[i] = mask;
                 place[i] = in ? kept + __popcll(mask & lanes_below(lane)) : -1;
                 kept += __popcll(mask);
             }
-            if (kept >= 1 && kept <= kWave && low != 0) {
+            // One edge left and no expansion ticket to be had: every one of these traversals takes that edge.
+            if (kept == 1 && low != 0 && no_ticket_for_anyone()) {
+                pruned = true;
+#pragma unroll
+                for (int i = 0; i < kSlices; ++i)
+                    if (in_slice[i] != 0) {
+                        const int at = __builtin_ctzll(in_slice[i]);
+                        take_all((uint32_t)__builtin_amdgcn_readlane((int)all.link[i], at), at + i * kWave);
+                    }
+            }
+            if (!pruned && kept >= 1 && kept <= kWave && low != 0) {
                 pruned = true;
                 // through LDS into one edge per lane
                 EdgeSet<1> few{{0.0f}, {0.0f}, {1}, {0u}, {0u}, {-1}};
