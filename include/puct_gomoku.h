@@ -72,6 +72,9 @@ typedef struct {
                                   compute units while the tree's own workgroup backs the step up (fused search only; fewer
                                   are used when the device cannot keep trees * (1 + evaluators) workgroups resident);
                                   0 = the tree's workgroup does it itself.  The trees are the same either way. */
+    int32_t agent_fences;      /* 0: a tree and its evaluators hand over through the L2 they share when they find themselves
+                                  on one XCD (they report where they run, and write the L2 back until all have), 1: they always
+                                  write the L2 back, as they must on different XCDs.  Same trees either way; 1 is slower. */
 } puct_gomoku_config;
 
 typedef struct {

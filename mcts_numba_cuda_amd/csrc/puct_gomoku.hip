@@ -58,6 +58,7 @@ struct LoopArgs {
     float dirichlet_alpha;
     struct EvalRequests *requests;   // [trees]
     int evaluators;                  // workgroups per tree that work out the priors of new nodes (fused search), 0 = none
+    int agent_fences;                // hand-overs between a tree and its evaluators always write the L2 back
 };
 
 // What a tree's workgroup hands to its evaluator workgroups, step by step: the non-terminal children the step created.
@@ -68,8 +69,12 @@ struct EvalRequests {
     int n;       // entries of the step
     int child[kMaxWavesPerBlock];       // node to evaluate, -1 = nothing to do for this entry
     uint64_t hash[kMaxWavesPerBlock];   // its position's hash
+    int xcc[1 + 8];                     // XCD that the tree's workgroup [0] and its evaluators [1..] run on, -1 = not known yet
 };
 constexpr int kMaxEvaluators = 8;
+static_assert(sizeof(EvalRequests::xcc) == sizeof(int) * (1 + kMaxEvaluators), "one entry per workgroup of a tree");
+
+__device__ __forceinline__ int my_xcc() { return (int)(__builtin_amdgcn_s_getreg(6164) & 0xfu); }   // HW_REG_XCC_ID, bits 3:0
 constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s of the 100 MHz clock: a partner that is not there
 
 // What a step keeps per traversal between its phases.  The paths ([traversals][path_depth] words) follow in dynamic LDS.
@@ -775,6 +780,7 @@ __global__ __launch_bounds__(kWave) void init_kernel(const LoopArgs g, const uin
         rq.done = 0;
         rq.abort = 0;
         rq.n = 0;
+        for (int &x : rq.xcc) x = -1;
     }
     if (n_legal > 0) write_priors(g, tree, 0, board, lane, psyn_board_hash(psyn_tree_seed(g.seed, tree), board), n_legal);
 }
@@ -919,6 +925,7 @@ __device__ void evaluate_pair(const LoopArgs &g, EvalLds &L, int tree, int first
 
 __device__ void evaluator_loop(const LoopArgs &g, EvalLds &L, int tree, int helper, int wave, int lane) {
     EvalRequests &rq = g.requests[tree];
+    if (threadIdx.x == 0) __hip_atomic_store(&rq.xcc[1 + helper], my_xcc(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     for (int step = 0;; ++step) {
         if (threadIdx.x == 0) {
             const uint64_t start = wall_clock64();
@@ -949,7 +956,9 @@ __device__ void evaluator_loop(const LoopArgs &g, EvalLds &L, int tree, int help
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (threadIdx.x == 0 && worked_off > 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            // The tree's workgroup wrote its XCD down before it handed out its first step.  On the same XCD the priors
+            // are where it reads them, in the L2 that both share; anywhere else the L2 must be written back first.
+            if (g.agent_fences || poll_word(&rq.xcc[0]) != my_xcc()) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             __hip_atomic_fetch_add(&rq.done, worked_off, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -997,8 +1006,10 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, 
         s.node_count = g.node_count[tree];
         s.requested = 0;
         s.gave_up = 0;
+        if (farm) __hip_atomic_store(&rq.xcc[0], my_xcc(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
+    bool same_l2 = false;   // known: every evaluator of the tree runs on this workgroup's XCD
     uint64_t t0 = wave == 0 ? wall_clock64() : 0;
     for (int step = 0; step < g.steps; ++step) {
         select_phase(g, s, paths, tree, wave, lane, n_waves, work.nodes_read, work.edges_scored);
@@ -1018,7 +1029,15 @@ __global__ __launch_bounds__(kTrav *kWave) void search_kernel(const LoopArgs g, 
         if (farm && threadIdx.x == 0) {   // ... and the evaluators may start on this step's nodes
             rq.n = s.requests;
             s.requested += s.requests;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            if (!same_l2 && !g.agent_fences) {
+                same_l2 = true;
+                for (int h = 1; h <= g.evaluators; ++h) same_l2 = same_l2 && poll_word(&rq.xcc[h]) == my_xcc();
+            }
+            // The phase barrier above has the step's nodes and requests in the L2.  Evaluators on the same XCD read them
+            // there (their acquire drops what their L1 holds); for any other, or one not heard of yet, the L2 is written
+            // back first, which is the expensive part of an agent-scope release.
+            if (same_l2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // rq.n
+            else __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             __hip_atomic_store(&rq.tag, step + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (wave == 0) t2 = wall_clock64();
@@ -1213,6 +1232,7 @@ extern "C" int puct_gomoku_create(const puct_gomoku_config *c, puct_gomoku_engin
     g.m = c->board_m; g.n = c->board_n; g.cells = c->board_m * c->board_n; g.max_nodes = c->max_nodes;
     g.traversals = c->traversals; g.path_depth = c->path_depth; g.steps = 0;
     g.seed = c->seed; g.dirichlet_alpha = c->dirichlet_alpha; g.evaluators = c->evaluators;
+    g.agent_fences = c->agent_fences != 0;
     hipError_t err = hipStreamCreate(&e->stream);
     if (err == hipSuccess) err = hipEventCreate(&e->ev0);
     if (err == hipSuccess) err = hipEventCreate(&e->ev1);

@@ -25,7 +25,7 @@ class Config(ctypes.Structure):
                 ("traversals", ctypes.c_int32), ("max_nodes", ctypes.c_int32), ("path_depth", ctypes.c_int32),
                 ("cpuct", ctypes.c_float), ("c_pw", ctypes.c_float), ("alpha_pw", ctypes.c_float),
                 ("dirichlet_alpha", ctypes.c_float), ("seed", ctypes.c_uint64),
-                ("device", ctypes.c_int32), ("evaluators", ctypes.c_int32)]
+                ("device", ctypes.c_int32), ("evaluators", ctypes.c_int32), ("agent_fences", ctypes.c_int32)]
 
 
 class Result(ctypes.Structure):
@@ -75,14 +75,15 @@ class PUCTGomoku:
     """PUCT search on Gomoku with virtual loss: `trees` independent trees on one root, `traversals` selections per
     tree and step (claims taken in a fixed order, so a search is reproducible), a synthetic evaluator (Dirichlet(dirichlet_alpha) priors over the legal cells and a
     value in [-1, 1), both pure functions of the position and the seed); `evaluators` workgroups per tree work out the
-    priors of new nodes beside the tree's own workgroup (0: it does that itself; same trees either way).  `run` returns the cell with the most root
+    priors of new nodes beside the tree's own workgroup (0: it does that itself; same trees either way; `agent_fences` makes them hand over with full
+    device-scope releases even where they share an L2, which is slower and changes nothing else).  `run` returns the cell with the most root
     visits; `root_n`, `root_q`, `selections`, `performance_info` describe the last search."""
 
     def __init__(self, board_shape=(15, 15), trees=16, traversals=16, max_nodes=16384, path_depth=64, cpuct=1.5,
-                 c_pw=1.0, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, device=0, evaluators=4):
+                 c_pw=1.0, alpha_pw=0.5, dirichlet_alpha=0.3, seed=0, device=0, evaluators=4, agent_fences=False):
         self.cfg = Config(int(board_shape[0]), int(board_shape[1]), int(trees), int(traversals), int(max_nodes),
                           int(path_depth), float(cpuct), float(c_pw), float(alpha_pw), float(dirichlet_alpha), int(seed),
-                          int(device), int(evaluators))
+                          int(device), int(evaluators), int(bool(agent_fences)))
         self._engine = ctypes.c_void_p()
         _check(_lib().puct_gomoku_create(ctypes.byref(self.cfg), ctypes.byref(self._engine)))
         self.result = None

@@ -62,8 +62,8 @@ def test_search_equals_oracle(shape, stones, traversals, steps, max_nodes, depth
     kw = dict(trees=5, traversals=traversals, max_nodes=max_nodes, path_depth=depth, cpuct=1.5, c_pw=c_pw, dirichlet_alpha=0.3, seed=9)
     want = po.gomoku_search(board, turn, steps, **kw)
     gc.check_trees(want, board, turn, shape[0], shape[1], max_nodes, depth)
-    for fused, evaluators in ((True, 4), (True, 0), (True, 8), (False, 0)):
-        e = PUCTGomoku(board_shape=shape, evaluators=evaluators, **kw)
+    for fused, evaluators, agent_fences in ((True, 4, False), (True, 0, False), (True, 8, False), (True, 4, True), (False, 0, False)):
+        e = PUCTGomoku(board_shape=shape, evaluators=evaluators, agent_fences=agent_fences, **kw)
         best = e.run(board, turn, steps, fused=fused)
         got = read_all(e)
         assert_same_trees(got, want)
