@@ -13,6 +13,8 @@
 #include <float.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/puct_select.h"
 
 namespace puct {
@@ -108,11 +110,14 @@ __device__ __forceinline__ bool valid_select_shape(int path_depth, int nodes, in
 }
 
 // Progressive widening, src/puct/puct_gpu_v3_cpp.cu:150-157.
-__device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int n_node, int edges) {
-    const float val = (alpha_pw == 0.5f) ? c_pw * sqrtf((float)n_node) : c_pw * powf((float)n_node, alpha_pw);
+__device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int n_node, int edges, float sqrt_n_node) {
+    const float val = (alpha_pw == 0.5f) ? c_pw * sqrt_n_node : c_pw * powf((float)n_node, alpha_pw);
     if (val >= (float)edges) return edges;
     const int allowed = (int)ceilf(val);
     return allowed > 1 ? allowed : 1;
+}
+__device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int n_node, int edges) {
+    return allowed_children(c_pw, alpha_pw, n_node, edges, sqrtf((float)n_node));
 }
 
 // src/puct/puct_gpu_v3_cpp.cu:171-180
@@ -133,6 +138,56 @@ __device__ __forceinline__ uint64_t candidate_key(float score, int eid, int tie_
     int key = eid - tie_offset;
     if (key < 0) key += span;
     return ((uint64_t)ordered << 32) | ((uint32_t)(0xFFFF - key) << 16) | (uint32_t)eid;
+}
+
+// The same order with the score and the edge index kept apart, for the selections with node-level virtual loss: a
+// 32-bit key per edge whose unsigned order is the order of the scores (0 = not a candidate, as above), the largest of
+// which is found with one `v_max_u32` per DPP step; the edge among the equal ones comes from the lane masks of the
+// comparison with that maximum, on the scalar unit.
+__device__ __forceinline__ uint32_t score_key(float score) {
+    if (!(score >= -FLT_MAX)) return 0;
+    const uint32_t b = __float_as_uint(score + 0.0f);
+    return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    auto step = [](uint32_t x, auto ctrl) {
+        const uint32_t o = (uint32_t)dpp<decltype(ctrl)::value>((int)x);
+        return o > x ? o : x;
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});
+    v = step(v, std::integral_constant<int, 0x4E>{});
+    v = step(v, std::integral_constant<int, 0x141>{});
+    v = step(v, std::integral_constant<int, 0x140>{});
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+    return ab > cd ? ab : cd;
+}
+
+// The edge with the largest key (keys[i] belongs to edge lane + 64 i; `skip` takes no part); among equal keys the one
+// whose index rotated by tie_offset is smallest, i.e. the first at or after tie_offset, else the first.  kNoEdge if no
+// key is above 0.  Every lane returns the same value.
+template <int S>
+__device__ __forceinline__ int best_edge(const uint32_t (&keys)[S], int lane, int skip, int tie_offset) {
+    uint32_t k[S], m = 0;
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+        k[i] = lane + i * kWave == skip ? 0u : keys[i];
+        m = k[i] > m ? k[i] : m;
+    }
+    m = wave_max_u32(m);
+    if (m == 0) return kNoEdge;
+    int at_or_after = kNoEdge, first = kNoEdge;
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+        const uint64_t equal = __builtin_amdgcn_ballot_w64(k[i] == m);
+        const int from = tie_offset - i * kWave;   // lanes of this slice at or after the offset: from `from` on
+        const uint64_t late = equal & (from <= 0 ? ~0ull : from >= kWave ? 0ull : ~0ull << from);
+        if (first == kNoEdge && equal != 0) first = i * kWave + __builtin_ctzll(equal);
+        if (at_or_after == kNoEdge && late != 0) at_or_after = i * kWave + __builtin_ctzll(late);
+    }
+    return at_or_after != kNoEdge ? at_or_after : first;
 }
 
 // Takes back the virtual loss of the first `depth` path entries (src/puct/puct_gpu_v3_cpp.cu:206-217).  The entries
@@ -390,9 +445,13 @@ __device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, cons
 // exchanges (the traversals of a tree that reach a node together all claim the same child, and compare-and-swap then
 // costs a round trip per traversal ahead).
 
-// One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.
+// One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.  A level is written once per
+// number S of 64-edge slices that the node's expanded edges fill (1..4, the same for all lanes): what bounds these
+// kernels is the wavefronts' instruction issue, vector and scalar together, and a level written for "up to four slices"
+// spends a third of it on finding out, slice by slice, that a slice is not there.
 template <bool PRECLAIM>
 __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, int tree, int wid, int lane) {
+    static_assert(kPasses == 4, "the levels below are written for one to four slices");
     const size_t out = (size_t)tree * a.warps + wid;
     int *path = a.out_path_eids + out * a.path_depth;
     const int node_limit = a.node_count[tree];
@@ -405,6 +464,8 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
         edges > 0 && edges <= PUCT_PACKED_EDGE_MASK + 1) {
         int node = 0, depth = 0;
         while (true) {
+            // (the same in all lanes; said so that the level's addresses and branches are worked out once per wavefront)
+            node = __builtin_amdgcn_readfirstlane(node), depth = __builtin_amdgcn_readfirstlane(depth);
             if (node < 0 || node >= node_limit) {
                 rollback_node_path(a, path, tree, depth, lane, node_limit);
                 break;
@@ -415,16 +476,13 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                 break;
             }
             const size_t nrow = trow + node, erow = nrow * edges;
+            const int *row_c = a.edge_child_id + erow, *row_n = a.edge_N + erow;   // one address per wavefront, the lane is the offset
+            const float *row_p = a.edge_prior + erow, *row_w = a.edge_W + erow;
             // the first 64 edges are requested together with the node's own words, before the node's width is known
-            int n[kPasses], f[kPasses], c[kPasses];
-            float p[kPasses], w[kPasses];
-            n[0] = 0, c[0] = -1, p[0] = 0.0f, w[0] = 0.0f;
-            if (lane < edges) {
-                c[0] = a.edge_child_id[erow + lane];
-                n[0] = a.edge_N[erow + lane];
-                p[0] = a.edge_prior[erow + lane];
-                w[0] = a.edge_W[erow + lane];
-            }
+            // (lanes beyond the row read its last edge and take no part)
+            const int at0 = lane < edges ? lane : edges - 1;
+            const int c0 = row_c[at0], n0 = row_n[at0];
+            const float p0 = row_p[at0], w0 = row_w[at0];
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
             if (node_info == PUCT_NODE_EXPANDED_TERMINAL) {
@@ -437,180 +495,178 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                 break;
             }
             const int cur_expanded = node_info;
-#pragma unroll
-            for (int i = 1; i < kPasses; ++i) {
-                n[i] = 0, c[i] = -1, p[i] = 0.0f, w[i] = 0.0f;
-                const int eid = lane + i * kWave;
-                if (i * kWave < cur_expanded && eid < cur_expanded) {
-                    c[i] = a.edge_child_id[erow + eid];
-                    n[i] = a.edge_N[erow + eid];
-                    p[i] = a.edge_prior[erow + eid];
-                    w[i] = a.edge_W[erow + eid];
-                }
-            }
-            // an edge takes part when it is expanded and leads to a node of the tree; its virtual visits are its child's
-            bool valid[kPasses];
-            int total = 0;
-#pragma unroll
-            for (int i = 0; i < kPasses; ++i) {
-                valid[i] = lane + i * kWave < cur_expanded && c[i] >= 0 && c[i] < node_limit;
-                f[i] = (i * kWave < cur_expanded && valid[i]) ? load_relaxed(a.node_inflight + trow + c[i]) : 0;
-            }
-#pragma unroll
-            for (int i = 0; i < kPasses; ++i) total += valid[i] ? n[i] + f[i] : 0;
-            total = wave_sum(total);
-            const int parent_eff = total > 1 ? total : 1;   // :407-416
-            const int allowed = (PRECLAIM && cur_expanded == 0) ? 1 : allowed_children(a.c_pw, a.alpha_pw, parent_eff, edges);
 
-            if (allowed > cur_expanded) {
-                // Expansion ticket, :389-403.  Tickets are only given back by the backup, and a ticket beyond the quota is
-                // returned at once, so a counter that already shows the quota used up stays that way for this launch.
-                int expand_slot = -1;
-                if (cur_expanded + expand_inflight < allowed) {
-                    if (lane == 0) {
-                        const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
-                        if (slot < allowed)
-                            expand_slot = slot;
-                        else
-                            atomicSub(&a.node_expand_inflight[nrow], 1);
-                    }
-                    expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
+            // The level proper; returns the child the traversal moves on to, or -1 when it ends here.
+            auto level = [&](auto slices) __attribute__((always_inline)) -> int {
+                constexpr int S = decltype(slices)::value;   // (S - 1) * 64 < cur_expanded <= S * 64, or no edge at all (S = 1)
+                int n[S], f[S], c[S];
+                float p[S], w[S];
+                bool cand[S];
+                c[0] = c0, n[0] = n0, p[0] = p0, w[0] = w0;
+#pragma unroll
+                for (int i = 1; i < S; ++i) {
+                    const int eid = lane + i * kWave, at = i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1;
+                    c[i] = row_c[at], n[i] = row_n[at], p[i] = row_p[at], w[i] = row_w[at];
                 }
-                if (expand_slot >= 0) {
-                    final_packed = pack_selection_v2(PUCT_SELECT_EXPAND, node, expand_slot);
-                    final_len = depth + 1;
-                } else {
-                    rollback_node_path(a, path, tree, depth, lane, node_limit);
+                // an edge takes part when it is expanded and leads to a node of the tree; its virtual visits are its
+                // child's (the other lanes read the root's counter and drop it)
+                int total = 0;
+#pragma unroll
+                for (int i = 0; i < S; ++i) {
+                    cand[i] = (i < S - 1 || lane + i * kWave < cur_expanded) && (uint32_t)c[i] < (uint32_t)node_limit;
+                    const int visits = load_relaxed(a.node_inflight + trow + (cand[i] ? c[i] : 0));
+                    f[i] = cand[i] ? visits : 0;
                 }
-                break;
-            }
+#pragma unroll
+                for (int i = 0; i < S; ++i) total += cand[i] ? n[i] + f[i] : 0;
+                total = wave_sum(total);
+                const int parent_eff = total > 1 ? total : 1;   // :407-416
+                const float sqrt_parent = sqrtf((float)parent_eff);
+                const int allowed = (PRECLAIM && cur_expanded == 0) ? 1 : allowed_children(a.c_pw, a.alpha_pw, parent_eff, edges, sqrt_parent);
 
-            const float sqrt_parent = sqrtf((float)parent_eff);
-            int best_eid = kNoEdge, held = 0;
-            if (PRECLAIM) {
-                // :448-483: claim every candidate, score it with the count found, keep the winner's claim
-                int tie_offset = wid;
-                if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
-                uint64_t key = 0;
-#pragma unroll
-                for (int i = 0; i < kPasses; ++i) {
-                    if (i * kWave < cur_expanded && valid[i]) {
-                        const int before = atomicAdd(&a.node_inflight[trow + c[i]], 1);
-                        const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], before, sqrt_parent),
-                                                         lane + i * kWave, tie_offset, cur_expanded);
-                        key = k > key ? k : key;
+                if (allowed > cur_expanded) {
+                    // Expansion ticket, :389-403.  Tickets are only given back by the backup, and a ticket beyond the quota is
+                    // returned at once, so a counter that already shows the quota used up stays that way for this launch.
+                    int expand_slot = -1;
+                    if (cur_expanded + expand_inflight < allowed) {
+                        if (lane == 0) {
+                            const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
+                            if (slot < allowed)
+                                expand_slot = slot;
+                            else
+                                atomicSub(&a.node_expand_inflight[nrow], 1);
+                        }
+                        expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
                     }
-                }
-                const uint64_t best = wave_max(key);
-                if (best != 0) best_eid = (int)(best & 0xFFFFu);
-#pragma unroll
-                for (int i = 0; i < kPasses; ++i)
-                    if (i * kWave < cur_expanded && valid[i] && lane + i * kWave != best_eid)
-                        atomicSub(&a.node_inflight[trow + c[i]], 1);
-                held = best_eid != kNoEdge ? 1 : 0;
-            } else {
-                // :520-560 with MAX_RECALC_RETRY = 2 written out: the best edge by the counters as read; its child is
-                // claimed; if that child already carried claims and the node has other edges, the claim is given back and
-                // the best of the other edges is claimed and kept whatever it carries (none: the first winner again).
-                // The counters for the second evaluation are requested together with the first claim, before it is known
-                // whether they will be needed: the reference reads them after its release, but nothing orders those
-                // loads after its relaxed atomics on other counters, and the first winner's own counter is not among the
-                // ones the second evaluation looks at.
-                // every candidate's place in the order "higher score first, then the smaller edge index" (:110-117), 0 = none
-                uint64_t keys[kPasses];
-                auto score_edges = [&] {
-#pragma unroll
-                    for (int i = 0; i < kPasses; ++i)
-                        keys[i] = (i * kWave < cur_expanded && valid[i])
-                                      ? candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], f[i], sqrt_parent), lane + i * kWave, 0, cur_expanded)
-                                      : 0;
-                };
-                auto best_without = [&](int skip) {
-                    uint64_t key = 0;
-#pragma unroll
-                    for (int i = 0; i < kPasses; ++i)
-                        if (lane + i * kWave != skip) key = keys[i] > key ? keys[i] : key;
-                    const uint64_t best = wave_max(key);
-                    return best != 0 ? (int)(best & 0xFFFFu) : kNoEdge;
-                };
-                auto child_of = [&](int eid) {
-                    const int at = eid & (kWave - 1), pass = eid / kWave;
-                    int child = __builtin_amdgcn_readlane(c[0], at);
-#pragma unroll
-                    for (int i = 1; i < kPasses; ++i)
-                        if (pass == i) child = __builtin_amdgcn_readlane(c[i], at);
-                    return child;
-                };
-                // one more visit on `child`'s counter, kept unless the counter was negative or full (:329-331): the value found
-                auto claim = [&](int child, int &found) {
-                    int v = 0;
-                    if (lane == 0) v = atomicAdd(&a.node_inflight[trow + child], 1);
-                    found = __builtin_amdgcn_readfirstlane(v);
-                    if (found < 0 || found >= INT32_MAX) {
-                        if (lane == 0) atomicSub(&a.node_inflight[trow + child], 1);
-                        return 0;
-                    }
-                    return 1;
-                };
-                score_edges();
-                best_eid = best_without(-1);
-                if (best_eid != kNoEdge) {
-                    const int first_child = child_of(best_eid), first_eid = best_eid;
-                    const int seen = [&] {
-                        const int at = first_eid & (kWave - 1), pass = first_eid / kWave;
-                        int v = __builtin_amdgcn_readlane(f[0], at);
-#pragma unroll
-                        for (int i = 1; i < kPasses; ++i)
-                            if (pass == i) v = __builtin_amdgcn_readlane(f[i], at);
-                        return v;
-                    }();
-                    bool second_round = false;
-                    if (seen > 0 && seen < INT32_MAX && cur_expanded > 1) {
-                        // The winner's counter already held visits when it was read.  In the execution in which no other
-                        // traversal acts between that read and this traversal's claim, the claim finds the same value: a
-                        // conflict, upon which the claim is given back and the other edges are evaluated on counters
-                        // that are still the ones read (so the scores stand).  That execution is the one taken: nothing is
-                        // added to the first winner's counter and nothing taken back.  (A claim that is added and taken back
-                        // differs from it only in what other traversals may see in passing, and costs two of the three
-                        // atomics and two of the five round trips of a level.)
-                        second_round = true;
+                    if (expand_slot >= 0) {
+                        final_packed = pack_selection_v2(PUCT_SELECT_EXPAND, node, expand_slot);
+                        final_len = depth + 1;
                     } else {
-                        int found = 0, v = 0;
-                        if (lane == 0) v = atomicAdd(&a.node_inflight[trow + first_child], 1);
+                        rollback_node_path(a, path, tree, depth, lane, node_limit);
+                    }
+                    return -1;
+                }
+
+                // puct_score in two parts: the mean value and the numerator of the exploration term do not depend on the
+                // virtual visits, so an evaluation on counters read again divides once per edge, not twice
+                float q[S], num[S];
 #pragma unroll
-                        for (int i = 0; i < kPasses; ++i)   // (the counters as first read are not needed any more)
-                            if (cur_expanded > 1 && i * kWave < cur_expanded && valid[i]) f[i] = load_relaxed(a.node_inflight + trow + c[i]);
+                for (int i = 0; i < S; ++i) {
+                    // (a slice none of whose edges has a visit or a value has q = +0 without dividing)
+                    q[i] = 0.0f;
+                    if (__builtin_amdgcn_ballot_w64(n[i] > 0 && __float_as_uint(w[i]) != 0u) != 0) q[i] = n[i] > 0 ? w[i] / (float)n[i] : 0.0f;
+                    num[i] = a.cpuct * p[i] * sqrt_parent;
+                }
+                uint32_t keys[S];
+                auto score_slice = [&](int i, int visits) {
+                    return cand[i] ? score_key(q[i] + num[i] / (float)(n[i] + visits + 1)) : 0u;
+                };
+                auto of_edge = [&](const int (&v)[S], int eid) {
+                    const int at = eid & (kWave - 1), pass = eid / kWave;
+                    int r = __builtin_amdgcn_readlane(v[0], at);
+#pragma unroll
+                    for (int i = 1; i < S; ++i)
+                        if (pass == i) r = __builtin_amdgcn_readlane(v[i], at);
+                    return r;
+                };
+                int best_eid = kNoEdge, held = 0;
+                if (PRECLAIM) {
+                    // :448-483: claim every candidate, score it with the count found, keep the winner's claim
+                    int tie_offset = wid;
+                    if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
+#pragma unroll
+                    for (int i = 0; i < S; ++i) {
+                        int before = 0;
+                        if (cand[i]) before = atomicAdd(&a.node_inflight[trow + c[i]], 1);
+                        keys[i] = score_slice(i, before);
+                    }
+                    best_eid = best_edge<S>(keys, lane, -1, tie_offset);
+#pragma unroll
+                    for (int i = 0; i < S; ++i)
+                        if (cand[i] && lane + i * kWave != best_eid) atomicSub(&a.node_inflight[trow + c[i]], 1);
+                    held = best_eid != kNoEdge ? 1 : 0;
+                } else {
+                    // :520-560 with MAX_RECALC_RETRY = 2 written out: the best edge by the counters as read; its child is
+                    // claimed; if that child already carried claims and the node has other edges, the claim is given back and
+                    // the best of the other edges is claimed and kept whatever it carries (none: the first winner again).
+                    // The counters for the second evaluation are requested together with the first claim (just ahead of it, so
+                    // that the wait for the claim's result covers them), before it is known whether they will be needed: the
+                    // reference reads them after its release, but nothing orders those loads after its relaxed atomics on
+                    // other counters, and the first winner's own counter is not among the ones the second evaluation looks at.
+                    // one more visit on `child`'s counter, kept unless the counter was negative or full (:329-331): the value found
+                    auto claim = [&](int child, int &found) {
+                        int v = 0;
+                        if (lane == 0) v = atomicAdd(&a.node_inflight[trow + child], 1);
                         found = __builtin_amdgcn_readfirstlane(v);
                         if (found < 0 || found >= INT32_MAX) {
-                            if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
-                        } else if (found == 0 || cur_expanded <= 1) {
-                            held = 1;
-                        } else {
-                            if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
+                            if (lane == 0) atomicSub(&a.node_inflight[trow + child], 1);
+                            return 0;
+                        }
+                        return 1;
+                    };
+#pragma unroll
+                    for (int i = 0; i < S; ++i) keys[i] = score_slice(i, f[i]);
+                    best_eid = best_edge<S>(keys, lane, -1, 0);
+                    if (best_eid != kNoEdge) {
+                        const int first_child = of_edge(c, best_eid), first_eid = best_eid;
+                        const int seen = of_edge(f, first_eid);
+                        bool second_round = false;
+                        if (seen > 0 && seen < INT32_MAX && cur_expanded > 1) {
+                            // The winner's counter already held visits when it was read.  In the execution in which no other
+                            // traversal acts between that read and this traversal's claim, the claim finds the same value: a
+                            // conflict, upon which the claim is given back and the other edges are evaluated on counters
+                            // that are still the ones read (so the scores stand).  That execution is the one taken: nothing is
+                            // added to the first winner's counter and nothing taken back.  (A claim that is added and taken back
+                            // differs from it only in what other traversals may see in passing, and costs two of the three
+                            // atomics and two of the five round trips of a level.)
                             second_round = true;
-                            score_edges();   // on the counters read again
+                        } else {
+                            int again[S];
+#pragma unroll
+                            for (int i = 0; i < S; ++i) {
+                                const int visits = load_relaxed(a.node_inflight + trow + (cand[i] ? c[i] : 0));
+                                again[i] = cand[i] ? visits : 0;
+                            }
+                            int found;
+                            if (claim(first_child, found) == 0) {
+                                // (the counter cannot be claimed: nothing is held)
+                            } else if (found == 0 || cur_expanded <= 1) {
+                                held = 1;
+                            } else {
+                                if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
+                                second_round = true;
+                                // on the counters read again; other traversals' claims sit on a few edges, so most slices of a
+                                // wide node read what they read before and keep their scores
+#pragma unroll
+                                for (int i = 0; i < S; ++i)
+                                    if (S == 1 || __builtin_amdgcn_ballot_w64(again[i] != f[i]) != 0) keys[i] = score_slice(i, again[i]);
+                            }
+                        }
+                        if (second_round) {
+                            const int second = best_edge<S>(keys, lane, first_eid, 0);
+                            if (second != kNoEdge) best_eid = second;
+                            int found2;
+                            held = claim(of_edge(c, best_eid), found2);
                         }
                     }
-                    if (second_round) {
-                        const int second = best_without(first_eid);
-                        if (second != kNoEdge) best_eid = second;
-                        int found2;
-                        held = claim(child_of(best_eid), found2);
-                    }
                 }
-            }
-            if (held == 0) {   // no edge leads anywhere (or the winner's counter cannot be claimed)
-                rollback_node_path(a, path, tree, depth, lane, node_limit);
-                break;
-            }
-            const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
-            int best_child = __builtin_amdgcn_readlane(c[0], best_lane);
-#pragma unroll
-            for (int i = 1; i < kPasses; ++i)
-                if (best_pass == i) best_child = __builtin_amdgcn_readlane(c[i], best_lane);
-            // (only edges that lead to a node of the tree were candidates, so best_child is one)
-            if (lane == 0) path[depth] = (node << 8) | best_eid;
-            node = best_child;
+                if (held == 0) {   // no edge leads anywhere (or the winner's counter cannot be claimed)
+                    rollback_node_path(a, path, tree, depth, lane, node_limit);
+                    return -1;
+                }
+                // (only edges that lead to a node of the tree were candidates, so the child is one)
+                if (lane == 0) path[depth] = (node << 8) | best_eid;
+                return of_edge(c, best_eid);
+            };
+
+            const int slices = (cur_expanded + kWave - 1) / kWave;
+            int next;
+            if (slices <= 1) next = level(std::integral_constant<int, 1>{});
+            else if (slices == 2) next = level(std::integral_constant<int, 2>{});
+            else if (slices == 3) next = level(std::integral_constant<int, 3>{});
+            else next = level(std::integral_constant<int, 4>{});
+            if (next < 0) break;
+            node = next;
             depth += 1;
         }
     }

@@ -12,7 +12,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_kernel(const 
 
 template <bool PRECLAIM>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void node_select_kernel(const NodeSelectArgs a) {
-    const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
     if (wid >= a.warps) return;
     node_select_traversal<PRECLAIM>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
