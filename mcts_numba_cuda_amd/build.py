@@ -17,11 +17,16 @@ HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
                # instruction cache lines moved measured rates by 3 % between otherwise identical builds
                "-falign-loops=64",
                "-Wno-unknown-warning-option"]
+# The PUCT kernels claim with one lane of a wavefront (`if (lane == 0) atomicAdd(...)`).  The compiler's pass that turns a
+# wavefront's atomics on one address into one atomic of the sum does not see that a single lane is active, and wraps
+# each claim in a lane count and a broadcast (a dozen instructions per claim in kernels bound by instruction issue;
+# the node-level winner-recalc selection is 4-5 % faster without it).
+EXTRA_FLAGS = {PUCT_LIB: ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"]}
 
 
 def build_one(lib, sources, verbose=False):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS + ["-o", lib] + [os.path.join(CSRC, s) for s in sources]
+    cmd = [hipcc] + HIPCC_FLAGS + EXTRA_FLAGS.get(lib, []) + ["-o", lib] + [os.path.join(CSRC, s) for s in sources]
     if verbose:
         print(" ".join(cmd))
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

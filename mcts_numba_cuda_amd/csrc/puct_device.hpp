@@ -6,8 +6,12 @@
 //   * the first 64 edges of a node (all of them for almost every node under progressive widening) are loaded once,
 //     together with the node's own words, before anything about the node is known, so a level costs one round of
 //     loads and one claim instead of a chain of dependent loads;
-//   * the reference's total order on edges (score descending, rotated edge index ascending) is folded into one 64-bit
-//     key, so the arg-max is a single max-reduction over DPP row operations and four lane reads.
+//   * the reference's total order on edges (score descending, rotated edge index ascending) is taken in two steps: the
+//     largest score by a max-reduction of 32-bit keys over DPP row operations, the edge among the equal ones from the
+//     lane masks of the comparison with it, on the scalar unit;
+//   * a level is written once per number of 64-edge slices the node fills, and everything that is the same in all
+//     lanes (node, depth, row addresses, branches) is kept on the scalar side: the kernels are bound by instruction
+//     issue, not by the memory they read.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <float.h>
@@ -120,14 +124,11 @@ __device__ __forceinline__ int allowed_children(float c_pw, float alpha_pw, int 
     return allowed_children(c_pw, alpha_pw, n_node, edges, sqrtf((float)n_node));
 }
 
-// src/puct/puct_gpu_v3_cpp.cu:171-180
-__device__ __forceinline__ float puct_score(float cpuct, float prior, float w, int n, int inflight, float sqrt_parent) {
-    const float q = n > 0 ? w / (float)n : 0.0f;
-    const float u = cpuct * prior * sqrt_parent / (float)(n + inflight + 1);
-    return q + u;
-}
+// The score of an edge (src/puct/puct_gpu_v3_cpp.cu:171-180) is q + u with q = n > 0 ? w / n : 0 and
+// u = cpuct * prior * sqrt_parent / (n + inflight + 1), in single precision, operation by operation.  The selections
+// below keep q and the numerator of u per edge and divide again when the in-flight counts have been read again.
 
-// One 64-bit key per candidate edge whose unsigned order is the reference's order "higher score first, then smaller
+// One 64-bit key per candidate edge (used by the Gomoku search loop) whose unsigned order is the reference's order "higher score first, then smaller
 // rotated edge index" (src/puct/puct_gpu_v3_cpp.cu:51-71).  0 means "not a candidate": the reference starts from
 // (-FLT_MAX, no edge) and accepts a score that is greater than or equal to it, so NaN and -inf never win.  -0.0f is
 // made +0.0f because the reference compares floats, for which the two are equal.
@@ -140,7 +141,7 @@ __device__ __forceinline__ uint64_t candidate_key(float score, int eid, int tie_
     return ((uint64_t)ordered << 32) | ((uint32_t)(0xFFFF - key) << 16) | (uint32_t)eid;
 }
 
-// The same order with the score and the edge index kept apart, for the selections with node-level virtual loss: a
+// The same order with the score and the edge index kept apart, for the selection kernels of this file: a
 // 32-bit key per edge whose unsigned order is the order of the scores (0 = not a candidate, as above), the largest of
 // which is found with one `v_max_u32` per DPP step; the edge among the equal ones comes from the lane masks of the
 // comparison with that maximum, on the scalar unit.
@@ -203,8 +204,12 @@ __device__ __forceinline__ void rollback_path(const SelectArgs &a, const int *pa
     }
 }
 
-// One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.
+// One traversal (tree, wid) by one wavefront; every lane of the wavefront must call it.  A level is written once per
+// number S of 64-edge slices that the node's expanded edges fill (1..4, the same for all lanes): these kernels are bound
+// by the wavefronts' instruction issue, vector and scalar together, and a level written for "up to four slices" spends a
+// third of it on finding out, slice by slice, that a slice is not there.
 __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, int wid, int lane) {
+    static_assert(kPasses == 4, "the levels below are written for one to four slices");
     const size_t out = (size_t)tree * a.warps + wid;
     int *path = a.out_path_eids + out * a.path_depth;
     const int node_cnt = a.tree_nodes[tree];
@@ -219,22 +224,21 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
     } else {
         int node = 0, depth = 0;
         while (true) {
+            // (the same in all lanes; said so that the level's addresses and branches are worked out once per wavefront)
+            node = __builtin_amdgcn_readfirstlane(node), depth = __builtin_amdgcn_readfirstlane(depth);
             levels += 1;
             const size_t nrow = (size_t)tree * nodes + node;
             const size_t erow = nrow * edges;
+            const int *row_n = a.edge_N + erow, *row_c = a.edge_child_id + erow;   // one address per wavefront, the lane is the offset
+            int *row_f = a.edge_inflight + erow;
+            const float *row_p = a.edge_prior + erow, *row_w = a.edge_W + erow;
 
-            // Everything a level can need from the first 64 edges, requested in one go; the edges of wider nodes follow
-            // once the node's width is known and stay in registers for the rest of the level.
-            int n[kPasses], f[kPasses], c[kPasses];
-            float p[kPasses], w[kPasses];
-            n[0] = 0, f[0] = 0, c[0] = -1, p[0] = 0.0f, w[0] = 0.0f;
-            if (lane < edges) {
-                n[0] = a.edge_N[erow + lane];
-                f[0] = load_relaxed(a.edge_inflight + erow + lane);
-                p[0] = a.edge_prior[erow + lane];
-                w[0] = a.edge_W[erow + lane];
-                c[0] = a.edge_child_id[erow + lane];
-            }
+            // Everything a level can need from the first 64 edges, requested in one go, before the node's width is known
+            // (lanes beyond the row read its last edge and take no part); the edges of wider nodes follow once it is
+            // and stay in registers for the rest of the level.
+            const int at0 = lane < edges ? lane : edges - 1;
+            const int n0 = row_n[at0], f0 = load_relaxed(row_f + at0), c0 = row_c[at0];
+            const float p0 = row_p[at0], w0 = row_w[at0];
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
             const int capacity = a.node_capacity ? a.node_capacity[nrow] : edges;
@@ -258,127 +262,155 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
 
             const int cur_expanded = node_info;
             edges_seen += cur_expanded;
-#pragma unroll
-            for (int i = 1; i < kPasses; ++i) {
-                n[i] = 0, f[i] = 0, c[i] = -1, p[i] = 0.0f, w[i] = 0.0f;
-                const int eid = lane + i * kWave;
-                if (i * kWave < cur_expanded && eid < cur_expanded) {
-                    n[i] = a.edge_N[erow + eid];
-                    f[i] = load_relaxed(a.edge_inflight + erow + eid);
-                    p[i] = a.edge_prior[erow + eid];
-                    w[i] = a.edge_W[erow + eid];
-                    c[i] = a.edge_child_id[erow + eid];
-                }
-            }
-            int parent_eff = 1, allowed = 1;
-            if (cur_expanded != 1 || a.c_pw != 0.0f) {
-                int total = 0;
-#pragma unroll
-                for (int i = 0; i < kPasses; ++i) total += lane + i * kWave < cur_expanded ? n[i] + f[i] : 0;
-                total = wave_sum(total);
-                parent_eff = total > 1 ? total : 1;
-                allowed = allowed_children(a.c_pw, a.alpha_pw, parent_eff, capacity);
-            }
 
-            if (allowed > cur_expanded) {
-                // Expansion ticket, src/puct/puct_gpu_v3_cpp.cu:219-233.
-                int expand_slot = -1;
-                if (cur_expanded + expand_inflight < allowed) {
-                    if (lane == 0) {
-                        const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
-                        if (slot < allowed)
-                            expand_slot = slot;
-                        else
-                            atomicSub(&a.node_expand_inflight[nrow], 1);
+            // The level proper; returns the child the traversal moves on to, or -1 when it ends here.
+            auto level = [&](auto slices) __attribute__((always_inline)) -> int {
+                constexpr int S = decltype(slices)::value;   // (S - 1) * 64 < cur_expanded <= S * 64, or no edge at all (S = 1)
+                int n[S], f[S], c[S], at[S];
+                float p[S], w[S];
+                bool in_node[S];
+                n[0] = n0, f[0] = f0, c[0] = c0, p[0] = p0, w[0] = w0, at[0] = at0;
+#pragma unroll
+                for (int i = 1; i < S; ++i) {
+                    const int eid = lane + i * kWave;
+                    at[i] = i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1;
+                    n[i] = row_n[at[i]], f[i] = load_relaxed(row_f + at[i]), p[i] = row_p[at[i]], w[i] = row_w[at[i]], c[i] = row_c[at[i]];
+                }
+#pragma unroll
+                for (int i = 0; i < S; ++i) in_node[i] = i < S - 1 || lane + i * kWave < cur_expanded;
+
+                int parent_eff = 1, allowed = 1;
+                float sqrt_parent = 1.0f;
+                if (cur_expanded != 1 || a.c_pw != 0.0f) {
+                    int total = 0;
+#pragma unroll
+                    for (int i = 0; i < S; ++i) total += in_node[i] ? n[i] + f[i] : 0;
+                    total = wave_sum(total);
+                    parent_eff = total > 1 ? total : 1;
+                    sqrt_parent = sqrtf((float)parent_eff);
+                    allowed = allowed_children(a.c_pw, a.alpha_pw, parent_eff, capacity, sqrt_parent);
+                }
+
+                if (allowed > cur_expanded) {
+                    // Expansion ticket, src/puct/puct_gpu_v3_cpp.cu:219-233.
+                    int expand_slot = -1;
+                    if (cur_expanded + expand_inflight < allowed) {
+                        if (lane == 0) {
+                            const int slot = cur_expanded + atomicAdd(&a.node_expand_inflight[nrow], 1);
+                            if (slot < allowed)
+                                expand_slot = slot;
+                            else
+                                atomicSub(&a.node_expand_inflight[nrow], 1);
+                        }
+                        expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
                     }
-                    expand_slot = __builtin_amdgcn_readfirstlane(expand_slot);
+                    if (expand_slot >= 0) {
+                        final_packed = pack_selection(PUCT_SELECT_EXPAND, node, expand_slot, PUCT_REASON_OK_EXPAND);
+                        final_len = depth + 1;
+                        return -1;
+                    }
+                    if (cur_expanded == 0) {
+                        rollback_path(a, path, tree, depth, lane, node_cnt);
+                        final_packed = pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_EXPAND_INFLIGHT);
+                        return -1;
+                    }
                 }
-                if (expand_slot >= 0) {
-                    final_packed = pack_selection(PUCT_SELECT_EXPAND, node, expand_slot, PUCT_REASON_OK_EXPAND);
-                    final_len = depth + 1;
-                    break;
-                }
-                if (cur_expanded == 0) {
-                    rollback_path(a, path, tree, depth, lane, node_cnt);
-                    final_packed = pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_EXPAND_INFLIGHT);
-                    break;
-                }
-            }
 
-            int tie_offset = wid;
-            if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
+                int tie_offset = wid;
+                if (tie_offset >= cur_expanded) tie_offset %= cur_expanded;
 
-            int best_eid = 0, held = 0;
-            if (cur_expanded == 1) {
-                if (lane == 0) atomicAdd(&a.edge_inflight[erow], 1);
-                held = 1;
-            } else {
-                // Winner-recalc claim, src/puct/puct_gpu_v3_cpp.cu:235-275: score all edges, try to move the winner's
-                // in-flight count from the value the score was computed with to that value plus one, rescore once if
-                // another traversal got there first.
-                const float sqrt_parent = sqrtf((float)parent_eff);
-                best_eid = kNoEdge;
-                for (int attempt = 0; attempt < a.recalc_attempts; ++attempt) {
-                    uint64_t key = 0;
-                    int my_inflight = 0;
+                auto of_edge = [&](const int (&v)[S], int eid) {
+                    const int lane_of = eid & (kWave - 1), pass = eid / kWave;
+                    int r = __builtin_amdgcn_readlane(v[0], lane_of);
 #pragma unroll
-                    for (int i = 0; i < kPasses; ++i) {
-                        const int eid = lane + i * kWave;
-                        if (i * kWave < cur_expanded && eid < cur_expanded) {
-                            const int fi = attempt == 0 ? f[i] : load_relaxed(a.edge_inflight + erow + eid);
-                            const uint64_t k = candidate_key(puct_score(a.cpuct, p[i], w[i], n[i], fi, sqrt_parent), eid,
-                                                             tie_offset, cur_expanded);
-                            if (k > key) {
-                                key = k;
-                                my_inflight = fi;
+                    for (int i = 1; i < S; ++i)
+                        if (pass == i) r = __builtin_amdgcn_readlane(v[i], lane_of);
+                    return r;
+                };
+
+                int best_eid = 0, held = 0;
+                if (cur_expanded == 1) {
+                    if (lane == 0) atomicAdd(row_f, 1);
+                    held = 1;
+                } else {
+                    // Winner-recalc claim, src/puct/puct_gpu_v3_cpp.cu:235-275: score all edges, try to move the winner's
+                    // in-flight count from the value the score was computed with to that value plus one, rescore once if
+                    // another traversal got there first.  The mean value and the numerator of the exploration term do not
+                    // depend on the in-flight counts, so a second evaluation divides once per edge, and only in the slices
+                    // whose counts have changed (other traversals' claims sit on a few edges).
+                    float q[S], num[S];
+#pragma unroll
+                    for (int i = 0; i < S; ++i) {
+                        // (a slice none of whose edges has a visit or a value has q = +0 without dividing)
+                        q[i] = 0.0f;
+                        if (__builtin_amdgcn_ballot_w64(n[i] > 0 && __float_as_uint(w[i]) != 0u) != 0) q[i] = n[i] > 0 ? w[i] / (float)n[i] : 0.0f;
+                        num[i] = a.cpuct * p[i] * sqrt_parent;
+                    }
+                    uint32_t keys[S];
+                    auto score_slice = [&](int i, int inflight) {
+                        return in_node[i] ? score_key(q[i] + num[i] / (float)(n[i] + inflight + 1)) : 0u;
+                    };
+                    best_eid = kNoEdge;
+                    for (int attempt = 0; attempt < a.recalc_attempts; ++attempt) {
+                        if (attempt == 0) {
+#pragma unroll
+                            for (int i = 0; i < S; ++i) keys[i] = score_slice(i, f[i]);
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < S; ++i) {
+                                const int fi = load_relaxed(row_f + at[i]);
+                                if (__builtin_amdgcn_ballot_w64(fi != f[i]) != 0) {
+                                    f[i] = fi;
+                                    keys[i] = score_slice(i, fi);
+                                }
                             }
                         }
+                        best_eid = best_edge<S>(keys, lane, -1, tie_offset);
+                        if (best_eid == kNoEdge) break;
+                        const int best_inflight = of_edge(f, best_eid);
+                        int got = 0;
+                        if (lane == 0) {
+                            const int prev = atomicCAS(row_f + best_eid, best_inflight, best_inflight + 1);
+                            got = prev == best_inflight ? 1 : 0;
+                        }
+                        held = __builtin_amdgcn_readfirstlane(got);
+                        if (held) break;
                     }
-                    const uint64_t best = wave_max(key);
-                    if (best == 0) {
-                        best_eid = kNoEdge;
-                        break;
+                    if (a.soft_winner != 0 && held == 0 && best_eid != kNoEdge) {
+                        if (lane == 0) atomicAdd(row_f + best_eid, 1);
+                        held = 1;
                     }
-                    best_eid = (int)(best & 0xFFFFu);
-                    const int best_inflight = __builtin_amdgcn_readlane(my_inflight, best_eid & (kWave - 1));
-                    int got = 0;
-                    if (lane == 0) {
-                        const int prev = atomicCAS(&a.edge_inflight[erow + best_eid], best_inflight, best_inflight + 1);
-                        got = prev == best_inflight ? 1 : 0;
-                    }
-                    held = __builtin_amdgcn_readfirstlane(got);
-                    if (held) break;
                 }
-                if (a.soft_winner != 0 && held == 0 && best_eid != kNoEdge) {
-                    if (lane == 0) atomicAdd(&a.edge_inflight[erow + best_eid], 1);
-                    held = 1;
+
+                if (held == 0) {
+                    rollback_path(a, path, tree, depth, lane, node_cnt);
+                    final_packed =
+                        best_eid == kNoEdge
+                            ? pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NO_VALID_EDGE)
+                            : pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_WINNER_RECALC);
+                    return -1;
                 }
-            }
 
-            if (held == 0) {
-                rollback_path(a, path, tree, depth, lane, node_cnt);
-                final_packed =
-                    best_eid == kNoEdge
-                        ? pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NO_VALID_EDGE)
-                        : pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_WINNER_RECALC);
-                break;
-            }
+                const int best_child = of_edge(c, best_eid);
+                if (best_child < 0 || best_child >= node_cnt) {
+                    if (lane == 0) atomicSub(row_f + best_eid, 1);
+                    rollback_path(a, path, tree, depth, lane, node_cnt);
+                    final_packed =
+                        pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_CHILD_OOB);
+                    return -1;
+                }
+                if (lane == 0) path[depth] = (node << 8) | best_eid;
+                return best_child;
+            };
 
-            const int best_lane = best_eid & (kWave - 1), best_pass = best_eid / kWave;
-            int best_child = __builtin_amdgcn_readlane(c[0], best_lane);
-#pragma unroll
-            for (int i = 1; i < kPasses; ++i)
-                if (best_pass == i) best_child = __builtin_amdgcn_readlane(c[i], best_lane);
-            if (best_child < 0 || best_child >= node_cnt) {
-                if (lane == 0) atomicSub(&a.edge_inflight[erow + best_eid], 1);
-                rollback_path(a, path, tree, depth, lane, node_cnt);
-                final_packed =
-                    pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_CHILD_OOB);
-                break;
-            }
-
-            if (lane == 0) path[depth] = (node << 8) | best_eid;
-            node = best_child;
+            const int slices = (cur_expanded + kWave - 1) / kWave;
+            int next;
+            if (slices <= 1) next = level(std::integral_constant<int, 1>{});
+            else if (slices == 2) next = level(std::integral_constant<int, 2>{});
+            else if (slices == 3) next = level(std::integral_constant<int, 3>{});
+            else next = level(std::integral_constant<int, 4>{});
+            if (next < 0) break;
+            node = next;
             depth += 1;
         }
     }

@@ -5,7 +5,7 @@ namespace {
 using namespace puct;
 
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_kernel(const SelectArgs a) {
-    const int wid = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+    const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
     if (wid >= a.warps) return;
     select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
