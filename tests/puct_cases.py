@@ -290,6 +290,30 @@ def case_tie_rotation_by_wid(r):
     assert inflight_sum(r.release()) == 0
 
 
+def case_tie_rotation_across_slices_and_around(r):
+    """200 expanded edges with prior 0 (scores do not depend on what is in flight); the best Q sits on edges 3, 70 and
+    130.  Traversal wid takes the first of them at or after index wid, and edge 3 again once wid is beyond 130 (the
+    rotated index eid - wid mod 200 is smallest there), whatever the interleaving; with the soft winner every claim
+    lands, so the counts are known too.  140 traversals: offsets in every 64-edge slice, spread over nine workgroups."""
+    span, warps, best = 200, 140, (3, 70, 130)
+    c = make_case(nodes=span + 1, actions=256, warps=warps, path_depth=2)
+    c["node_expanded"][0, 0] = span
+    c["node_expanded"][0, 1:] = TERMINAL
+    c["edge_child"][0, 0, :span] = np.arange(1, span + 1)
+    c["edge_n"][0, 0, :span] = 4
+    c["edge_w"][0, 0, :span] = 1.0
+    c["edge_w"][0, 0, list(best)] = 2.0
+    c["edge_prior"][0, 0, :span] = 0.0
+    h = r.select(c, c_pw=0.0, soft_winner=1)
+    want = [next((e for e in best if e >= wid), best[0]) for wid in range(warps)]
+    assert h["out_path"][0, :, 0].tolist() == want
+    assert [decode(x) for x in h["out_selected"][0]] == [(TERMINAL_KIND, 0, e + 1) for e in want]
+    counts = np.zeros(256, np.int32)
+    np.add.at(counts, want, 1)
+    assert np.array_equal(h["edge_inflight"][0, 0], counts)
+    assert inflight_sum(r.release()) == 0
+
+
 def case_wide_node_beyond_one_wavefront(r):
     """200 expanded edges; the single best one sits at index 137 (beyond the first 64 lanes) because of its prior."""
     e = 200
@@ -353,7 +377,7 @@ REFERENCE_CASES = [case_fresh_root_expand, case_terminal_root, case_invalid_chil
                    case_fully_expanded_select_release, case_fully_expanded_select_backup, case_depth_limit,
                    case_zero_n_edge_selectable, case_encoding_boundaries]
 ARITHMETIC_CASES = [case_hand_computed_scores, case_virtual_loss_lowers_score, case_tie_rotation_by_wid,
-                    case_wide_node_beyond_one_wavefront, case_nan_and_minus_inf_never_win, case_deep_chain_rollback,
+                    case_tie_rotation_across_slices_and_around, case_wide_node_beyond_one_wavefront, case_nan_and_minus_inf_never_win, case_deep_chain_rollback,
                     case_deep_chain_terminal]
 ALL_CASES = REFERENCE_CASES + ARITHMETIC_CASES
 

@@ -215,6 +215,36 @@ def case_ties(r, variant):
     assert r.select(c, variant, c_pw=0.0)["out_path"][0, 0, 0] == 2
 
 
+def case_ties_across_slices_and_around(r, variant):
+    """200 expanded edges with prior 0 (a score is its Q, whatever the counters hold); the best Q sits on edges 3, 70 and
+    130.  Under every interleaving: the preclaim kernel's traversal wid takes the first of them at or after index wid and
+    edge 3 again once wid is beyond 130 (:121-144); of the winner-recalc kernel's traversals exactly one keeps edge 3
+    (the claim that found the child free), all others meet a conflict there and keep the best of the rest, edge 70
+    (:520-560).  140 traversals: rotation offsets in every 64-edge slice, spread over nine workgroups."""
+    span, warps, best = 200, 140, (3, 70, 130)
+    c = make_case(nodes=span + 1, actions=256, warps=warps, path_depth=2)
+    c["node_expanded"][0, 0] = span
+    c["node_expanded"][0, 1:] = TERMINAL
+    c["edge_child"][0, 0, :span] = np.arange(1, span + 1)
+    c["edge_n"][0, 0, :span] = 4
+    c["edge_w"][0, 0, :span] = 1.0
+    c["edge_w"][0, 0, list(best)] = 2.0
+    c["edge_prior"][0, 0, :span] = 0.0
+    h = r.select(c, variant, c_pw=0.0)
+    got = h["out_path"][0, :, 0].tolist()
+    if variant == "preclaim":
+        want = [next((e for e in best if e >= wid), best[0]) for wid in range(warps)]
+        assert got == want
+    else:
+        want = [3] + [70] * (warps - 1)
+        assert sorted(got) == want
+    assert [decode(x) for x in h["out_selected"][0]] == [(TERMINAL_KIND, 0, e + 1) for e in got]
+    counts = np.zeros(span + 1, np.int32)
+    np.add.at(counts, [e + 1 for e in want], 1)
+    assert np.array_equal(h["node_inflight"][0], counts)
+    assert inflight_sum(r.backup(zeros_like_path(h))) == 0
+
+
 def case_preclaim_rotation_by_wid(r, variant):
     """Four traversals on four equal edges.  One after another (the oracle), the preclaim kernel's traversal wid finds the
     children taken before it one claim heavier and, among the equal rest, prefers edge wid (:121-144): four different
@@ -331,7 +361,7 @@ REFERENCE_CASES = [case_fresh_root_expand_roundtrip, case_terminal_root, case_in
                    case_child_beyond_node_count, case_progressive_widening_unique_slots,
                    case_fully_expanded_select_and_backup, case_depth_limit, case_encoding_boundaries]
 ARITHMETIC_CASES = [case_hand_computed_scores, case_edges_that_lead_nowhere_are_no_candidates, case_ties,
-                    case_preclaim_rotation_by_wid, case_winner_recalc_conflict, case_fresh_node_quota,
+                    case_ties_across_slices_and_around, case_preclaim_rotation_by_wid, case_winner_recalc_conflict, case_fresh_node_quota,
                     case_wide_node_beyond_one_wavefront, case_nan_and_minus_inf_never_win, case_deep_chain]
 ALL_CASES = REFERENCE_CASES + ARITHMETIC_CASES
 
