@@ -4,14 +4,14 @@
 namespace {
 using namespace puct;
 
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void select_kernel(const SelectArgs a) {
+__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) void select_kernel(const SelectArgs a) {
     const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
     if (wid >= a.warps) return;
     select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
 template <bool PRECLAIM>
-__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void node_select_kernel(const NodeSelectArgs a) {
+__global__ __launch_bounds__(kMaxWavesPerBlock *kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) void node_select_kernel(const NodeSelectArgs a) {
     const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
     if (wid >= a.warps) return;
     node_select_traversal<PRECLAIM>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
