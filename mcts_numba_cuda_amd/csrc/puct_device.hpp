@@ -454,8 +454,33 @@ __device__ __forceinline__ int pack_selection_v2(int kind, int node, int slot) {
     return (kind << PUCT_PACKED_KIND_SHIFT) | (slot << PUCT_PACKED_SLOT_SHIFT) | node;
 }
 
+// The virtual visits of one tree's nodes, node_inflight[tree, :].  While a launch runs they are read and changed by
+// the traversals of that tree only; when those are the wavefronts of one workgroup (up to 16 traversals per tree) and the
+// tree's counters fit, the workgroup keeps them in LDS for the launch (LOCAL): loaded at the start, stored at the end, and
+// every claim in between is an LDS atomic instead of one performed at the memory side (the preclaim kernel makes two per
+// edge and level; in device memory they were what bounded it).
+typedef __attribute__((address_space(3))) int *LdsInts;
+template <bool LOCAL>
+struct NodeVisits {
+    int *in_memory;     // node_inflight + tree * nodes
+    LdsInts in_lds;     // the same counters, workgroup's copy
+    __device__ __forceinline__ int peek(int node) const {
+        if (LOCAL) return __hip_atomic_load(in_lds + node, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return load_relaxed(in_memory + node);
+    }
+    __device__ __forceinline__ int add(int node, int v) const {   // returns the count found
+        if (LOCAL) return __hip_atomic_fetch_add(in_lds + node, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return atomicAdd(in_memory + node, v);
+    }
+    __device__ __forceinline__ void sub(int node, int v) const {
+        if (LOCAL) __hip_atomic_fetch_sub(in_lds + node, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else atomicSub(in_memory + node, v);
+    }
+};
+
 // src/puct/puct_gpu_v2.py:291-310: the claims of the first `depth` path entries live on the child each entry leads to.
-__device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, const int *path, int tree, int depth, int lane,
+template <bool LOCAL>
+__device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, const NodeVisits<LOCAL> &visits_of, const int *path, int tree, int depth, int lane,
                                                    int node_limit) {
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");   // lane 0 stored the entries
     for (int d = lane; d < depth; d += kWave) {
@@ -464,7 +489,7 @@ __device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, cons
         const int parent = encoded >> 8, slot = encoded & 0xFF;
         if (parent < node_limit && slot < a.edges) {
             const int child = a.edge_child_id[((size_t)tree * a.nodes + parent) * a.edges + slot];
-            if (child >= 0 && child < node_limit) atomicSub(&a.node_inflight[(size_t)tree * a.nodes + child], 1);
+            if (child >= 0 && child < node_limit) visits_of.sub(child, 1);
         }
     }
 }
@@ -481,8 +506,8 @@ __device__ __forceinline__ void rollback_node_path(const NodeSelectArgs &a, cons
 // number S of 64-edge slices that the node's expanded edges fill (1..4, the same for all lanes): what bounds these
 // kernels is the wavefronts' instruction issue, vector and scalar together, and a level written for "up to four slices"
 // spends a third of it on finding out, slice by slice, that a slice is not there.
-template <bool PRECLAIM>
-__device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, int tree, int wid, int lane) {
+template <bool PRECLAIM, bool LOCAL>
+__device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, const NodeVisits<LOCAL> &visits_of, int tree, int wid, int lane) {
     static_assert(kPasses == 4, "the levels below are written for one to four slices");
     const size_t out = (size_t)tree * a.warps + wid;
     int *path = a.out_path_eids + out * a.path_depth;
@@ -499,7 +524,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
             // (the same in all lanes; said so that the level's addresses and branches are worked out once per wavefront)
             node = __builtin_amdgcn_readfirstlane(node), depth = __builtin_amdgcn_readfirstlane(depth);
             if (node < 0 || node >= node_limit) {
-                rollback_node_path(a, path, tree, depth, lane, node_limit);
+                rollback_node_path(a, visits_of, path, tree, depth, lane, node_limit);
                 break;
             }
             if (depth >= a.path_depth) {   // the path buffer is full: stop before reading or claiming anything here
@@ -523,7 +548,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                 break;
             }
             if (node_info < 0 || node_info > edges) {
-                rollback_node_path(a, path, tree, depth, lane, node_limit);
+                rollback_node_path(a, visits_of, path, tree, depth, lane, node_limit);
                 break;
             }
             const int cur_expanded = node_info;
@@ -546,7 +571,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
 #pragma unroll
                 for (int i = 0; i < S; ++i) {
                     cand[i] = (i < S - 1 || lane + i * kWave < cur_expanded) && (uint32_t)c[i] < (uint32_t)node_limit;
-                    const int visits = load_relaxed(a.node_inflight + trow + (cand[i] ? c[i] : 0));
+                    const int visits = visits_of.peek(cand[i] ? c[i] : 0);
                     f[i] = cand[i] ? visits : 0;
                 }
 #pragma unroll
@@ -574,7 +599,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                         final_packed = pack_selection_v2(PUCT_SELECT_EXPAND, node, expand_slot);
                         final_len = depth + 1;
                     } else {
-                        rollback_node_path(a, path, tree, depth, lane, node_limit);
+                        rollback_node_path(a, visits_of, path, tree, depth, lane, node_limit);
                     }
                     return -1;
                 }
@@ -609,13 +634,13 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
 #pragma unroll
                     for (int i = 0; i < S; ++i) {
                         int before = 0;
-                        if (cand[i]) before = atomicAdd(&a.node_inflight[trow + c[i]], 1);
+                        if (cand[i]) before = visits_of.add(c[i], 1);
                         keys[i] = score_slice(i, before);
                     }
                     best_eid = best_edge<S>(keys, lane, -1, tie_offset);
 #pragma unroll
                     for (int i = 0; i < S; ++i)
-                        if (cand[i] && lane + i * kWave != best_eid) atomicSub(&a.node_inflight[trow + c[i]], 1);
+                        if (cand[i] && lane + i * kWave != best_eid) visits_of.sub(c[i], 1);
                     held = best_eid != kNoEdge ? 1 : 0;
                 } else {
                     // :520-560 with MAX_RECALC_RETRY = 2 written out: the best edge by the counters as read; its child is
@@ -628,10 +653,10 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                     // one more visit on `child`'s counter, kept unless the counter was negative or full (:329-331): the value found
                     auto claim = [&](int child, int &found) {
                         int v = 0;
-                        if (lane == 0) v = atomicAdd(&a.node_inflight[trow + child], 1);
+                        if (lane == 0) v = visits_of.add(child, 1);
                         found = __builtin_amdgcn_readfirstlane(v);
                         if (found < 0 || found >= INT32_MAX) {
-                            if (lane == 0) atomicSub(&a.node_inflight[trow + child], 1);
+                            if (lane == 0) visits_of.sub(child, 1);
                             return 0;
                         }
                         return 1;
@@ -656,7 +681,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                             int again[S];
 #pragma unroll
                             for (int i = 0; i < S; ++i) {
-                                const int visits = load_relaxed(a.node_inflight + trow + (cand[i] ? c[i] : 0));
+                                const int visits = visits_of.peek(cand[i] ? c[i] : 0);
                                 again[i] = cand[i] ? visits : 0;
                             }
                             int found;
@@ -665,7 +690,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                             } else if (found == 0 || cur_expanded <= 1) {
                                 held = 1;
                             } else {
-                                if (lane == 0) atomicSub(&a.node_inflight[trow + first_child], 1);
+                                if (lane == 0) visits_of.sub(first_child, 1);
                                 second_round = true;
                                 // on the counters read again; other traversals' claims sit on a few edges, so most slices of a
                                 // wide node read what they read before and keep their scores
@@ -683,7 +708,7 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, i
                     }
                 }
                 if (held == 0) {   // no edge leads anywhere (or the winner's counter cannot be claimed)
-                    rollback_node_path(a, path, tree, depth, lane, node_limit);
+                    rollback_node_path(a, visits_of, path, tree, depth, lane, node_limit);
                     return -1;
                 }
                 // (only edges that lead to a node of the tree were candidates, so the child is one)

@@ -10,11 +10,23 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) __attribute__((amdgpu_wav
     select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
-template <bool PRECLAIM>
+// LOCAL: the tree's traversals are this workgroup's wavefronts (grid.y == 1) and its virtual-visit counters are kept
+// in the workgroup's dynamic LDS for the launch (a.nodes words).
+template <bool PRECLAIM, bool LOCAL>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) void node_select_kernel(const NodeSelectArgs a) {
+    extern __shared__ int tree_visits[];
     const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
-    if (wid >= a.warps) return;
-    node_select_traversal<PRECLAIM>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
+    int *const in_memory = a.node_inflight + (size_t)blockIdx.x * a.nodes;
+    const NodeVisits<LOCAL> visits_of{in_memory, (LdsInts)tree_visits};
+    if (LOCAL) {
+        for (int i = threadIdx.x; i < a.nodes; i += blockDim.x) tree_visits[i] = in_memory[i];
+        __syncthreads();
+    }
+    if (LOCAL || wid < a.warps) node_select_traversal<PRECLAIM, LOCAL>(a, visits_of, blockIdx.x, wid, threadIdx.x & (kWave - 1));
+    if (LOCAL) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < a.nodes; i += blockDim.x) in_memory[i] = tree_visits[i];
+    }
 }
 
 template <bool NODE_LEVEL>
@@ -23,6 +35,8 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_kernel(const 
     if (wid >= a.warps) return;
     backup_traversal<NODE_LEVEL>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
+
+constexpr int kLocalVisitNodes = 4096;
 
 // One wavefront per traversal; a tree with more than 16 traversals is spread over several workgroups.
 inline void launch_shape(int trees, int warps, dim3 &grid, dim3 &block) {
@@ -60,7 +74,11 @@ int launch_node_select(float cpuct, float c_pw, float alpha_pw, const int *edge_
                      out_path_eids, out_path_len, trees,             nodes,         edges,        warps,  path_depth};
     dim3 grid, block;
     launch_shape(trees, warps, grid, block);
-    hipLaunchKernelGGL(node_select_kernel<PRECLAIM>, grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
+    // (the counters of a tree in LDS: up to 4096 nodes, so that a CU still holds four workgroups)
+    if (grid.y == 1 && nodes > 0 && nodes <= kLocalVisitNodes)
+        hipLaunchKernelGGL((node_select_kernel<PRECLAIM, true>), grid, block, sizeof(int) * (size_t)nodes, reinterpret_cast<hipStream_t>(stream), a);
+    else
+        hipLaunchKernelGGL((node_select_kernel<PRECLAIM, false>), grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
     return static_cast<int>(hipGetLastError());
 }
 }  // namespace
