@@ -305,10 +305,11 @@ def bench_puct_node_select(args):
               and not d["node_expand_inflight"].numpy().any())
     invalid_share = float((kinds == 0).mean())
     selections = steps * trees * warps
-    # per level: the node word and ticket counter, child / N / W / prior of every edge and the child's counter (a gather);
-    # the preclaim kernel also adds to and takes from every child's counter: two atomic read-modify-writes per edge
-    level_bytes = 8 + (20 + (8 if variant == puct.VARIANT_PRECLAIM else 0)) * actions + 4
-    alg_bytes = trees * warps * depth * level_bytes
+    # per level: the node word and ticket counter, child / N / W / prior of every edge, one path entry.  The children's
+    # virtual-visit counters, which both kernels gather and the preclaim kernel updates twice per edge, are held in the
+    # workgroup's LDS for the launch (a tree's 8 traversals are one workgroup): 2 x 4 bytes per node and launch
+    level_bytes = 8 + 16 * actions + 4
+    alg_bytes = trees * warps * depth * level_bytes + trees * (actions + 1) * 8
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import puct_oracle as po
@@ -340,10 +341,10 @@ def bench_puct_node_select(args):
            "roofline": {"bound": "hbm", "achieved": traffic / launch_s / 1e9 if traffic else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": traffic / launch_s / 1e9 / HBM_PEAK_GBS if traffic else None, "traffic": traffic,
                         "traffic_source": {"file": prof["file"], "commit": prof.get("commit"), "stale": prof.get("stale")} if prof else None,
-                        "kernel": f"node_select_kernel<{str(variant == puct.VARIANT_PRECLAIM).lower()}>", "avg_launch_ms": ms / steps,
+                        "kernel": f"node_select_kernel<{str(variant == puct.VARIANT_PRECLAIM).lower()}, true>", "avg_launch_ms": ms / steps,
                         "l2_level": {"requested_bytes_per_launch": alg_bytes, "requested_GB_per_s": alg_bytes / launch_s / 1e9,
-                                     "note": "node word, ticket counter, child / N / W / prior of every edge and the child's counter "
-                                             "per level and traversal; the preclaim kernel adds two atomic updates per edge"}},
+                                     "note": "node word, ticket counter, child / N / W / prior of every edge per level and traversal; "
+                                             "the virtual-visit counters are in LDS during the launch"}},
            "cpu_baseline": cpu}
     print(json.dumps(out))
 
