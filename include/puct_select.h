@@ -59,7 +59,10 @@ extern "C" {
  * Replaces puct_select_winner_recalc_launch of src/puct/puct_gpu_v3_cpp.cu:450-481 (kernel :277-448): same
  * signature, same semantics, same packing.  The reference launches `trees` blocks of `warps * 32` threads; this
  * library launches one 64-lane wavefront per (tree, wid) and splits trees with more than 16 traversals over several
- * workgroups, so `warps` is not limited to 32.
+ * workgroups, so `warps` is not limited to 32.  With up to 16 traversals per tree and nodes * edges <= 8192 a launch
+ * keeps every tree's edge_inflight in the LDS of the one workgroup that runs the tree's traversals (read at the start,
+ * written back at the end; the claims in between are LDS operations).  As with any output array, nothing else on the
+ * device may read or write edge_inflight while the launch runs; launches on one stream, or ordered by events, are fine.
  */
 int puct_select_winner_recalc_launch(float cpuct, float c_pw, float alpha_pw, int soft_winner,
                                      const int *edge_child_id, const float *edge_prior, const float *edge_W,

@@ -191,16 +191,45 @@ __device__ __forceinline__ int best_edge(const uint32_t (&keys)[S], int lane, in
     return at_or_after != kNoEdge ? at_or_after : first;
 }
 
+// The claims in flight on one tree's edges, edge_inflight[tree, :, :].  While a launch runs they are read and changed by
+// the traversals of that tree only; when those are the wavefronts of one workgroup (up to 16 traversals per tree) and the
+// tree is small enough (nodes * edges words), the workgroup keeps them in LDS for the launch (LOCAL): loaded at the
+// start, stored at the end, every read of a node's row and every claim in between an LDS operation instead of an
+// agent-scope load and an atomic performed at the memory side.
+typedef __attribute__((address_space(3))) int *LdsInts;
+template <bool LOCAL>
+struct EdgeClaims {
+    int *in_memory;     // edge_inflight + tree * nodes * edges
+    LdsInts in_lds;     // the same counters, the workgroup's copy
+    // (row: first slot of a node's edges, the same in all lanes -- in memory one address per wavefront, the edge is the offset)
+    __device__ __forceinline__ int peek(uint32_t row, uint32_t edge) const {
+        if (LOCAL) return __hip_atomic_load(in_lds + (row + edge), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return load_relaxed((in_memory + row) + edge);
+    }
+    __device__ __forceinline__ void add(uint32_t row, uint32_t edge, int v) const {
+        if (LOCAL) __hip_atomic_fetch_add(in_lds + (row + edge), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else atomicAdd((in_memory + row) + edge, v);
+    }
+    __device__ __forceinline__ int cas(uint32_t row, uint32_t edge, int expected, int desired) const {   // returns the value found
+        if (LOCAL) {
+            __hip_atomic_compare_exchange_strong(in_lds + (row + edge), &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            return expected;
+        }
+        return atomicCAS((in_memory + row) + edge, expected, desired);
+    }
+};
+
 // Takes back the virtual loss of the first `depth` path entries (src/puct/puct_gpu_v3_cpp.cu:206-217).  The entries
 // were stored by lane 0 of this wavefront; the fence completes those stores before other lanes read them back.
-__device__ __forceinline__ void rollback_path(const SelectArgs &a, const int *path, int tree, int depth, int lane,
+template <bool LOCAL>
+__device__ __forceinline__ void rollback_path(const SelectArgs &a, const EdgeClaims<LOCAL> &claims, const int *path, int tree, int depth, int lane,
                                               int node_cnt) {
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
     for (int d = lane; d < depth; d += kWave) {
         const int encoded = load_relaxed(path + d);
         const int parent = encoded >> 8, slot = encoded & 0xFF;
         if (parent >= 0 && parent < node_cnt && slot < a.edges)
-            atomicSub(&a.edge_inflight[((size_t)tree * a.nodes + parent) * a.edges + slot], 1);
+            claims.add((uint32_t)parent * (uint32_t)a.edges, (uint32_t)slot, -1);
     }
 }
 
@@ -208,7 +237,8 @@ __device__ __forceinline__ void rollback_path(const SelectArgs &a, const int *pa
 // number S of 64-edge slices that the node's expanded edges fill (1..4, the same for all lanes): these kernels are bound
 // by the wavefronts' instruction issue, vector and scalar together, and a level written for "up to four slices" spends a
 // third of it on finding out, slice by slice, that a slice is not there.
-__device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, int wid, int lane) {
+template <bool LOCAL>
+__device__ __forceinline__ void select_traversal(const SelectArgs &a, const EdgeClaims<LOCAL> &claims, int tree, int wid, int lane) {
     static_assert(kPasses == 4, "the levels below are written for one to four slices");
     const size_t out = (size_t)tree * a.warps + wid;
     int *path = a.out_path_eids + out * a.path_depth;
@@ -230,14 +260,14 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
             const size_t nrow = (size_t)tree * nodes + node;
             const size_t erow = nrow * edges;
             const int *row_n = a.edge_N + erow, *row_c = a.edge_child_id + erow;   // one address per wavefront, the lane is the offset
-            int *row_f = a.edge_inflight + erow;
+            const uint32_t row_f = (uint32_t)node * (uint32_t)edges;   // the node's row in the tree's claims
             const float *row_p = a.edge_prior + erow, *row_w = a.edge_W + erow;
 
             // Everything a level can need from the first 64 edges, requested in one go, before the node's width is known
             // (lanes beyond the row read its last edge and take no part); the edges of wider nodes follow once it is
             // and stay in registers for the rest of the level.
             const int at0 = lane < edges ? lane : edges - 1;
-            const int n0 = row_n[at0], f0 = load_relaxed(row_f + at0), c0 = row_c[at0];
+            const int n0 = row_n[at0], f0 = claims.peek(row_f, (uint32_t)at0), c0 = row_c[at0];
             const float p0 = row_p[at0], w0 = row_w[at0];
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
@@ -249,7 +279,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                 break;
             }
             if (node_info < 0 || node_info > edges) {
-                rollback_path(a, path, tree, depth, lane, node_cnt);
+                rollback_path(a, claims, path, tree, depth, lane, node_cnt);
                 final_packed =
                     pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NODE_INFO);
                 break;
@@ -274,7 +304,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                 for (int i = 1; i < S; ++i) {
                     const int eid = lane + i * kWave;
                     at[i] = i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1;
-                    n[i] = row_n[at[i]], f[i] = load_relaxed(row_f + at[i]), p[i] = row_p[at[i]], w[i] = row_w[at[i]], c[i] = row_c[at[i]];
+                    n[i] = row_n[at[i]], f[i] = claims.peek(row_f, (uint32_t)at[i]), p[i] = row_p[at[i]], w[i] = row_w[at[i]], c[i] = row_c[at[i]];
                 }
 #pragma unroll
                 for (int i = 0; i < S; ++i) in_node[i] = i < S - 1 || lane + i * kWave < cur_expanded;
@@ -310,7 +340,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                         return -1;
                     }
                     if (cur_expanded == 0) {
-                        rollback_path(a, path, tree, depth, lane, node_cnt);
+                        rollback_path(a, claims, path, tree, depth, lane, node_cnt);
                         final_packed = pack_selection(PUCT_SELECT_BUSY, node, 0, PUCT_REASON_BUSY_EXPAND_INFLIGHT);
                         return -1;
                     }
@@ -330,7 +360,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
 
                 int best_eid = 0, held = 0;
                 if (cur_expanded == 1) {
-                    if (lane == 0) atomicAdd(row_f, 1);
+                    if (lane == 0) claims.add(row_f, 0u, 1);
                     held = 1;
                 } else {
                     // Winner-recalc claim, src/puct/puct_gpu_v3_cpp.cu:235-275: score all edges, try to move the winner's
@@ -358,7 +388,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                         } else {
 #pragma unroll
                             for (int i = 0; i < S; ++i) {
-                                const int fi = load_relaxed(row_f + at[i]);
+                                const int fi = claims.peek(row_f, (uint32_t)at[i]);
                                 if (__builtin_amdgcn_ballot_w64(fi != f[i]) != 0) {
                                     f[i] = fi;
                                     keys[i] = score_slice(i, fi);
@@ -370,20 +400,20 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
                         const int best_inflight = of_edge(f, best_eid);
                         int got = 0;
                         if (lane == 0) {
-                            const int prev = atomicCAS(row_f + best_eid, best_inflight, best_inflight + 1);
+                            const int prev = claims.cas(row_f, (uint32_t)best_eid, best_inflight, best_inflight + 1);
                             got = prev == best_inflight ? 1 : 0;
                         }
                         held = __builtin_amdgcn_readfirstlane(got);
                         if (held) break;
                     }
                     if (a.soft_winner != 0 && held == 0 && best_eid != kNoEdge) {
-                        if (lane == 0) atomicAdd(row_f + best_eid, 1);
+                        if (lane == 0) claims.add(row_f, (uint32_t)best_eid, 1);
                         held = 1;
                     }
                 }
 
                 if (held == 0) {
-                    rollback_path(a, path, tree, depth, lane, node_cnt);
+                    rollback_path(a, claims, path, tree, depth, lane, node_cnt);
                     final_packed =
                         best_eid == kNoEdge
                             ? pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_NO_VALID_EDGE)
@@ -393,8 +423,8 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, int tree, 
 
                 const int best_child = of_edge(c, best_eid);
                 if (best_child < 0 || best_child >= node_cnt) {
-                    if (lane == 0) atomicSub(row_f + best_eid, 1);
-                    rollback_path(a, path, tree, depth, lane, node_cnt);
+                    if (lane == 0) claims.add(row_f, (uint32_t)best_eid, -1);
+                    rollback_path(a, claims, path, tree, depth, lane, node_cnt);
                     final_packed =
                         pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_CHILD_OOB);
                     return -1;
@@ -459,7 +489,6 @@ __device__ __forceinline__ int pack_selection_v2(int kind, int node, int slot) {
 // tree's counters fit, the workgroup keeps them in LDS for the launch (LOCAL): loaded at the start, stored at the end, and
 // every claim in between is an LDS atomic instead of one performed at the memory side (the preclaim kernel makes two per
 // edge and level; in device memory they were what bounded it).
-typedef __attribute__((address_space(3))) int *LdsInts;
 template <bool LOCAL>
 struct NodeVisits {
     int *in_memory;     // node_inflight + tree * nodes

@@ -4,10 +4,24 @@
 namespace {
 using namespace puct;
 
+// LOCAL: the tree's traversals are this workgroup's wavefronts (grid.y == 1) and the claims on its edges are kept in
+// the workgroup's dynamic LDS for the launch (a.nodes * a.edges words).
+template <bool LOCAL>
 __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) void select_kernel(const SelectArgs a) {
+    extern __shared__ int tree_claims[];
     const int wid = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave);   // the same in all lanes
-    if (wid >= a.warps) return;
-    select_traversal(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
+    const int words = a.nodes * a.edges;
+    int *const in_memory = a.edge_inflight + (size_t)blockIdx.x * a.nodes * a.edges;
+    const EdgeClaims<LOCAL> claims{in_memory, (LdsInts)tree_claims};
+    if (LOCAL) {
+        for (int i = threadIdx.x; i < words; i += blockDim.x) tree_claims[i] = in_memory[i];
+        __syncthreads();
+    }
+    if (LOCAL || wid < a.warps) select_traversal<LOCAL>(a, claims, blockIdx.x, wid, threadIdx.x & (kWave - 1));
+    if (LOCAL) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < words; i += blockDim.x) in_memory[i] = tree_claims[i];
+    }
 }
 
 // LOCAL: the tree's traversals are this workgroup's wavefronts (grid.y == 1) and its virtual-visit counters are kept
@@ -37,6 +51,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_kernel(const 
 }
 
 constexpr int kLocalVisitNodes = 4096;
+constexpr int kLocalClaimSlots = 8192;
 
 // One wavefront per traversal; a tree with more than 16 traversals is spread over several workgroups.
 inline void launch_shape(int trees, int warps, dim3 &grid, dim3 &block) {
@@ -59,7 +74,12 @@ extern "C" int puct_select_winner_recalc_launch(float cpuct, float c_pw, float a
                  trees,        nodes,         edges,           warps,                path_depth};
     dim3 grid, block;
     launch_shape(trees, warps, grid, block);
-    hipLaunchKernelGGL(select_kernel, grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
+    // (the claims of a tree in LDS: up to 8192 edge slots, so that a CU still holds four workgroups)
+    const long long slots = (long long)nodes * edges;
+    if (grid.y == 1 && slots > 0 && slots <= kLocalClaimSlots)
+        hipLaunchKernelGGL(select_kernel<true>, grid, block, sizeof(int) * (size_t)slots, reinterpret_cast<hipStream_t>(stream), a);
+    else
+        hipLaunchKernelGGL(select_kernel<false>, grid, block, 0, reinterpret_cast<hipStream_t>(stream), a);
     return static_cast<int>(hipGetLastError());
 }
 
