@@ -103,7 +103,7 @@ int puct_edge_backup_launch(int virtual_loss, float *edge_W, int *edge_N, int *e
  * Selection word (:352-354, no reason field, no BUSY kind): (kind << 22) | (expand_slot << 14) | node; a traversal
  * that ends without a selection (no expansion ticket left, no edge that leads to a node of the tree, inconsistent
  * node words) has given its claims back and reports PUCT_PACKED_INVALID_V2 with path length 0.
- * With up to 16 traversals per tree and up to 4096 nodes per tree a launch keeps every tree's node_inflight row in the
+ * With up to 16 traversals per tree and up to 16384 nodes per tree a launch keeps every tree's node_inflight row in the
  * LDS of the one workgroup that runs the tree's traversals (read at the start, written back at the end; the claims in
  * between are LDS atomics).  As with any output array, nothing else on the device may read or write node_inflight
  * while the launch runs; launches on one stream, or ordered by events, are fine.

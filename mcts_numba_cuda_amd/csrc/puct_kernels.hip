@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kMaxWavesPerBlock *kWave) void backup_kernel(const 
     backup_traversal<NODE_LEVEL>(a, blockIdx.x, wid, threadIdx.x & (kWave - 1));
 }
 
-constexpr int kLocalVisitNodes = 4096;
+constexpr int kLocalVisitNodes = 16384;   // (what a selection word can name; 64 KB of LDS, two workgroups per CU: still ahead of counters in memory)
 constexpr int kLocalClaimSlots = 8192;
 
 // One wavefront per traversal; a tree with more than 16 traversals is spread over several workgroups.
@@ -94,7 +94,7 @@ int launch_node_select(float cpuct, float c_pw, float alpha_pw, const int *edge_
                      out_path_eids, out_path_len, trees,             nodes,         edges,        warps,  path_depth};
     dim3 grid, block;
     launch_shape(trees, warps, grid, block);
-    // (the counters of a tree in LDS: up to 4096 nodes, so that a CU still holds four workgroups)
+    // (the counters of a tree in LDS: up to 16384 nodes)
     if (grid.y == 1 && nodes > 0 && nodes <= kLocalVisitNodes)
         hipLaunchKernelGGL((node_select_kernel<PRECLAIM, true>), grid, block, sizeof(int) * (size_t)nodes, reinterpret_cast<hipStream_t>(stream), a);
     else

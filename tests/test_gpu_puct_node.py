@@ -52,12 +52,12 @@ def test_known_answers(case, variant):
 @pytest.mark.parametrize("variant", nc.VARIANTS)
 @pytest.mark.parametrize("actions,nodes,depth,cpuct,c_pw", [(6, 300, 16, 1.5, 1.0), (225, 2000, 8, 1.5, 0.0),
                                                             (256, 600, 4, 0.7, 2.0), (3, 4000, 64, 1.0, 0.5),
-                                                            (5, 4096, 24, 1.2, 1.0), (5, 4097, 24, 1.2, 1.0)])
+                                                            (5, 16384, 24, 1.2, 1.0), (5, 16385, 24, 1.2, 1.0)])
 def test_single_traversal_matches_oracle_exactly(actions, nodes, depth, cpuct, c_pw, variant):
     """One traversal per tree is deterministic: every array must equal the oracle's, over several select/backup rounds on
     the same trees (the statistics drift apart as soon as one score comparison differs).  In every other round the
     claims of the selection are left in place for the next one, so that the kernels also score against virtual visits.
-    (Up to 4096 nodes per tree the kernels keep a tree's virtual-visit counters in LDS during a launch, beyond that in
+    (Up to 16384 nodes per tree the kernels keep a tree's virtual-visit counters in LDS during a launch, beyond that in
     device memory: the last two cases sit on either side.)"""
     rng = np.random.default_rng(actions * 1000 + nodes)
     case = nc.random_forest(rng, trees=64, nodes=nodes, actions=actions, warps=1, path_depth=depth)
