@@ -101,6 +101,15 @@ __device__ __forceinline__ int load_relaxed(const int *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// A field of one edge of a tree: the tree's array (one address per wavefront, kept in scalar registers for the whole
+// traversal) plus a 32-bit byte offset per lane.  A tree is at most 2^14 nodes of 256 edges, 16 MB per field, so the
+// offset fits, and a load is one instruction with nothing to add to a 64-bit address first.
+template <class T>
+__device__ __forceinline__ T *at_bytes(T *tree_field, uint32_t byte_offset) {
+    typedef std::conditional_t<std::is_const<T>::value, const char, char> Byte;
+    return reinterpret_cast<T *>(reinterpret_cast<Byte *>(tree_field) + byte_offset);
+}
+
 // ---- selection ---------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int pack_selection(int kind, int node, int slot, int reason) {
     return (reason << PUCT_PACKED_REASON_SHIFT) | (kind << PUCT_PACKED_KIND_SHIFT) | (slot << PUCT_PACKED_SLOT_SHIFT) |
@@ -201,21 +210,21 @@ template <bool LOCAL>
 struct EdgeClaims {
     int *in_memory;     // edge_inflight + tree * nodes * edges
     LdsInts in_lds;     // the same counters, the workgroup's copy
-    // (row: first slot of a node's edges, the same in all lanes -- in memory one address per wavefront, the edge is the offset)
-    __device__ __forceinline__ int peek(uint32_t row, uint32_t edge) const {
-        if (LOCAL) return __hip_atomic_load(in_lds + (row + edge), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        return load_relaxed((in_memory + row) + edge);
+    // (at: byte offset of the edge's slot in the tree, (node * edges + edge) * 4)
+    __device__ __forceinline__ int peek(uint32_t at) const {
+        if (LOCAL) return __hip_atomic_load(in_lds + (at >> 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return load_relaxed(at_bytes(in_memory, at));
     }
-    __device__ __forceinline__ void add(uint32_t row, uint32_t edge, int v) const {
-        if (LOCAL) __hip_atomic_fetch_add(in_lds + (row + edge), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        else atomicAdd((in_memory + row) + edge, v);
+    __device__ __forceinline__ void add(uint32_t at, int v) const {
+        if (LOCAL) __hip_atomic_fetch_add(in_lds + (at >> 2), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        else atomicAdd(at_bytes(in_memory, at), v);
     }
-    __device__ __forceinline__ int cas(uint32_t row, uint32_t edge, int expected, int desired) const {   // returns the value found
+    __device__ __forceinline__ int cas(uint32_t at, int expected, int desired) const {   // returns the value found
         if (LOCAL) {
-            __hip_atomic_compare_exchange_strong(in_lds + (row + edge), &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_compare_exchange_strong(in_lds + (at >> 2), &expected, desired, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             return expected;
         }
-        return atomicCAS((in_memory + row) + edge, expected, desired);
+        return atomicCAS(at_bytes(in_memory, at), expected, desired);
     }
 };
 
@@ -229,7 +238,7 @@ __device__ __forceinline__ void rollback_path(const SelectArgs &a, const EdgeCla
         const int encoded = load_relaxed(path + d);
         const int parent = encoded >> 8, slot = encoded & 0xFF;
         if (parent >= 0 && parent < node_cnt && slot < a.edges)
-            claims.add((uint32_t)parent * (uint32_t)a.edges, (uint32_t)slot, -1);
+            claims.add(((uint32_t)parent * (uint32_t)a.edges + (uint32_t)slot) * 4u, -1);
     }
 }
 
@@ -252,23 +261,23 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
     if (!valid_select_shape(a.path_depth, nodes, node_cnt, edges)) {
         final_packed = pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_SHAPE);
     } else {
+        const size_t tree_edges = (size_t)tree * nodes * edges;
+        const int *const tree_n = a.edge_N + tree_edges, *const tree_c = a.edge_child_id + tree_edges;
+        const float *const tree_p = a.edge_prior + tree_edges, *const tree_w = a.edge_W + tree_edges;
         int node = 0, depth = 0;
         while (true) {
             // (the same in all lanes; said so that the level's addresses and branches are worked out once per wavefront)
             node = __builtin_amdgcn_readfirstlane(node), depth = __builtin_amdgcn_readfirstlane(depth);
             levels += 1;
             const size_t nrow = (size_t)tree * nodes + node;
-            const size_t erow = nrow * edges;
-            const int *row_n = a.edge_N + erow, *row_c = a.edge_child_id + erow;   // one address per wavefront, the lane is the offset
-            const uint32_t row_f = (uint32_t)node * (uint32_t)edges;   // the node's row in the tree's claims
-            const float *row_p = a.edge_prior + erow, *row_w = a.edge_W + erow;
+            const uint32_t row4 = (uint32_t)node * (uint32_t)edges * 4u;   // byte offset of the node's edges in the tree's fields
 
             // Everything a level can need from the first 64 edges, requested in one go, before the node's width is known
             // (lanes beyond the row read its last edge and take no part); the edges of wider nodes follow once it is
             // and stay in registers for the rest of the level.
-            const int at0 = lane < edges ? lane : edges - 1;
-            const int n0 = row_n[at0], f0 = claims.peek(row_f, (uint32_t)at0), c0 = row_c[at0];
-            const float p0 = row_p[at0], w0 = row_w[at0];
+            const uint32_t at0 = row4 + (uint32_t)(lane < edges ? lane : edges - 1) * 4u;
+            const int n0 = *at_bytes(tree_n, at0), f0 = claims.peek(at0), c0 = *at_bytes(tree_c, at0);
+            const float p0 = *at_bytes(tree_p, at0), w0 = *at_bytes(tree_w, at0);
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
             const int capacity = a.node_capacity ? a.node_capacity[nrow] : edges;
@@ -296,15 +305,21 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
             // The level proper; returns the child the traversal moves on to, or -1 when it ends here.
             auto level = [&](auto slices) __attribute__((always_inline)) -> int {
                 constexpr int S = decltype(slices)::value;   // (S - 1) * 64 < cur_expanded <= S * 64, or no edge at all (S = 1)
-                int n[S], f[S], c[S], at[S];
+                constexpr int CS = S <= 2 ? S : 1;   // slices whose row of children is requested with the scores' fields (see best_child below)
+                int n[S], f[S], c[CS];
+                // byte offset of the edge that this lane looks at in slice i (lanes beyond the node's edges: its last edge)
+                auto at = [&](int i) {
+                    const int eid = lane + i * kWave;
+                    return i == 0 ? at0 : row4 + (uint32_t)(i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1) * 4u;
+                };
                 float p[S], w[S];
                 bool in_node[S];
-                n[0] = n0, f[0] = f0, c[0] = c0, p[0] = p0, w[0] = w0, at[0] = at0;
+                n[0] = n0, f[0] = f0, p[0] = p0, w[0] = w0, c[0] = c0;
 #pragma unroll
                 for (int i = 1; i < S; ++i) {
-                    const int eid = lane + i * kWave;
-                    at[i] = i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1;
-                    n[i] = row_n[at[i]], f[i] = claims.peek(row_f, (uint32_t)at[i]), p[i] = row_p[at[i]], w[i] = row_w[at[i]], c[i] = row_c[at[i]];
+                    const uint32_t here = at(i);
+                    n[i] = *at_bytes(tree_n, here), f[i] = claims.peek(here), p[i] = *at_bytes(tree_p, here), w[i] = *at_bytes(tree_w, here);
+                    if (i < CS) c[i] = *at_bytes(tree_c, here);
                 }
 #pragma unroll
                 for (int i = 0; i < S; ++i) in_node[i] = i < S - 1 || lane + i * kWave < cur_expanded;
@@ -358,9 +373,13 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
                     return r;
                 };
 
-                int best_eid = 0, held = 0;
+                // Where the winner leads: for nodes of up to 128 edges the row of children came with the scores' fields; of a
+                // wider node only its first 64, and beyond them just the winner's word is asked for, on its way while the
+                // claim is made (the rest of that row is a sixth of what such a level reads -- and those launches are bound by
+                // what they read -- and three registers per lane; at 128 edges waiting for the word cost more than the row).
+                int best_eid = 0, held = 0, best_child = c0;   // (cur_expanded == 1: lane 0's is read below)
                 if (cur_expanded == 1) {
-                    if (lane == 0) claims.add(row_f, 0u, 1);
+                    if (lane == 0) claims.add(row4, 1);
                     held = 1;
                 } else {
                     // Winner-recalc claim, src/puct/puct_gpu_v3_cpp.cu:235-275: score all edges, try to move the winner's
@@ -388,7 +407,7 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
                         } else {
 #pragma unroll
                             for (int i = 0; i < S; ++i) {
-                                const int fi = claims.peek(row_f, (uint32_t)at[i]);
+                                const int fi = claims.peek(at(i));
                                 if (__builtin_amdgcn_ballot_w64(fi != f[i]) != 0) {
                                     f[i] = fi;
                                     keys[i] = score_slice(i, fi);
@@ -398,16 +417,22 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
                         best_eid = best_edge<S>(keys, lane, -1, tie_offset);
                         if (best_eid == kNoEdge) break;
                         const int best_inflight = of_edge(f, best_eid);
+                        if (best_eid < CS * kWave) {
+                            best_child = __builtin_amdgcn_readlane(c[0], best_eid & (kWave - 1));
+                            if (CS > 1 && best_eid >= kWave) best_child = __builtin_amdgcn_readlane(c[CS - 1], best_eid & (kWave - 1));
+                        } else {
+                            best_child = load_relaxed(at_bytes(tree_c, row4 + (uint32_t)best_eid * 4u));   // (every lane the same word)
+                        }
                         int got = 0;
                         if (lane == 0) {
-                            const int prev = claims.cas(row_f, (uint32_t)best_eid, best_inflight, best_inflight + 1);
+                            const int prev = claims.cas(row4 + (uint32_t)best_eid * 4u, best_inflight, best_inflight + 1);
                             got = prev == best_inflight ? 1 : 0;
                         }
                         held = __builtin_amdgcn_readfirstlane(got);
                         if (held) break;
                     }
                     if (a.soft_winner != 0 && held == 0 && best_eid != kNoEdge) {
-                        if (lane == 0) claims.add(row_f, (uint32_t)best_eid, 1);
+                        if (lane == 0) claims.add(row4 + (uint32_t)best_eid * 4u, 1);
                         held = 1;
                     }
                 }
@@ -421,9 +446,9 @@ __device__ __forceinline__ void select_traversal(const SelectArgs &a, const Edge
                     return -1;
                 }
 
-                const int best_child = of_edge(c, best_eid);
+                best_child = __builtin_amdgcn_readfirstlane(best_child);
                 if (best_child < 0 || best_child >= node_cnt) {
-                    if (lane == 0) claims.add(row_f, (uint32_t)best_eid, -1);
+                    if (lane == 0) claims.add(row4 + (uint32_t)best_eid * 4u, -1);
                     rollback_path(a, claims, path, tree, depth, lane, node_cnt);
                     final_packed =
                         pack_selection(PUCT_SELECT_INVALID, PUCT_PACKED_NODE_MASK, 0, PUCT_REASON_INVALID_CHILD_OOB);
