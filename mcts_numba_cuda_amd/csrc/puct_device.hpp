@@ -573,6 +573,9 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, c
     // src/puct/puct_gpu_v2.py:357-366
     if (a.path_depth >= 1 && nodes > 0 && node_limit > 0 && node_limit <= nodes && node_limit <= PUCT_PACKED_NODE_LIMIT &&
         edges > 0 && edges <= PUCT_PACKED_EDGE_MASK + 1) {
+        const size_t tree_edges = trow * edges;
+        const int *const tree_c = a.edge_child_id + tree_edges, *const tree_n = a.edge_N + tree_edges;
+        const float *const tree_p = a.edge_prior + tree_edges, *const tree_w = a.edge_W + tree_edges;
         int node = 0, depth = 0;
         while (true) {
             // (the same in all lanes; said so that the level's addresses and branches are worked out once per wavefront)
@@ -586,14 +589,13 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, c
                 final_len = depth + 1;
                 break;
             }
-            const size_t nrow = trow + node, erow = nrow * edges;
-            const int *row_c = a.edge_child_id + erow, *row_n = a.edge_N + erow;   // one address per wavefront, the lane is the offset
-            const float *row_p = a.edge_prior + erow, *row_w = a.edge_W + erow;
+            const size_t nrow = trow + node;
+            const uint32_t row4 = (uint32_t)node * (uint32_t)edges * 4u;   // byte offset of the node's edges in the tree's fields
             // the first 64 edges are requested together with the node's own words, before the node's width is known
             // (lanes beyond the row read its last edge and take no part)
-            const int at0 = lane < edges ? lane : edges - 1;
-            const int c0 = row_c[at0], n0 = row_n[at0];
-            const float p0 = row_p[at0], w0 = row_w[at0];
+            const uint32_t at0 = row4 + (uint32_t)(lane < edges ? lane : edges - 1) * 4u;
+            const int c0 = *at_bytes(tree_c, at0), n0 = *at_bytes(tree_n, at0);
+            const float p0 = *at_bytes(tree_p, at0), w0 = *at_bytes(tree_w, at0);
             const int node_info = a.node_expanded[nrow];
             const int expand_inflight = load_relaxed(a.node_expand_inflight + nrow);
             if (node_info == PUCT_NODE_EXPANDED_TERMINAL) {
@@ -616,8 +618,9 @@ __device__ __forceinline__ void node_select_traversal(const NodeSelectArgs &a, c
                 c[0] = c0, n[0] = n0, p[0] = p0, w[0] = w0;
 #pragma unroll
                 for (int i = 1; i < S; ++i) {
-                    const int eid = lane + i * kWave, at = i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1;
-                    c[i] = row_c[at], n[i] = row_n[at], p[i] = row_p[at], w[i] = row_w[at];
+                    const int eid = lane + i * kWave;
+                    const uint32_t at = row4 + (uint32_t)(i < S - 1 || eid < cur_expanded ? eid : cur_expanded - 1) * 4u;
+                    c[i] = *at_bytes(tree_c, at), n[i] = *at_bytes(tree_n, at), p[i] = *at_bytes(tree_p, at), w[i] = *at_bytes(tree_w, at);
                 }
                 // an edge takes part when it is expanded and leads to a node of the tree; its virtual visits are its
                 // child's (the other lanes read the root's counter and drop it)
