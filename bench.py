@@ -212,10 +212,11 @@ def bench_puct_select(args):
     ms, wall, ok, busy_share = timed(0)
     ms_soft, _, ok_soft, busy_soft = timed(1)
     selections = steps * trees * warps
-    # per level: node word, ticket counter, and N / W / prior / child / in-flight of every edge; one path entry.  Exact
+    # per level: node word, ticket counter, N / W / prior / in-flight of every edge, where the edges lead (the whole
+    # child row for nodes of up to 128 edges, else its first 64 words and the winner's) and one path entry.  Exact
     # for the soft-winner run, in which every traversal walks all `depth` levels; with the strict claim a busy traversal
     # stops early, so only the completed ones are counted.
-    level_bytes = 8 + 20 * actions + 4
+    level_bytes = 8 + 16 * actions + (4 * actions if actions <= 128 else 4 * 64 + 4) + 4
     alg_bytes = int(trees * warps * (1.0 - busy_share)) * depth * level_bytes
     alg_bytes_soft = trees * warps * depth * level_bytes
     cpu = None
@@ -257,8 +258,10 @@ def bench_puct_select(args):
                         "kernel": "select_kernel", "avg_launch_ms": ms / steps,
                         "l2_level": {"requested_bytes_per_launch_completed_traversals": alg_bytes,
                                      "requested_GB_per_s": alg_bytes / launch_s / 1e9,
-                                     "note": "node word, ticket counter and five 4-byte fields per edge and level, for the "
-                                             "traversals that complete; busy ones stop after a third of the levels on average"}},
+                                     "note": "node word, ticket counter and the 4-byte fields per edge and level that the kernel asks for "
+                                             "(N, W, prior, in-flight; the child of every edge up to 128 edges, of the first 64 and "
+                                             "the winner beyond), for the traversals that complete; busy ones stop after a third of "
+                                             "the levels on average"}},
            "cpu_baseline": cpu}
     print(json.dumps(out))
 
