@@ -407,3 +407,35 @@ def random_forest(rng, trees, nodes, actions, warps, path_depth, terminal_fracti
         term = leaves[rng.random(leaves.size) < terminal_fraction]
         c["node_expanded"][t, term] = TERMINAL
     return c
+
+
+def wide_forest(rng, trees, nodes, actions, warps, path_depth, hubs=2, claims=0.05, terminal_fraction=0.15, fill=0.8):
+    """Random consistent trees with wide nodes: four new nodes in five hang under one of the first `hubs` nodes while
+    those have free edge slots, so the top levels fill several 64-edge slices; half of the priors come from four values
+    (equal scores in different slices), a fifth of the edges is unvisited, and a share `claims` of all edge slots
+    already holds one to three claims."""
+    c = make_case(trees=trees, nodes=nodes, actions=actions, warps=warps, path_depth=path_depth)
+    for t in range(trees):
+        used = int(max(2, nodes * fill))
+        c["node_count"][t] = used
+        expanded = np.zeros(nodes, np.int32)
+        for i in range(1, used):
+            while True:
+                p = int(rng.integers(0, min(i, hubs))) if rng.random() < 0.8 else int(rng.integers(0, i))
+                if expanded[p] < actions:
+                    break
+            s = expanded[p]
+            expanded[p] += 1
+            c["edge_child"][t, p, s] = i
+            n = int(rng.integers(0, 20)) if rng.random() < 0.8 else 0
+            c["edge_n"][t, p, s] = n
+            c["edge_w"][t, p, s] = np.float32(rng.uniform(-1, 1) * n)
+            c["edge_prior"][t, p, s] = np.float32(rng.choice([0.1, 0.25, 0.5, 1.0]) if rng.random() < 0.5 else rng.uniform(0.01, 1.0))
+        c["node_expanded"][t] = expanded
+        leaves = np.flatnonzero(expanded[:used] == 0)
+        term = leaves[rng.random(leaves.size) < terminal_fraction]
+        c["node_expanded"][t, term] = TERMINAL
+    if claims:
+        held = rng.random(c["edge_inflight"].shape) < claims
+        c["edge_inflight"][held] = rng.integers(1, 4, int(held.sum()))
+    return c

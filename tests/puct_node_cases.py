@@ -375,3 +375,18 @@ def random_forest(rng, trees, nodes, actions, warps, path_depth, broken_edges=0.
     broken = expanded & (rng.random(c["edge_child"].shape) < broken_edges)
     c["edge_child"][broken] = -1
     return c
+
+
+def wide_forest(rng, trees, nodes, actions, warps, path_depth, hubs=2, visits=0.05, broken_edges=0.03):
+    """puct_cases.wide_forest with node-level counters: a share `visits` of the nodes already carries one to three
+    virtual visits, and a share of the expanded edges leads nowhere."""
+    c = pc.wide_forest(rng, trees, nodes, actions, warps, path_depth, hubs=hubs, claims=0.0)
+    del c["edge_inflight"]
+    c["node_inflight"] = np.zeros((trees, nodes), np.int32)
+    if visits:
+        held = rng.random(c["node_inflight"].shape) < visits
+        c["node_inflight"][held] = rng.integers(1, 4, int(held.sum()))
+    expanded = np.arange(actions)[None, None, :] < np.maximum(c["node_expanded"], 0)[:, :, None]
+    broken = expanded & (rng.random(c["edge_child"].shape) < broken_edges)
+    c["edge_child"][broken] = -1
+    return c

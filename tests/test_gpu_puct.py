@@ -75,6 +75,28 @@ def test_single_traversal_matches_oracle_exactly(actions, nodes, depth, cpuct, c
         assert pc.inflight_sum(got) == 0
 
 
+@pytest.mark.parametrize("actions,nodes,hubs,claims,cpuct,c_pw,soft", [(256, 1200, 2, 0.05, 1.5, 0.0, 0), (193, 1200, 4, 0.3, 1.0, 16.0, 1),
+                                                                      (129, 300, 1, 0.3, 0.5, 0.0, 0), (65, 300, 8, 0.05, 4.0, 2.0, 1),
+                                                                      (225, 40, 1, 0.0, 0.0, 100.0, 0)])
+def test_wide_nodes_with_claims_in_flight_match_oracle_exactly(actions, nodes, hubs, claims, cpuct, c_pw, soft):
+    """As above on trees whose top levels fill two to four 64-edge slices, with random statistics, repeated priors and
+    claims already held on some edges (so the scores see virtual loss and a strict claim can find its edge taken)."""
+    rng = np.random.default_rng(actions * 1000 + nodes)
+    case = pc.wide_forest(rng, trees=32, nodes=nodes, actions=actions, warps=1, path_depth=12, hubs=hubs, claims=claims)
+    h = copy.deepcopy(case)
+    r = HipRunner()
+    for rnd in range(4):
+        got = r.select(case if rnd == 0 else to_host(r.d), cpuct=cpuct, c_pw=c_pw, soft_winner=soft)
+        po.select(h, cpuct=cpuct, c_pw=c_pw, soft_winner=soft)
+        for k in h:
+            assert np.array_equal(got[k], h[k], equal_nan=True), (rnd, k)
+        values = rng.uniform(-1, 1, h["out_path"].shape).astype(np.float32)
+        got = r.backup(values)
+        po.backup(h, values)
+        for k in h:
+            assert np.array_equal(got[k], h[k], equal_nan=True), (rnd, k)
+
+
 @pytest.mark.parametrize("trees,warps,soft", [(16, 8, 0), (16, 16, 0), (4, 40, 0), (16, 16, 1), (128, 4, 0)])
 def test_concurrent_traversals_keep_invariants(trees, warps, soft):
     rng = np.random.default_rng(trees * 100 + warps)

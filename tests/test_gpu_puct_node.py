@@ -78,6 +78,29 @@ def test_single_traversal_matches_oracle_exactly(actions, nodes, depth, cpuct, c
 
 
 @pytest.mark.parametrize("variant", nc.VARIANTS)
+@pytest.mark.parametrize("actions,nodes,hubs,visits,cpuct,c_pw", [(256, 1200, 2, 0.05, 1.5, 0.0), (193, 1200, 4, 0.3, 1.0, 16.0),
+                                                                 (129, 300, 1, 0.3, 0.5, 0.0), (65, 300, 8, 0.05, 4.0, 2.0),
+                                                                 (225, 40, 1, 0.0, 0.0, 100.0)])
+def test_wide_nodes_with_virtual_visits_match_oracle_exactly(actions, nodes, hubs, visits, cpuct, c_pw, variant):
+    """As above on trees whose top levels fill two to four 64-edge slices, with random statistics, repeated priors,
+    virtual visits already on some nodes and some expanded edges that lead nowhere."""
+    rng = np.random.default_rng(actions * 1000 + nodes)
+    case = nc.wide_forest(rng, trees=32, nodes=nodes, actions=actions, warps=1, path_depth=12, hubs=hubs, visits=visits)
+    h = copy.deepcopy(case)
+    r = HipRunner()
+    for rnd in range(4):
+        got = r.select(case if rnd == 0 else to_host(r.d), variant, cpuct=cpuct, c_pw=c_pw)
+        po.node_select(h, cpuct=cpuct, c_pw=c_pw, variant=variant)
+        for k in h:
+            assert np.array_equal(got[k], h[k], equal_nan=True), (rnd, k)
+        values = rng.uniform(-1, 1, h["out_path"].shape).astype(np.float32)
+        got = r.backup(values)
+        po.backup(h, values, node_level=True)
+        for k in h:
+            assert np.array_equal(got[k], h[k], equal_nan=True), (rnd, k)
+
+
+@pytest.mark.parametrize("variant", nc.VARIANTS)
 @pytest.mark.parametrize("trees,warps", [(16, 8), (16, 16), (4, 40), (128, 4)])
 def test_concurrent_traversals_keep_invariants(trees, warps, variant):
     rng = np.random.default_rng(trees * 100 + warps)
