@@ -43,11 +43,28 @@ def draw_case(rng):
                 stones=int(rng.integers(0, m * n // 2)), steps=steps)
 
 
-@pytest.mark.parametrize("block", range(4))
+def widen(rng, c):
+    """Moves a Gomoku case to a board beyond 16 x 16 (sides up to 32, up to 512 cells: the engine's two wide board formats)."""
+    while True:
+        m, n = int(rng.integers(5, 33)), int(rng.integers(5, 33))
+        if m * n <= 512 and (m > 16 or n > 16):
+            break
+    acp = c["variant"].startswith("acp")
+    c.update(shape=(m, n), stones=int(rng.integers(0, m * n // 3)), steps=int(rng.integers(2, 5)) if acp else int(rng.integers(10, 120)),
+             P=min(c["P"], 64 if acp else 256), T=min(c["T"], 8), device_memory=max(c["device_memory"], 0.05))
+    return c
+
+
+@pytest.mark.parametrize("block", range(5))
 def test_random_configurations(block):
+    """(Block 4: Gomoku on wide boards only.)"""
     rng = np.random.default_rng(1000 + block)
     for _ in range(30):
         c = draw_case(rng)
+        if block == 4:
+            if c["game"] != "gomoku":
+                continue
+            c = widen(rng, c)
         m, n = c["shape"]
         params = dict(n_trees=c["T"], n_playouts=c["P"], variant=c["variant"], device_memory=c["device_memory"], ucb_c=c["ucb_c"], seed=c["seed"])
         if c["game"] == "gomoku":
