@@ -92,6 +92,14 @@ __device__ __forceinline__ unsigned long long max_over_8_lanes(unsigned long lon
     o = dpp_move_u64<0x141>(key); key = o > key ? o : key;   // row_half_mirror
     return key;
 }
+// The same for a 32-bit key: one `v_max_u32` with a DPP operand per step.
+__device__ __forceinline__ uint32_t max_over_8_lanes(uint32_t key) {
+    uint32_t o;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0xB1, 0xf, 0xf, true); key = o > key ? o : key;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x4E, 0xf, 0xf, true); key = o > key ? o : key;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0x141, 0xf, 0xf, true); key = o > key ? o : key;
+    return key;
+}
 
 // ---- agent-scope synchronisation between workgroups --------------------------------------------
 __device__ __forceinline__ uint32_t atomic_add_acq_rel(uint32_t *p, uint32_t v) {
