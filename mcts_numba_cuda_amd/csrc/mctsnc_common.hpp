@@ -77,22 +77,9 @@ __device__ __forceinline__ float ucb_value(int32_t wins, int32_t n, double log_p
 // is smallest; for slots below 8 the order of the 3-bit reversal equals that of any wider reversal.
 __device__ __forceinline__ uint32_t bitrev3(uint32_t a) { return ((a & 1u) << 2) | (a & 2u) | ((a >> 2) & 1u); }
 
-// Maximum of a 64-bit key over each group of 8 adjacent lanes, in every lane of the group, with DPP moves (xor 1 and
-// xor 2 inside a quad, then the mirror image within the half row) instead of LDS permutes.  All 64 lanes must be active.
-template <int CTRL>
-__device__ __forceinline__ unsigned long long dpp_move_u64(unsigned long long v) {
-    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, 0xf, 0xf, true);
-    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, 0xf, 0xf, true);
-    return ((unsigned long long)hi << 32) | lo;
-}
-__device__ __forceinline__ unsigned long long max_over_8_lanes(unsigned long long key) {
-    unsigned long long o;
-    o = dpp_move_u64<0xB1>(key); key = o > key ? o : key;    // quad_perm [1,0,3,2]
-    o = dpp_move_u64<0x4E>(key); key = o > key ? o : key;    // quad_perm [2,3,0,1]
-    o = dpp_move_u64<0x141>(key); key = o > key ? o : key;   // row_half_mirror
-    return key;
-}
-// The same for a 32-bit key: one `v_max_u32` with a DPP operand per step.
+// Maximum of a 32-bit key over each group of 8 adjacent lanes, in every lane of the group: one `v_max_u32` with a DPP
+// operand per step (xor 1 and xor 2 inside a quad, then the mirror image within the half row) instead of LDS permutes.
+// All 64 lanes must be active.
 __device__ __forceinline__ uint32_t max_over_8_lanes(uint32_t key) {
     uint32_t o;
     o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)key, 0xB1, 0xf, 0xf, true); key = o > key ? o : key;
