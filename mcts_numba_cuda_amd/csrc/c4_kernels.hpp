@@ -862,9 +862,10 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
         if (ACP && !SOLO) {
             if (wave == 0) {
                 unsigned long long *mail = hdr->mail[gen & 1];
-                // Same-XCC publish: the only tree data a team workgroup stores during a step are its child's record and
-                // its share of the path records, both by this wavefront (wave 0); they must have been acknowledged by
-                // the L2 before the result word that lets the other workgroups go on is stored.
+                // Same-XCC publish: the only tree data a team workgroup stores during a step are its child's record, by
+                // this wavefront (wave 0), and its share of the path records, each by the wavefront that backed the level
+                // up (which waited for them before the barrier that ended the backup); they must have been acknowledged
+                // by the L2 before the result word that lets the other workgroups go on is stored.
                 if (xcd_local) wait_own_stores_at_l2();
                 if (lane == 0) {
                     const unsigned long long v = ((unsigned long long)(gen + 1u) << 32) | ((unsigned long long)(uint32_t)res_neg << 16) | (unsigned long long)(uint32_t)res_pos;
