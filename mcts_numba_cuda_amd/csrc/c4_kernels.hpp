@@ -1082,8 +1082,9 @@ __device__ __forceinline__ void search_body(const SearchArgs &args, const int r,
 // XCD-aware decode: consecutive blockIdx values go to different XCDs, so the G workgroups of one set are spaced 8
 // apart and meet in one L2.  Set u starts on tree u; when a launch has more trees than sets (a large batch of
 // searches), a set that has finished its tree takes the next one from the queue: workgroup 0 draws the index and
-// leaves it in the finished tree's header for the others.  Five wavefronts per SIMD (at most 96 vector registers, two
-// dwords spilled) let five workgroups share a CU in such batches; a single search is no slower for it.
+// leaves it in the finished tree's header for the others.  Five wavefronts per SIMD (at most 96 vector registers: none
+// spilled by the team kernel, two dwords by the one with playout pools) let five workgroups share a CU in such batches; a
+// single search is no slower for it.
 template <class Game, bool ACP, bool SOLO, bool POOL = false>
 __device__ __forceinline__ void search_trees(const SearchArgs &args) {
     const int b = blockIdx.x;
